@@ -1,0 +1,215 @@
+#!/usr/bin/env python3
+"""Benchmark of the packed-KV decode attention hot path on one MI355X.
+
+A step = one layer's decode attention (split pass + merge pass) over one batch of synthetic,
+already-packed KV resident in HBM.  Default workload: Llama-3.1-8B-shaped decode, 32 Q / 8 KV
+heads, head_dim 128, batch 16, 32k context (BASELINE.json configs[1]).  Steps rotate over several
+independent copies of the cache so that every step streams from HBM rather than from the 256 MB
+Infinity Cache.  Prints ONE JSON line.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c1|c0|c4] [--copies N]
+"""
+import argparse
+import json
+import os
+import sys
+import time
+import types
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+WORKLOADS = {
+    # name: (B, H_Q, H_KV, T, description)
+    "c0": (1, 32, 8, 4096, "decode B=1 32Q/8KV D=128 ctx=4096 (configs[0])"),
+    "c1": (16, 32, 8, 32768, "Llama-3.1-8B-shaped decode B=16 32Q/8KV D=128 ctx=32768, 2-bit Kitty KV (configs[1])"),
+    "c4": (1, 64, 8, 131072, "long-context decode B=1 64Q/8KV D=128 ctx=131072 (configs[4])"),
+}
+HBM_PEAK_GBPS = 8000.0
+
+
+def synth_kv(B, H, T, D, seed, device, student_t=False):
+    """K ~ N(0,1) with 8 fixed outlier channels per head scaled x10, V ~ N(0,1); fp16 [B,H,T,D]."""
+    import torch
+    g = torch.Generator(device=device).manual_seed(seed)
+    K = torch.empty((B, H, T, D), dtype=torch.float16, device=device)
+    V = torch.empty((B, H, T, D), dtype=torch.float16, device=device)
+    mult = torch.ones((H, 1, D), dtype=torch.float32, device=device)
+    pg = torch.Generator().manual_seed(seed)
+    for h in range(H):
+        mult[h, 0, torch.randperm(D, generator=pg)[:8].to(device)] = 10.0
+    for b in range(B):
+        K[b] = (torch.randn((H, T, D), generator=g, device=device, dtype=torch.float32) * mult).half()
+        V[b] = torch.randn((H, T, D), generator=g, device=device, dtype=torch.float32).half()
+    return K, V
+
+
+def algorithmic_bytes(B, H_Q, H_KV, layer):
+    """Bytes one decode step has to move: packed pages + metadata + fp16 windows + Q and O."""
+    pk, pv = layer.PageCount_K, layer.PageCount_V
+    per_head_packed = 5760 * pk + 4608 * pv
+    per_head_fp16 = 256 * (2 * layer.Sink_Count + layer.Q_Buffer_Count_K + layer.Q_Buffer_Count_V + layer.Local_Count_V)
+    qo = 2 * H_Q * 128 * 2
+    return B * (H_KV * (per_head_packed + per_head_fp16) + qo), B * H_KV * per_head_packed
+
+
+def cpu_baseline(K_row, V_row, q_row, H_Q, H_KV, B_full, budget_s=20.0):
+    """The reference's CPU path (fake-quant simulator + eager attention) on one sequence of the
+    workload, on the host cores; scaled by the batch size to the workload's step."""
+    import torch
+    from oracle import sim_baseline as S
+    cores = os.cpu_count() or 1
+    threads = min(cores, 16)
+    torch.set_num_threads(threads)
+    K, V = K_row.clone(), V_row.clone()
+    t0 = time.perf_counter()
+    S.simulate_prefill(K, V)
+    t_quant = time.perf_counter() - t0
+    S.eager_attention(q_row, K, V, 128 ** -0.5, H_Q // H_KV)          # warm-up
+    reps, t_att = 0, 0.0
+    while reps < 3 or (t_att < budget_s / 2 and reps < 20):
+        t0 = time.perf_counter()
+        S.eager_attention(q_row, K, V, 128 ** -0.5, H_Q // H_KV)
+        t_att += time.perf_counter() - t0
+        reps += 1
+    us = t_att / reps * 1e6 * B_full
+    return {
+        "value": us, "unit": "us/step", "cores": threads, "kind": "port",
+        "sample": (f"1 of {B_full} sequences of the workload (dense fake-quantized fp16 KV, eager GQA attention, "
+                   f"{reps} reps, torch {threads} threads), time x{B_full}; fake-quant of that sequence took "
+                   f"{t_quant:.2f} s once"),
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", default="c1", choices=sorted(WORKLOADS))
+    ap.add_argument("--copies", type=int, default=0, help="independent cache copies to rotate over (0 = auto)")
+    ap.add_argument("--splits", type=int, default=0)
+    ap.add_argument("--variant", type=int, default=0)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build measures the one-GPU kernel path only; run with --gpus 1 "
+              "(no collectives, sharding or multi-rank code exists in this path)", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    import kitty_amd
+    from kitty_amd import _lib
+    lib = _lib.lib()                     # raises when the HIP library is not built: no fallback
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    dev = torch.device("cuda:0")
+    B, H_Q, H_KV, T, desc = WORKLOADS[args.workload]
+    D = 128
+    cfg = types.SimpleNamespace(num_hidden_layers=1, head_dim=D, num_key_value_heads=H_KV,
+                                num_attention_heads=H_Q, hidden_size=H_Q * D)
+    max_len = T + 256
+
+    # ---- build the packed caches with the quantizer under test ---------------------------------
+    K, V = synth_kv(B, H_KV, T, D, 1000 + int(args.workload[1]), dev)
+    probe = kitty_amd.KittyCache(cfg, B, max_len, device=dev)
+    probe.update(K, V, 0)
+    probe.quantize_prefill(0)
+    total_bytes, packed_bytes = algorithmic_bytes(B, H_Q, H_KV, probe.kv_cache[0])
+    copies = args.copies or max(2, -(-3 * 256 * 2 ** 20 // total_bytes))      # > 3x the Infinity Cache
+    caches = [probe]
+    quant_ms = []
+    for i in range(1, copies + 2):       # the extra rounds only time the quantizer
+        c = caches[i] if i < len(caches) else kitty_amd.KittyCache(cfg, B, max_len, device=dev)
+        c.update(K, V, 0)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        c.quantize_prefill(0)
+        e1.record()
+        torch.cuda.synchronize()
+        quant_ms.append(e0.elapsed_time(e1))
+        if i < copies:
+            caches.append(c)
+    L0 = probe.kv_cache[0]
+    quant_in_bytes = 2 * B * H_KV * (L0.PageCount_K + L0.PageCount_V) * 128 * D
+    quant_gbps = quant_in_bytes / (min(quant_ms) * 1e-3) / 1e9
+
+    q = torch.randn((B, H_Q, 1, D), generator=torch.Generator(device=dev).manual_seed(7), device=dev,
+                    dtype=torch.float32).half()
+    out = torch.empty((B, 1, H_Q, D), dtype=torch.float16, device=dev)
+    max_tiles = 1 + (T - L0.Sink_Count + 127) // 128
+    splits = args.splits or lib.kitty_decode_attn_default_splits(B, H_KV, max_tiles)
+    ws_bytes = lib.kitty_decode_attn_workspace_bytes(B, H_Q, D, splits)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    descs = [c.kv_cache[0].descriptor() for c in caches]
+    stream = torch.cuda.current_stream(dev).cuda_stream
+    scaling = D ** -0.5
+
+    def step(i, ev=None):
+        d = descs[i % len(descs)]
+        if ev is not None:
+            ev[0].record()
+        rc = lib.kitty_decode_attn_split(d, q.data_ptr(), B, H_Q, scaling, ws.data_ptr(), ws_bytes, splits,
+                                         args.variant, stream)
+        if ev is not None:
+            ev[1].record()
+        _lib.check(rc, "split")
+        _lib.check(lib.kitty_decode_attn_merge(ws.data_ptr(), ws_bytes, B, H_Q, D, splits, out.data_ptr(), stream),
+                   "merge")
+
+    for i in range(args.warmup):
+        step(i)
+    torch.cuda.synchronize()
+    events = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        step(i, events[i])
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms_per_step = wall / args.steps * 1e3
+    kern_us = sorted(a.elapsed_time(b) * 1e3 for a, b in events)
+    kern_avg_us = sum(kern_us) / len(kern_us)
+    achieved = total_bytes / (kern_avg_us * 1e-6) / 1e9
+
+    # cache-hot figure (same copy every step), reported separately
+    hot_ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(20)]
+    for i in range(20):
+        step(0, hot_ev[i])
+    torch.cuda.synchronize()
+    hot_us = sorted(a.elapsed_time(b) * 1e3 for a, b in hot_ev)[len(hot_ev) // 2]
+
+    result = {
+        "metric": "packed_kv_decode_attention_us_per_step",
+        "value": ms_per_step * 1e3,
+        "unit": "us/step",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": False,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "u8 codes + f16 scales/zeros, f32 accumulate",
+        "data": "synthetic (seeded N(0,1) K with 8 outlier channels/head x10, N(0,1) V, random-init)",
+        "config": {"workload": desc, "batch": B, "q_heads": H_Q, "kv_heads": H_KV, "head_dim": D, "context": T,
+                   "pages_k": L0.PageCount_K, "pages_v": L0.PageCount_V, "num_splits": splits,
+                   "variant": args.variant, "cache_copies_rotated": len(caches)},
+        "roofline": {
+            "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+            "frac": achieved / HBM_PEAK_GBPS, "traffic": None,
+            "kernel": "decode split pass", "kernel_avg_us": kern_avg_us, "kernel_median_us": kern_us[len(kern_us) // 2],
+            "algorithmic_bytes_per_launch": total_bytes, "packed_bytes_per_launch": packed_bytes,
+            "packed_gbps": packed_bytes / (kern_avg_us * 1e-6) / 1e9,
+            "packed_frac": packed_bytes / (kern_avg_us * 1e-6) / 1e9 / HBM_PEAK_GBPS,
+            "cache_hot_kernel_us": hot_us,
+        },
+        "quantizer": {"gbps_in": quant_gbps, "ms": min(quant_ms), "input_bytes": quant_in_bytes,
+                      "what": "quantize_prefill of the whole context (K select+quantize+pack, V quantize+pack)"},
+    }
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(K[:1].cpu(), V[:1].cpu(), q[:1].cpu(), H_Q, H_KV, B)
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,149 @@
+/*
+ * kitty_hip.h - C ABI of the MI355X (gfx950) implementation of Kitty's quantized-KV hot path.
+ *
+ * Every entry point is asynchronous and ordered on the HIP stream passed in (NULL = the default
+ * stream), allocates nothing, frees nothing and keeps no state between calls except a thread-local
+ * error string.  All data pointers are device pointers owned by the caller.  Return value: 0 on
+ * success, a negative KITTY_E_* code when an argument is rejected on the host before anything is
+ * launched, a positive hipError_t when a launch fails.  kitty_last_error() describes the last
+ * failure on the calling thread.
+ *
+ * Each function names the reference interface it replaces (paths relative to the reference
+ * checkout, src/kitty/kvcache/...).
+ */
+#ifndef KITTY_HIP_H
+#define KITTY_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define KITTY_ABI_VERSION 1
+
+enum {
+  KITTY_OK = 0,
+  KITTY_E_NULL = -1,        /* a required pointer is NULL */
+  KITTY_E_SHAPE = -2,       /* unsupported head_dim / page_size / boost count / group size */
+  KITTY_E_RANGE = -3,       /* a count or offset is out of range for the buffers described */
+  KITTY_E_ALIGN = -4,       /* a pointer or stride breaks the alignment the kernels rely on */
+  KITTY_E_WORKSPACE = -5    /* workspace too small */
+};
+
+/*
+ * One layer's storage, field for field the tensors of the reference's KVCache_Layer
+ * (utils_kv_per_layer.py:12-95).  Strides are in bytes.  fp16 windows are [MAX_BS, H_KV, rows, D]
+ * with D contiguous; *_stride_b / *_stride_h give their batch and head strides.
+ *
+ * Occupancy is given either by the scalar counters (the reference: host ints shared by the whole
+ * batch, utils_kv_per_layer.py:53-54,65,71-72,79-80) or, when seq_counts is not NULL, per
+ * sequence: int32 [B][KITTY_SEQ_COUNT_FIELDS] on the device in the order of the enum below.
+ */
+enum {
+  KITTY_CNT_SINK = 0,       /* Sink_Count            (0..S)                                   */
+  KITTY_CNT_PAGES_K = 1,    /* PageCount_K                                                    */
+  KITTY_CNT_QBUF_K = 2,     /* Q_Buffer_Count_K      (0..PAGE_SIZE)                           */
+  KITTY_CNT_PAGES_V = 3,    /* PageCount_V                                                    */
+  KITTY_CNT_QBUF_V = 4,     /* Q_Buffer_Count_V      (0..PAGE_SIZE)                           */
+  KITTY_CNT_LOCAL_V = 5,    /* Local_Count_V         (0..PAGE_SIZE)                           */
+  KITTY_CNT_LOCAL_OFF = 6,  /* Write_Offset_Local_V  (ring head = oldest row)                 */
+  KITTY_CNT_RESERVED = 7,
+  KITTY_SEQ_COUNT_FIELDS = 8
+};
+
+typedef struct kitty_kv_layer {
+  int32_t H_KV, D, D_BOOSTED, PAGE_SIZE, S, MAX_PAGE;
+  int32_t counts[KITTY_SEQ_COUNT_FIELDS];       /* used when seq_counts == NULL */
+  const int32_t* seq_counts;                    /* optional, device, [B][8] */
+
+  const uint8_t* key_cache;    int64_t key_cache_stride_page;     /* KeyCache            */
+  const void*    key_meta;     int64_t key_meta_stride_page;      /* KeyCache_metadata   */
+  const uint8_t* value_cache;  int64_t value_cache_stride_page;   /* ValueCache          */
+  const void*    value_meta;   int64_t value_meta_stride_page;    /* ValueCache_metadata */
+  const int64_t* page_table_k; int64_t page_table_k_stride_b;     /* PageTable_K         */
+  const int64_t* page_table_v; int64_t page_table_v_stride_b;     /* PageTable_V         */
+
+  const void* sink_k;  const void* sink_v;      /* Sink_Buffer_K/V  [MAX_BS,H_KV,S,D]         */
+  int64_t sink_stride_b, sink_stride_h;
+  const void* qbuf_k;  const void* qbuf_v;      /* Q_Buffer_K/V     [MAX_BS,H_KV,PAGE_SIZE,D] */
+  const void* local_v;                          /* Local_Buffer_V   [MAX_BS,H_KV,PAGE_SIZE,D] */
+  int64_t win_stride_b, win_stride_h;           /* shared by the three PAGE_SIZE-row windows  */
+} kitty_kv_layer;
+
+int kitty_abi_version(void);
+const char* kitty_last_error(void);
+
+/*
+ * Channel-boost selection.  Replaces the torch ops of quantize_pack_k
+ * (kernels/kitty_quant_pack.py:275-288): score = mean over the page's tokens of |K| rounded to
+ * fp16, top-d_boost channels, slot_map[ch] = rank or d_boost.  Tie rule: higher score first, then
+ * lower channel index.  key is fp16 [B,H,T,D] with D contiguous and byte strides as given; pages
+ * are the `pages` consecutive PAGE_SIZE-token groups starting at token t_offset.
+ * slot_map: uint8 [B,H,pages,D] contiguous.
+ */
+int kitty_select_boost_k(const void* key, int64_t stride_b, int64_t stride_h, int64_t stride_t,
+                         int B, int H, int T, int D, int t_offset, int pages, int page_size, int d_boost,
+                         uint8_t* slot_map, void* stream);
+
+/*
+ * Replaces quantize_pack_k_kernel and its launch (kernels/kitty_quant_pack.py:13-152, 291-312).
+ * Quantizes `pages` pages of every (b,h) into cache pages page_table[b][page_offset + p].
+ * slot_map NULL: the selection above is fused into the same kernel (one pass over K).
+ * slot_map given: uint8 [B,H,pages,D], consumed exactly like the reference kernel consumes
+ * dense_sparse_idx.  meta is fp16 [pages_total,H,D,2] (scale, zero).
+ */
+int kitty_quant_pack_k(const void* key, int64_t stride_b, int64_t stride_h, int64_t stride_t,
+                       int B, int H, int T, int D, int t_offset, int pages, int page_size, int d_boost,
+                       const uint8_t* slot_map,
+                       const int64_t* page_table, int64_t page_table_stride_b, int page_offset,
+                       uint8_t* cache, int64_t cache_stride_page,
+                       void* meta, int64_t meta_stride_page,
+                       int64_t cache_pages, void* stream);
+
+/*
+ * Replaces quantize_pack_v_kernel and its launch (kernels/kitty_quant_pack.py:155-249, 339-356).
+ * meta is fp16 [pages_total,H,PAGE_SIZE,2] (scale, zero) per token.
+ */
+int kitty_quant_pack_v(const void* value, int64_t stride_b, int64_t stride_h, int64_t stride_t,
+                       int B, int H, int T, int D, int t_offset, int pages, int page_size,
+                       const int64_t* page_table, int64_t page_table_stride_b, int page_offset,
+                       uint8_t* cache, int64_t cache_stride_page,
+                       void* meta, int64_t meta_stride_page,
+                       int64_t cache_pages, void* stream);
+
+/*
+ * Decode attention over the packed cache.  Replaces qk_kernel + torch softmax + sv_kernel as
+ * orchestrated by kitty_attention_forward (kernels/kitty_attention.py:403-526): one fused
+ * split-K pass (QK^T, online softmax, PV per split of the sequence) and a merge pass.
+ * q: fp16 [B,H_Q,1,D] contiguous.  out: fp16 [B,1,H_Q,D] contiguous.
+ * workspace: at least kitty_decode_attn_workspace_bytes(B,H_Q,D,num_splits) bytes, 256-aligned.
+ * num_splits <= 0 picks kitty_decode_attn_default_splits().  variant: 0 = default kernel,
+ * 1 = the plain reference-order kernel (fp16 dequantization, no matrix cores).
+ */
+size_t kitty_decode_attn_workspace_bytes(int B, int H_Q, int D, int num_splits);
+int kitty_decode_attn_default_splits(int B, int H_KV, int max_tiles);
+int kitty_decode_attn(const kitty_kv_layer* layer, const void* q, int B, int H_Q, float scaling,
+                      void* out, void* workspace, size_t workspace_bytes, int num_splits,
+                      int variant, void* stream);
+
+/*
+ * The two passes of kitty_decode_attn on their own.  The split pass leaves, per (b, hq, split),
+ * the running maximum of the logits in log2 units, the running sum and the un-normalised output
+ * in the workspace; the merge pass combines `num_splits` such partials per (b, hq).  A caller that
+ * shards one long sequence over several devices runs the split pass on each shard, gathers the
+ * partials into one workspace (splits of all shards side by side) and runs the merge pass once.
+ * No counterpart in the reference, whose grid is (B, H_KV) with no split over the sequence
+ * (kernels/kitty_attention.py:433,484).
+ */
+int kitty_decode_attn_split(const kitty_kv_layer* layer, const void* q, int B, int H_Q, float scaling,
+                            void* workspace, size_t workspace_bytes, int num_splits, int variant,
+                            void* stream);
+int kitty_decode_attn_merge(const void* workspace, size_t workspace_bytes, int B, int H_Q, int D,
+                            int num_splits, void* out, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* KITTY_HIP_H */

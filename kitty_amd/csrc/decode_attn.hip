@@ -1,0 +1,134 @@
+// C ABI entry points of decode attention: argument checks on the host, then the fused split-K
+// pass and the merge pass on the caller's stream.
+#include "decode_common.h"
+
+namespace kitty {
+void launch_decode_plain(const kitty_kv_layer& L, const void* q, int B, int H_Q, float scaling, float* ws_ml,
+                         float* ws_acc, int num_splits, hipStream_t stream);
+void launch_decode_merge(const float* ws_ml, const float* ws_acc, void* out, int B, int H_Q, int num_splits,
+                         hipStream_t stream);
+bool decode_mfma_supported(const kitty_kv_layer& L, int H_Q);
+void launch_decode_mfma(const kitty_kv_layer& L, const void* q, int B, int H_Q, float scaling, float* ws_ml,
+                        float* ws_acc, int num_splits, hipStream_t stream);
+}  // namespace kitty
+
+using namespace kitty;
+
+extern "C" size_t kitty_decode_attn_workspace_bytes(int B, int H_Q, int D, int num_splits) {
+  if (B <= 0 || H_Q <= 0 || D != kD || num_splits <= 0) return 0;
+  return ws_total_bytes(B, H_Q, num_splits);
+}
+
+// Enough workgroups to cover every SIMD of the 256 CUs a few times over, never more splits than
+// there are tiles.
+extern "C" int kitty_decode_attn_default_splits(int B, int H_KV, int max_tiles) {
+  if (B <= 0 || H_KV <= 0 || max_tiles <= 0) return 1;
+  const int units = B * H_KV;
+  int s = (2048 + units - 1) / units;
+  if (s > max_tiles) s = max_tiles;
+  if (s > 512) s = 512;
+  return s < 1 ? 1 : s;
+}
+
+namespace {
+
+int check_layer(const kitty_kv_layer* layer, const void* q, int B, int H_Q, int* max_tiles) {
+  KITTY_REQUIRE(layer && q, KITTY_E_NULL, "layer / q is NULL");
+  const kitty_kv_layer& L = *layer;
+  KITTY_REQUIRE(L.D == kD && L.PAGE_SIZE == kPage, KITTY_E_SHAPE,
+                "kernels are built for head_dim 128 and page_size 128, got D=%d page_size=%d", L.D, L.PAGE_SIZE);
+  KITTY_REQUIRE(L.H_KV >= 1 && H_Q >= L.H_KV && H_Q % L.H_KV == 0, KITTY_E_SHAPE,
+                "H_Q=%d must be a positive multiple of H_KV=%d", H_Q, L.H_KV);
+  KITTY_REQUIRE(H_Q / L.H_KV <= 16, KITTY_E_SHAPE, "KV_GROUP (%d) exceeds MAX_KV_GROUP (16)", H_Q / L.H_KV);
+  KITTY_REQUIRE(L.D_BOOSTED >= 0 && L.D_BOOSTED <= kD && k_head_bytes(L.D_BOOSTED) % 16 == 0, KITTY_E_SHAPE,
+                "unsupported D_BOOSTED=%d", L.D_BOOSTED);
+  KITTY_REQUIRE(L.S >= 0 && L.S <= kPage && L.MAX_PAGE >= 0, KITTY_E_SHAPE, "S=%d must be in [0, 128]", L.S);
+  KITTY_REQUIRE(B >= 1 && B <= 65535 && L.H_KV <= 65535, KITTY_E_RANGE, "bad batch size %d", B);
+  KITTY_REQUIRE(L.key_cache && L.key_meta && L.value_cache && L.value_meta && L.page_table_k && L.page_table_v &&
+                    L.sink_k && L.sink_v && L.qbuf_k && L.qbuf_v && L.local_v,
+                KITTY_E_NULL, "a cache tensor pointer is NULL");
+  KITTY_REQUIRE(((uintptr_t)L.key_cache % 16) == 0 && L.key_cache_stride_page % 16 == 0 &&
+                    ((uintptr_t)L.value_cache % 16) == 0 && L.value_cache_stride_page % 16 == 0 &&
+                    ((uintptr_t)L.key_meta % 16) == 0 && L.key_meta_stride_page % 16 == 0 &&
+                    ((uintptr_t)L.value_meta % 16) == 0 && L.value_meta_stride_page % 16 == 0 &&
+                    ((uintptr_t)L.sink_k % 16) == 0 && ((uintptr_t)L.sink_v % 16) == 0 &&
+                    ((uintptr_t)L.qbuf_k % 16) == 0 && ((uintptr_t)L.qbuf_v % 16) == 0 &&
+                    ((uintptr_t)L.local_v % 16) == 0 && L.sink_stride_b % 16 == 0 && L.sink_stride_h % 16 == 0 &&
+                    L.win_stride_b % 16 == 0 && L.win_stride_h % 16 == 0 && ((uintptr_t)q % 16) == 0,
+                KITTY_E_ALIGN, "cache tensors and q need 16-byte alignment");
+  KITTY_REQUIRE(L.key_cache_stride_page >= (int64_t)L.H_KV * k_head_bytes(L.D_BOOSTED) &&
+                    L.value_cache_stride_page >= (int64_t)L.H_KV * kVBytes &&
+                    L.key_meta_stride_page >= (int64_t)L.H_KV * kD * 4 &&
+                    L.value_meta_stride_page >= (int64_t)L.H_KV * kPage * 4,
+                KITTY_E_RANGE, "a page stride is smaller than one page");
+  *max_tiles = 2 + L.MAX_PAGE;
+  if (!L.seq_counts) {
+    const int* c = L.counts;
+    KITTY_REQUIRE(c[KITTY_CNT_SINK] >= 0 && c[KITTY_CNT_SINK] <= L.S && c[KITTY_CNT_PAGES_K] >= 0 &&
+                      c[KITTY_CNT_PAGES_K] <= L.MAX_PAGE && c[KITTY_CNT_PAGES_V] >= 0 &&
+                      c[KITTY_CNT_PAGES_V] <= L.MAX_PAGE && c[KITTY_CNT_QBUF_K] >= 0 &&
+                      c[KITTY_CNT_QBUF_K] <= kPage && c[KITTY_CNT_QBUF_V] >= 0 && c[KITTY_CNT_QBUF_V] <= kPage &&
+                      c[KITTY_CNT_LOCAL_V] >= 0 && c[KITTY_CNT_LOCAL_V] <= kPage && c[KITTY_CNT_LOCAL_OFF] >= 0 &&
+                      c[KITTY_CNT_LOCAL_OFF] < kPage,
+                  KITTY_E_RANGE, "a cache counter is out of range");
+    const int nk = c[KITTY_CNT_PAGES_K] * kPage + c[KITTY_CNT_QBUF_K];
+    const int nv = c[KITTY_CNT_PAGES_V] * kPage + c[KITTY_CNT_QBUF_V] + c[KITTY_CNT_LOCAL_V];
+    KITTY_REQUIRE(nk == nv, KITTY_E_RANGE, "seqlen_K: %d, seqlen_V: %d", nk + c[KITTY_CNT_SINK],
+                  nv + c[KITTY_CNT_SINK]);
+    *max_tiles = 1 + (nk + kPage - 1) / kPage;
+  }
+  return 0;
+}
+
+int check_workspace(const void* workspace, size_t workspace_bytes, int B, int H_Q, int num_splits) {
+  KITTY_REQUIRE(workspace != nullptr, KITTY_E_NULL, "workspace is NULL");
+  KITTY_REQUIRE(((uintptr_t)workspace % 256) == 0, KITTY_E_ALIGN, "workspace needs 256-byte alignment");
+  KITTY_REQUIRE(num_splits >= 1 && num_splits <= 65535, KITTY_E_RANGE, "num_splits=%d out of range", num_splits);
+  KITTY_REQUIRE(workspace_bytes >= ws_total_bytes(B, H_Q, num_splits), KITTY_E_WORKSPACE,
+                "workspace of %zu bytes is smaller than the %zu needed for %d splits", workspace_bytes,
+                ws_total_bytes(B, H_Q, num_splits), num_splits);
+  return 0;
+}
+
+}  // namespace
+
+extern "C" int kitty_decode_attn_split(const kitty_kv_layer* layer, const void* q, int B, int H_Q, float scaling,
+                                       void* workspace, size_t workspace_bytes, int num_splits, int variant,
+                                       void* stream) {
+  int max_tiles = 0;
+  if (int rc = check_layer(layer, q, B, H_Q, &max_tiles)) return rc;
+  if (int rc = check_workspace(workspace, workspace_bytes, B, H_Q, num_splits)) return rc;
+  KITTY_REQUIRE(variant == 0 || variant == 1, KITTY_E_SHAPE, "unknown variant %d", variant);
+  const kitty_kv_layer& L = *layer;
+  float* ws_ml = (float*)workspace;
+  float* ws_acc = (float*)((uint8_t*)workspace + ws_ml_bytes(B, H_Q, num_splits));
+  if (variant == 0 && decode_mfma_supported(L, H_Q))
+    launch_decode_mfma(L, q, B, H_Q, scaling, ws_ml, ws_acc, num_splits, (hipStream_t)stream);
+  else
+    launch_decode_plain(L, q, B, H_Q, scaling, ws_ml, ws_acc, num_splits, (hipStream_t)stream);
+  return check_launch("kitty_decode_attn_split");
+}
+
+extern "C" int kitty_decode_attn_merge(const void* workspace, size_t workspace_bytes, int B, int H_Q, int D,
+                                       int num_splits, void* out, void* stream) {
+  KITTY_REQUIRE(out != nullptr, KITTY_E_NULL, "out is NULL");
+  KITTY_REQUIRE(D == kD && B >= 1 && B <= 65535 && H_Q >= 1, KITTY_E_SHAPE, "bad B=%d H_Q=%d D=%d", B, H_Q, D);
+  KITTY_REQUIRE(((uintptr_t)out % 16) == 0, KITTY_E_ALIGN, "out needs 16-byte alignment");
+  if (int rc = check_workspace(workspace, workspace_bytes, B, H_Q, num_splits)) return rc;
+  const float* ws_ml = (const float*)workspace;
+  const float* ws_acc = (const float*)((const uint8_t*)workspace + ws_ml_bytes(B, H_Q, num_splits));
+  launch_decode_merge(ws_ml, ws_acc, out, B, H_Q, num_splits, (hipStream_t)stream);
+  return check_launch("kitty_decode_attn_merge");
+}
+
+extern "C" int kitty_decode_attn(const kitty_kv_layer* layer, const void* q, int B, int H_Q, float scaling,
+                                 void* out, void* workspace, size_t workspace_bytes, int num_splits, int variant,
+                                 void* stream) {
+  int max_tiles = 0;
+  if (int rc = check_layer(layer, q, B, H_Q, &max_tiles)) return rc;
+  if (num_splits <= 0) num_splits = kitty_decode_attn_default_splits(B, layer->H_KV, max_tiles);
+  if (int rc = kitty_decode_attn_split(layer, q, B, H_Q, scaling, workspace, workspace_bytes, num_splits, variant,
+                                       stream))
+    return rc;
+  return kitty_decode_attn_merge(workspace, workspace_bytes, B, H_Q, layer->D, num_splits, out, stream);
+}

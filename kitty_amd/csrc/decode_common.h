@@ -1,0 +1,60 @@
+// Pieces shared by the decode-attention kernels: per-sequence occupancy, the tiling of a
+// sequence into 128-token tiles, the split-K workspace layout and the merge kernel.
+//
+// Token order (kitty_attention.py:89-207 for K, :270-386 for V) is chronological on both sides:
+//   K: [ sink rows | packed pages | Q_Buffer_K rows ]
+//   V: [ sink rows | packed pages | Q_Buffer_V rows | Local_Buffer_V rows from the ring head ]
+// Both sides start their pages right after the sink, so "body tile" i (tokens 128*i .. 128*i+127
+// after the sink) is K page i when i < PageCount_K, else the K Q-buffer; on the V side it is V
+// page i when i < PageCount_V, else rows of the fp16 region [Q_Buffer_V | Local ring].
+// Tile 0 is the sink; body tile i is tile i+1.
+#pragma once
+#include "kitty_common.h"
+
+namespace kitty {
+
+struct SeqCounts {
+  int sink, pk, rk, pv, rv, lv, off;
+  int nbody;    // tokens after the sink
+  int ntiles;   // 1 (sink) + ceil(nbody / 128)
+};
+
+__device__ inline SeqCounts load_counts(const kitty_kv_layer& L, int b) {
+  int c[KITTY_SEQ_COUNT_FIELDS];
+#pragma unroll
+  for (int i = 0; i < KITTY_SEQ_COUNT_FIELDS; ++i)
+    c[i] = L.seq_counts ? L.seq_counts[b * KITTY_SEQ_COUNT_FIELDS + i] : L.counts[i];
+  SeqCounts s;
+  // clamp to what the buffers hold: device-side counts cannot be validated on the host
+  s.sink = min(max(c[KITTY_CNT_SINK], 0), L.S);
+  s.pk = min(max(c[KITTY_CNT_PAGES_K], 0), L.MAX_PAGE);
+  s.rk = min(max(c[KITTY_CNT_QBUF_K], 0), kPage);
+  s.pv = min(max(c[KITTY_CNT_PAGES_V], 0), L.MAX_PAGE);
+  s.rv = min(max(c[KITTY_CNT_QBUF_V], 0), kPage);
+  s.lv = min(max(c[KITTY_CNT_LOCAL_V], 0), kPage);
+  s.off = c[KITTY_CNT_LOCAL_OFF] & (kPage - 1);
+  s.nbody = min(s.pk * kPage + s.rk, s.pv * kPage + s.rv + s.lv);
+  s.ntiles = 1 + (s.nbody + kPage - 1) / kPage;
+  return s;
+}
+
+// fp16 row of V for token u of the region that follows the V pages
+__device__ inline const __half* v_tail_row(const kitty_kv_layer& L, const SeqCounts& c, int b, int h, int u) {
+  const int64_t base = (int64_t)b * L.win_stride_b + (int64_t)h * L.win_stride_h;
+  if (u < c.rv) return (const __half*)((const uint8_t*)L.qbuf_v + base) + (int64_t)u * kD;
+  const int r = (c.off + (u - c.rv)) & (kPage - 1);
+  return (const __half*)((const uint8_t*)L.local_v + base) + (int64_t)r * kD;
+}
+
+// Split-K workspace: [B*H_Q*splits][2] floats (running max of the logits in log2 units, i.e.
+// logit * log2(e); running sum of 2^(logit2 - max)), then 256-aligned, [B*H_Q*splits][D] floats
+// of un-normalised output.
+__host__ __device__ inline size_t ws_ml_bytes(int B, int H_Q, int splits) {
+  size_t n = (size_t)B * H_Q * splits * 2 * sizeof(float);
+  return (n + 255) & ~(size_t)255;
+}
+__host__ __device__ inline size_t ws_total_bytes(int B, int H_Q, int splits) {
+  return ws_ml_bytes(B, H_Q, splits) + (size_t)B * H_Q * splits * kD * sizeof(float);
+}
+
+}  // namespace kitty

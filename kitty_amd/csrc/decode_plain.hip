@@ -1,0 +1,198 @@
+// Decode attention, plain variant: the reference's order of operations (dequantize a tile to fp16
+// with fp16 arithmetic, fp32 dot products, logits rounded to fp16) in one fused split-K pass on
+// the vector ALUs.  It is the readable baseline the matrix-core kernel is checked against on the
+// GPU and it accepts every boost count; it is not the fast path.
+#include "decode_common.h"
+
+using namespace kitty;
+
+namespace kitty {
+
+constexpr int kMaxGroup = 16;                        // kitty_attention.py:418
+constexpr int kMaxHeadBytes = kRowBytes * (kD + kD) + kD;   // d_boost up to D
+
+#pragma clang fp contract(off)
+__device__ inline float dequant_ref(uint32_t code, __half scale, __half zero) {
+  // fp16(code) * scale + zero with both operations rounded to fp16 (kitty_attention.py:162-165)
+  return __half2float(__hadd(__hmul(__ushort2half_rn((unsigned short)code), scale), zero));
+}
+#pragma clang fp contract(fast)
+
+__global__ __launch_bounds__(256) void decode_plain_kernel(kitty_kv_layer L, const __half* __restrict__ q, int H_Q,
+                                                           float scaling, float* __restrict__ ws_ml,
+                                                           float* __restrict__ ws_acc, int num_splits) {
+  const int split = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int G = H_Q / L.H_KV;
+  const int DB = L.D_BOOSTED;
+  const SeqCounts c = load_counts(L, b);
+  const int per = (c.ntiles + num_splits - 1) / num_splits;
+  const int tile_begin = split * per, tile_end = min(c.ntiles, tile_begin + per);
+
+  __shared__ float s_q[kMaxGroup][kD];
+  __shared__ __attribute__((aligned(16))) uint8_t s_codes[kMaxHeadBytes];
+  __shared__ __half2 s_meta[kD];
+  __shared__ float s_p[kMaxGroup][kPage];
+  __shared__ float s_part[2][kMaxGroup][kPage];
+  __shared__ float s_m[kMaxGroup], s_l[kMaxGroup], s_alpha[kMaxGroup];
+
+  for (int i = tid; i < G * kD; i += 256)
+    s_q[i / kD][i % kD] = __half2float(q[((int64_t)b * H_Q + (int64_t)h * G) * kD + i]);
+  if (tid < kMaxGroup) { s_m[tid] = -INFINITY; s_l[tid] = 0.f; }
+  float acc_o[kMaxGroup];
+#pragma unroll
+  for (int g = 0; g < kMaxGroup; ++g) acc_o[g] = 0.f;
+  __syncthreads();
+
+  const int t = tid & 127, half = tid >> 7;
+  const int64_t sink_base = (int64_t)b * L.sink_stride_b + (int64_t)h * L.sink_stride_h;
+  const int64_t win_base = (int64_t)b * L.win_stride_b + (int64_t)h * L.win_stride_h;
+
+  for (int tile = tile_begin; tile < tile_end; ++tile) {
+    const int body = tile - 1;                                  // -1 = sink
+    const int ntok = tile == 0 ? c.sink : min(kPage, c.nbody - body * kPage);
+    const bool k_packed = tile > 0 && body < c.pk;
+    const bool v_packed = tile > 0 && body < c.pv;
+
+    // ---- logits -----------------------------------------------------------------------------
+    float acc[kMaxGroup];
+#pragma unroll
+    for (int g = 0; g < kMaxGroup; ++g) acc[g] = 0.f;
+    if (k_packed) {
+      const int64_t pg = L.page_table_k[(int64_t)b * L.page_table_k_stride_b + body];
+      const uint8_t* src = L.key_cache + pg * L.key_cache_stride_page + (int64_t)h * k_head_bytes(DB);
+      for (int i = tid; i < k_head_bytes(DB) / 16; i += 256) ((uint4*)s_codes)[i] = ((const uint4*)src)[i];
+      if (tid < kD)
+        s_meta[tid] = *(const __half2*)((const uint8_t*)L.key_meta + pg * L.key_meta_stride_page +
+                                        ((int64_t)h * kD + tid) * 4);
+      __syncthreads();
+      const int sh = 2 * (t & 3);
+      const uint8_t* idx = s_codes + kRowBytes * (kD + DB);
+      for (int d = half * 64; d < half * 64 + 64; ++d) {
+        uint32_t code = (s_codes[d * kRowBytes + (t >> 2)] >> sh) & 3u;
+        const uint32_t slot = idx[d];
+        if (slot < (uint32_t)DB) code |= ((s_codes[kLoBytes + slot * kRowBytes + (t >> 2)] >> sh) & 3u) << 2;
+        const __half2 m = s_meta[d];
+        const float x = dequant_ref(code, __low2half(m), __high2half(m));
+#pragma unroll
+        for (int g = 0; g < kMaxGroup; ++g)
+          if (g < G) acc[g] += s_q[g][d] * x;
+      }
+    } else if (t < ntok) {
+      const __half* row = tile == 0 ? (const __half*)((const uint8_t*)L.sink_k + sink_base) + (int64_t)t * kD
+                                    : (const __half*)((const uint8_t*)L.qbuf_k + win_base) + (int64_t)t * kD;
+      for (int d = half * 64; d < half * 64 + 64; ++d) {
+        const float x = __half2float(row[d]);
+#pragma unroll
+        for (int g = 0; g < kMaxGroup; ++g)
+          if (g < G) acc[g] += s_q[g][d] * x;
+      }
+    }
+#pragma unroll
+    for (int g = 0; g < kMaxGroup; ++g)
+      if (g < G) s_part[half][g][t] = acc[g];
+    __syncthreads();
+
+    // ---- online softmax: one wave per query head ---------------------------------------------
+    for (int g = wave; g < G; g += 4) {
+      float v0 = -INFINITY, v1 = -INFINITY;
+      if (lane < ntok) v0 = __half2float(__float2half_rn((s_part[0][g][lane] + s_part[1][g][lane]) * scaling));
+      if (lane + 64 < ntok)
+        v1 = __half2float(__float2half_rn((s_part[0][g][lane + 64] + s_part[1][g][lane + 64]) * scaling));
+      float mx = fmaxf(v0, v1);
+#pragma unroll
+      for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
+      const float m_old = s_m[g];
+      const float m_new = fmaxf(m_old, mx);
+      const float p0 = (v0 == -INFINITY) ? 0.f : __expf(v0 - m_new);
+      const float p1 = (v1 == -INFINITY) ? 0.f : __expf(v1 - m_new);
+      float sum = p0 + p1;
+#pragma unroll
+      for (int o = 32; o > 0; o >>= 1) sum += __shfl_xor(sum, o);
+      const float alpha = (m_old == -INFINITY) ? 0.f : __expf(m_old - m_new);
+      s_p[g][lane] = p0;
+      s_p[g][lane + 64] = p1;
+      if (lane == 0) { s_m[g] = m_new; s_l[g] = s_l[g] * alpha + sum; s_alpha[g] = alpha; }
+    }
+    // ---- stage V ---------------------------------------------------------------------------
+    if (v_packed) {
+      const int64_t pg = L.page_table_v[(int64_t)b * L.page_table_v_stride_b + body];
+      const uint8_t* src = L.value_cache + pg * L.value_cache_stride_page + (int64_t)h * kVBytes;
+      ((uint4*)s_codes)[tid] = ((const uint4*)src)[tid];
+      if (tid < kPage)
+        s_meta[tid] = *(const __half2*)((const uint8_t*)L.value_meta + pg * L.value_meta_stride_page +
+                                        ((int64_t)h * kPage + tid) * 4);
+    }
+    __syncthreads();
+
+    // ---- out += P V : thread = (channel, half of the tile's tokens) ---------------------------
+    {
+      const int d = t;
+#pragma unroll
+      for (int g = 0; g < kMaxGroup; ++g)
+        if (g < G) acc_o[g] *= s_alpha[g];
+      const int t0 = half * 64, t1 = min(ntok, half * 64 + 64);
+      for (int tt = t0; tt < t1; ++tt) {
+        float x;
+        if (v_packed) {
+          const uint32_t code = (s_codes[tt * kRowBytes + (d >> 2)] >> (2 * (d & 3))) & 3u;
+          const __half2 m = s_meta[tt];
+          x = dequant_ref(code, __low2half(m), __high2half(m));
+        } else if (tile == 0) {
+          x = __half2float(((const __half*)((const uint8_t*)L.sink_v + sink_base))[(int64_t)tt * kD + d]);
+        } else {
+          x = __half2float(v_tail_row(L, c, b, h, (body - c.pv) * kPage + tt)[d]);
+        }
+#pragma unroll
+        for (int g = 0; g < kMaxGroup; ++g)
+          if (g < G) acc_o[g] += s_p[g][tt] * x;
+      }
+    }
+    __syncthreads();
+  }
+
+  // ---- write this split's partial --------------------------------------------------------------
+#pragma unroll
+  for (int g = 0; g < kMaxGroup; ++g)
+    if (g < G) s_part[half][g][t] = acc_o[g];
+  __syncthreads();
+  for (int i = tid; i < G * kD; i += 256) {
+    const int g = i / kD, d = i % kD;
+    const int64_t row = ((int64_t)b * H_Q + (int64_t)h * G + g) * num_splits + split;
+    ws_acc[row * kD + d] = s_part[0][g][d] + s_part[1][g][d];
+    if (d == 0) { ws_ml[row * 2] = s_m[g] * 1.44269504088896f; ws_ml[row * 2 + 1] = s_l[g]; }
+  }
+}
+
+// out[b, 0, hq, :] = sum_s acc_s * 2^(m_s - m) / sum_s l_s * 2^(m_s - m); the running maxima of
+// the partials are in log2 units.
+__global__ __launch_bounds__(128) void decode_merge_kernel(const float* __restrict__ ws_ml,
+                                                           const float* __restrict__ ws_acc,
+                                                           __half* __restrict__ out, int num_splits) {
+  const int64_t row0 = ((int64_t)blockIdx.y * gridDim.x + blockIdx.x) * num_splits;
+  const int d = threadIdx.x;
+  float m = -INFINITY;
+  for (int s = 0; s < num_splits; ++s) m = fmaxf(m, ws_ml[(row0 + s) * 2]);
+  float l = 0.f, o = 0.f;
+  for (int s = 0; s < num_splits; ++s) {
+    const float ms = ws_ml[(row0 + s) * 2];
+    const float w = (ms == -INFINITY) ? 0.f : exp2f(ms - m);
+    l += ws_ml[(row0 + s) * 2 + 1] * w;
+    o += ws_acc[(row0 + s) * kD + d] * w;
+  }
+  out[((int64_t)blockIdx.y * gridDim.x + blockIdx.x) * kD + d] = __float2half_rn(l > 0.f ? o / l : 0.f);
+}
+
+void launch_decode_plain(const kitty_kv_layer& L, const void* q, int B, int H_Q, float scaling, float* ws_ml,
+                         float* ws_acc, int num_splits, hipStream_t stream) {
+  hipLaunchKernelGGL(decode_plain_kernel, dim3(num_splits, L.H_KV, B), dim3(256), 0, stream, L, (const __half*)q,
+                     H_Q, scaling, ws_ml, ws_acc, num_splits);
+}
+
+void launch_decode_merge(const float* ws_ml, const float* ws_acc, void* out, int B, int H_Q, int num_splits,
+                         hipStream_t stream) {
+  hipLaunchKernelGGL(decode_merge_kernel, dim3(H_Q, B), dim3(kD), 0, stream, ws_ml, ws_acc, (__half*)out,
+                     num_splits);
+}
+
+}  // namespace kitty

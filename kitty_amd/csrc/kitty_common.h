@@ -1,0 +1,28 @@
+// Shared host/device helpers for the gfx950 kernels of the quantized-KV path.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdarg.h>
+
+#include "../../include/kitty_hip.h"
+
+namespace kitty {
+
+// Geometry the kernels are specialised for (the only one the reference uses: kitty.py:43-47).
+constexpr int kD = 128;        // head_dim
+constexpr int kPage = 128;     // tokens per page == quantization group
+constexpr int kRowBytes = 32;  // one 2-bit plane row: 128 codes
+constexpr int kLoBytes = kD * kRowBytes;                 // 4096: low plane of a K page-head
+constexpr int kVBytes = kPage * kRowBytes;               // 4096: a V page-head
+
+__host__ __device__ inline int k_head_bytes(int d_boost) { return kRowBytes * (kD + d_boost) + kD; }
+
+int set_error(int code, const char* fmt, ...);
+int check_launch(const char* what);
+
+}  // namespace kitty
+
+#define KITTY_REQUIRE(cond, code, ...) \
+  do { if (!(cond)) return kitty::set_error((code), __VA_ARGS__); } while (0)

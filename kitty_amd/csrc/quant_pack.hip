@@ -1,0 +1,311 @@
+// Quantize-and-pack kernels for gfx950: one workgroup per (page, kv-head, batch row).
+//
+// K pages: per-channel asymmetric quantization over the page's 128 tokens, 2 bits per code with
+// the boosted channels carrying 2 more bits in a second plane; the boost selection (mean |K| per
+// channel, top-d_boost) can run fused in the same pass over the tile.
+// V pages: per-token asymmetric 2-bit quantization over the 128 channels.
+//
+// Arithmetic contract (shared with the reference's Triton kernels, kitty_quant_pack.py:75-82,
+// 106-112, 201-204, 227-230): min/max, range, scale = range / qmax (IEEE fp32 divide, floored at
+// 1e-6), (x - min) / scale in fp32, floor(. + 0.5), clamp to [0, qmax]; the stored scale is the
+// fp32 scale rounded to fp16, the stored zero point is the minimum itself.
+#include "kitty_common.h"
+
+using namespace kitty;
+
+namespace {
+
+// |x| * 2^24 of an fp16 bit pattern as an exact integer (fits 41 bits for finite x).
+__device__ inline uint64_t abs_fixed(uint16_t bits) {
+  uint32_t e = (bits >> 10) & 31u, m = bits & 1023u;
+  return e == 0 ? (uint64_t)m : ((uint64_t)(1024u + m) << (e - 1));
+}
+
+// fp16 bit pattern of (S * 2^-31) rounded to nearest even, S = sum over 128 tokens of |x| * 2^24,
+// i.e. the mean of |x| rounded once.  Positive fp16 patterns order like their values.
+__device__ inline uint16_t mean_abs_fp16_bits(uint64_t S) {
+  if (S == 0) return 0;
+  int msb = 63 - __clzll((long long)S);
+  int E = msb - 31;
+  if (E >= -14) {
+    int shift = msb - 10;
+    uint64_t q;
+    if (shift > 0) {
+      q = S >> shift;
+      uint64_t rem = S & ((1ull << shift) - 1), half = 1ull << (shift - 1);
+      if (rem > half || (rem == half && (q & 1))) q++;
+    } else {
+      q = S << (-shift);
+    }
+    if (q == 2048) { q = 1024; E++; }
+    if (E > 15) return 0x7C00;
+    return (uint16_t)(((uint32_t)(E + 15) << 10) | (uint32_t)(q & 1023));
+  }
+  uint64_t q = S >> 7, rem = S & 127;
+  if (rem > 64 || (rem == 64 && (q & 1))) q++;
+  return (uint16_t)q;
+}
+
+__device__ inline float h2f(uint16_t bits) { return __half2float(__ushort_as_half(bits)); }
+
+// MODE 0: slot map given.  MODE 1: selection fused, then quantize.  MODE 2: selection only.
+template <int MODE>
+__global__ __launch_bounds__(256) void quant_pack_k_kernel(
+    const uint8_t* __restrict__ key, int64_t stride_b, int64_t stride_h, int64_t stride_t,
+    int t_offset, int d_boost,
+    const uint8_t* __restrict__ slot_map_in, uint8_t* __restrict__ slot_map_out, int pages,
+    const int64_t* __restrict__ page_table, int64_t pt_stride_b, int page_offset,
+    uint8_t* __restrict__ cache, int64_t cache_stride_page,
+    uint8_t* __restrict__ meta, int64_t meta_stride_page, int64_t cache_pages) {
+  const int p = blockIdx.x, h = blockIdx.y, b = blockIdx.z, H = gridDim.y;
+  const int tid = threadIdx.x;
+  const int tg = tid >> 4;   // tokens tg*8 .. tg*8+7
+  const int c8 = tid & 15;   // channels c8*8 .. c8*8+7
+
+  __shared__ float s_pmin[16][kD];
+  __shared__ float s_pmax[16][kD];
+  __shared__ uint64_t s_psum[MODE == 0 ? 1 : 16][kD];
+  __shared__ float s_scale[kD], s_min[kD], s_qmax[kD];
+  __shared__ uint16_t s_score[kD];
+  __shared__ __attribute__((aligned(16))) uint8_t s_idx[kD];
+  __shared__ __attribute__((aligned(16))) uint16_t s_lo[kD * 16];
+
+  const uint8_t* src = key + (int64_t)b * stride_b + (int64_t)h * stride_h +
+                       (int64_t)(t_offset + p * kPage + tg * 8) * stride_t + c8 * 16;
+  uint4 rows[8];
+#pragma unroll
+  for (int r = 0; r < 8; ++r) rows[r] = *(const uint4*)(src + (int64_t)r * stride_t);
+
+  // per-channel partial min / max (/ sum of |x|) over this thread's 8 tokens
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    float mn = INFINITY, mx = -INFINITY;
+    uint64_t sum = 0;
+#pragma unroll
+    for (int r = 0; r < 8; ++r) {
+      const uint32_t w = ((const uint32_t*)&rows[r])[j >> 1];
+      const uint16_t bits = (j & 1) ? (uint16_t)(w >> 16) : (uint16_t)(w & 0xffffu);
+      const float x = h2f(bits);
+      mn = fminf(mn, x);
+      mx = fmaxf(mx, x);
+      if (MODE != 0) sum += abs_fixed(bits);
+    }
+    s_pmin[tg][c8 * 8 + j] = mn;
+    s_pmax[tg][c8 * 8 + j] = mx;
+    if (MODE != 0) s_psum[tg][c8 * 8 + j] = sum;
+  }
+  __syncthreads();
+
+  float ch_min = 0.f, ch_max = 0.f;
+  if (tid < kD) {
+    float mn = s_pmin[0][tid], mx = s_pmax[0][tid];
+#pragma unroll
+    for (int i = 1; i < 16; ++i) { mn = fminf(mn, s_pmin[i][tid]); mx = fmaxf(mx, s_pmax[i][tid]); }
+    ch_min = mn; ch_max = mx;
+    if (MODE != 0) {
+      uint64_t sum = 0;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) sum += s_psum[i][tid];
+      s_score[tid] = mean_abs_fp16_bits(sum);
+    } else {
+      s_idx[tid] = slot_map_in[(((int64_t)b * H + h) * pages + p) * kD + tid];
+    }
+  }
+  if (MODE != 0) {
+    __syncthreads();
+    if (tid < kD) {
+      // rank = number of channels that sort before this one: higher score, or equal score and
+      // lower channel index
+      const uint16_t mine = s_score[tid];
+      int rank = 0;
+      for (int d = 0; d < kD; ++d) {
+        const uint16_t o = s_score[d];
+        rank += (o > mine) || (o == mine && d < tid);
+      }
+      const uint8_t slot = (uint8_t)(rank < d_boost ? rank : d_boost);
+      s_idx[tid] = slot;
+      if (slot_map_out) slot_map_out[(((int64_t)b * H + h) * pages + p) * kD + tid] = slot;
+    }
+    if (MODE == 2) return;
+  }
+
+  const int64_t pg = page_table[(int64_t)b * pt_stride_b + page_offset + p];
+  if (pg < 0 || pg >= cache_pages) return;   // never write outside the cache
+  uint8_t* dst = cache + pg * cache_stride_page + (int64_t)h * k_head_bytes(d_boost);
+
+  if (tid < kD) {
+    const bool boosted = s_idx[tid] < d_boost;
+    const float qmax = boosted ? 15.0f : 3.0f;
+    float scale = (ch_max - ch_min) / qmax;
+    scale = scale < 1e-6f ? 1e-6f : scale;
+    s_scale[tid] = scale;
+    s_min[tid] = ch_min;
+    s_qmax[tid] = qmax;
+    __half2 m2 = __halves2half2(__float2half_rn(scale), __float2half_rn(ch_min));
+    *(__half2*)(meta + pg * meta_stride_page + ((int64_t)h * kD + tid) * 4) = m2;
+  }
+  __syncthreads();
+
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    const int d = c8 * 8 + j;
+    const float scale = s_scale[d], mn = s_min[d], qmax = s_qmax[d];
+    uint32_t lo = 0, hi = 0;
+#pragma unroll
+    for (int r = 0; r < 8; ++r) {
+      const uint32_t w = ((const uint32_t*)&rows[r])[j >> 1];
+      const uint16_t bits = (j & 1) ? (uint16_t)(w >> 16) : (uint16_t)(w & 0xffffu);
+      const float xf = (h2f(bits) - mn) / scale;
+      const float q = fminf(fmaxf(floorf(xf + 0.5f), 0.0f), qmax);
+      const uint32_t code = (uint32_t)q;
+      lo |= (code & 3u) << (2 * r);
+      hi |= (code >> 2) << (2 * r);
+    }
+    s_lo[d * 16 + tg] = (uint16_t)lo;
+    const uint8_t slot = s_idx[d];
+    if (slot < d_boost) *(uint16_t*)(dst + kLoBytes + slot * kRowBytes + tg * 2) = (uint16_t)hi;
+  }
+  __syncthreads();
+  ((uint4*)dst)[tid] = ((const uint4*)s_lo)[tid];
+  if (tid < kD / 4) ((uint32_t*)(dst + kRowBytes * (kD + d_boost)))[tid] = ((const uint32_t*)s_idx)[tid];
+}
+
+// 256 threads: 8 consecutive lanes share a token (16 channels each), 4 tokens per thread.
+__global__ __launch_bounds__(256) void quant_pack_v_kernel(
+    const uint8_t* __restrict__ value, int64_t stride_b, int64_t stride_h, int64_t stride_t,
+    int t_offset,
+    const int64_t* __restrict__ page_table, int64_t pt_stride_b, int page_offset,
+    uint8_t* __restrict__ cache, int64_t cache_stride_page,
+    uint8_t* __restrict__ meta, int64_t meta_stride_page, int64_t cache_pages) {
+  const int p = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+  const int tid = threadIdx.x;
+  const int cg = tid & 7;
+  const int64_t pg = page_table[(int64_t)b * pt_stride_b + page_offset + p];
+  if (pg < 0 || pg >= cache_pages) return;
+  uint8_t* dst = cache + pg * cache_stride_page + (int64_t)h * kVBytes;
+  uint8_t* mdst = meta + pg * meta_stride_page + (int64_t)h * kPage * 4;
+  const uint8_t* src = value + (int64_t)b * stride_b + (int64_t)h * stride_h +
+                       (int64_t)(t_offset + p * kPage) * stride_t + cg * 32;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int t = (tid >> 3) + 32 * i;
+    const uint4 a = *(const uint4*)(src + (int64_t)t * stride_t);
+    const uint4 c = *(const uint4*)(src + (int64_t)t * stride_t + 16);
+    const uint32_t w[8] = {a.x, a.y, a.z, a.w, c.x, c.y, c.z, c.w};
+    float x[16];
+    float mn = INFINITY, mx = -INFINITY;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      x[2 * k] = h2f((uint16_t)(w[k] & 0xffffu));
+      x[2 * k + 1] = h2f((uint16_t)(w[k] >> 16));
+      mn = fminf(mn, fminf(x[2 * k], x[2 * k + 1]));
+      mx = fmaxf(mx, fmaxf(x[2 * k], x[2 * k + 1]));
+    }
+#pragma unroll
+    for (int o = 1; o < 8; o <<= 1) {
+      mn = fminf(mn, __shfl_xor(mn, o));
+      mx = fmaxf(mx, __shfl_xor(mx, o));
+    }
+    float scale = (mx - mn) / 3.0f;
+    scale = scale < 1e-6f ? 1e-6f : scale;
+    uint32_t packed = 0;
+#pragma unroll
+    for (int k = 0; k < 16; ++k) {
+      const float q = fminf(fmaxf(floorf((x[k] - mn) / scale + 0.5f), 0.0f), 3.0f);
+      packed |= (uint32_t)q << (2 * k);
+    }
+    *(uint32_t*)(dst + t * kRowBytes + cg * 4) = packed;
+    if (cg == 0) *(__half2*)(mdst + t * 4) = __halves2half2(__float2half_rn(scale), __float2half_rn(mn));
+  }
+}
+
+int check_src(const void* p, int64_t sb, int64_t sh, int64_t st, int B, int H, int T, int D, int t_offset,
+              int pages, int page_size) {
+  KITTY_REQUIRE(p != nullptr, KITTY_E_NULL, "source tensor is NULL");
+  KITTY_REQUIRE(D == kD && page_size == kPage, KITTY_E_SHAPE,
+                "kernels are built for head_dim 128 and page_size 128, got D=%d page_size=%d", D, page_size);
+  KITTY_REQUIRE(B >= 0 && H >= 1 && pages >= 0 && t_offset >= 0, KITTY_E_RANGE,
+                "bad B=%d H=%d pages=%d t_offset=%d", B, H, pages, t_offset);
+  KITTY_REQUIRE((int64_t)t_offset + (int64_t)pages * page_size <= (int64_t)T, KITTY_E_RANGE,
+                "pages [%d, %d) tokens exceed the source length %d", t_offset, t_offset + pages * page_size, T);
+  KITTY_REQUIRE(B <= 65535 && H <= 65535, KITTY_E_RANGE, "B and H must fit a grid dimension");
+  KITTY_REQUIRE(((uintptr_t)p % 16) == 0 && sb % 16 == 0 && sh % 16 == 0 && st % 16 == 0 && st >= D * 2,
+                KITTY_E_ALIGN, "source needs 16-byte aligned base and strides with D contiguous");
+  return 0;
+}
+
+int check_dst(const int64_t* page_table, int page_offset, const void* cache, int64_t cache_stride,
+              const void* meta, int64_t meta_stride, int64_t cache_pages, int64_t need_cache,
+              int64_t need_meta) {
+  KITTY_REQUIRE(page_table && cache && meta, KITTY_E_NULL, "page_table / cache / metadata is NULL");
+  KITTY_REQUIRE(page_offset >= 0 && cache_pages >= 0, KITTY_E_RANGE, "bad page_offset or cache_pages");
+  KITTY_REQUIRE(cache_stride >= need_cache && meta_stride >= need_meta, KITTY_E_RANGE,
+                "page stride too small: cache %lld < %lld or metadata %lld < %lld", (long long)cache_stride,
+                (long long)need_cache, (long long)meta_stride, (long long)need_meta);
+  KITTY_REQUIRE(((uintptr_t)cache % 16) == 0 && cache_stride % 16 == 0 && ((uintptr_t)meta % 4) == 0 &&
+                    meta_stride % 4 == 0,
+                KITTY_E_ALIGN, "cache needs 16-byte, metadata 4-byte alignment");
+  return 0;
+}
+
+}  // namespace
+
+extern "C" int kitty_select_boost_k(const void* key, int64_t stride_b, int64_t stride_h, int64_t stride_t,
+                                    int B, int H, int T, int D, int t_offset, int pages, int page_size, int d_boost,
+                                    uint8_t* slot_map, void* stream) {
+  if (int rc = check_src(key, stride_b, stride_h, stride_t, B, H, T, D, t_offset, pages, page_size)) return rc;
+  KITTY_REQUIRE(slot_map != nullptr, KITTY_E_NULL, "slot_map is NULL");
+  KITTY_REQUIRE(d_boost >= 0 && d_boost <= D, KITTY_E_SHAPE, "d_boost must be in [0, %d], got %d", D, d_boost);
+  if (B == 0 || pages == 0) return 0;
+  hipLaunchKernelGGL(quant_pack_k_kernel<2>, dim3(pages, H, B), dim3(256), 0, (hipStream_t)stream,
+                     (const uint8_t*)key, stride_b, stride_h, stride_t, t_offset, d_boost, nullptr, slot_map,
+                     pages, nullptr, 0, 0, nullptr, 0, nullptr, 0, 0);
+  return check_launch("kitty_select_boost_k");
+}
+
+extern "C" int kitty_quant_pack_k(const void* key, int64_t stride_b, int64_t stride_h, int64_t stride_t,
+                                  int B, int H, int T, int D, int t_offset, int pages, int page_size, int d_boost,
+                                  const uint8_t* slot_map,
+                                  const int64_t* page_table, int64_t page_table_stride_b, int page_offset,
+                                  uint8_t* cache, int64_t cache_stride_page,
+                                  void* meta, int64_t meta_stride_page, int64_t cache_pages, void* stream) {
+  if (int rc = check_src(key, stride_b, stride_h, stride_t, B, H, T, D, t_offset, pages, page_size)) return rc;
+  // the slot map is a uint8 with d_boost as the "not boosted" marker, and the high plane has
+  // d_boost rows: keep rows 4-byte friendly
+  KITTY_REQUIRE(d_boost >= 0 && d_boost <= D, KITTY_E_SHAPE, "d_boost must be in [0, %d], got %d", D, d_boost);
+  KITTY_REQUIRE((k_head_bytes(d_boost) % 16) == 0, KITTY_E_ALIGN,
+                "d_boost=%d gives a per-head page size that is not a multiple of 16 bytes", d_boost);
+  if (int rc = check_dst(page_table, page_offset, cache, cache_stride_page, meta, meta_stride_page, cache_pages,
+                         (int64_t)H * k_head_bytes(d_boost), (int64_t)H * kD * 4))
+    return rc;
+  if (B == 0 || pages == 0) return 0;
+  dim3 grid(pages, H, B), block(256);
+  if (slot_map)
+    hipLaunchKernelGGL(quant_pack_k_kernel<0>, grid, block, 0, (hipStream_t)stream, (const uint8_t*)key, stride_b,
+                       stride_h, stride_t, t_offset, d_boost, slot_map, nullptr, pages, page_table,
+                       page_table_stride_b, page_offset, cache, cache_stride_page, (uint8_t*)meta,
+                       meta_stride_page, cache_pages);
+  else
+    hipLaunchKernelGGL(quant_pack_k_kernel<1>, grid, block, 0, (hipStream_t)stream, (const uint8_t*)key, stride_b,
+                       stride_h, stride_t, t_offset, d_boost, nullptr, nullptr, pages, page_table,
+                       page_table_stride_b, page_offset, cache, cache_stride_page, (uint8_t*)meta,
+                       meta_stride_page, cache_pages);
+  return check_launch("kitty_quant_pack_k");
+}
+
+extern "C" int kitty_quant_pack_v(const void* value, int64_t stride_b, int64_t stride_h, int64_t stride_t,
+                                  int B, int H, int T, int D, int t_offset, int pages, int page_size,
+                                  const int64_t* page_table, int64_t page_table_stride_b, int page_offset,
+                                  uint8_t* cache, int64_t cache_stride_page,
+                                  void* meta, int64_t meta_stride_page, int64_t cache_pages, void* stream) {
+  if (int rc = check_src(value, stride_b, stride_h, stride_t, B, H, T, D, t_offset, pages, page_size)) return rc;
+  if (int rc = check_dst(page_table, page_offset, cache, cache_stride_page, meta, meta_stride_page, cache_pages,
+                         (int64_t)H * kVBytes, (int64_t)H * kPage * 4))
+    return rc;
+  if (B == 0 || pages == 0) return 0;
+  hipLaunchKernelGGL(quant_pack_v_kernel, dim3(pages, H, B), dim3(256), 0, (hipStream_t)stream,
+                     (const uint8_t*)value, stride_b, stride_h, stride_t, t_offset, page_table,
+                     page_table_stride_b, page_offset, cache, cache_stride_page, (uint8_t*)meta, meta_stride_page,
+                     cache_pages);
+  return check_launch("kitty_quant_pack_v");
+}

@@ -1,0 +1,155 @@
+"""``KittyCache``: the HF-Transformers cache plugin of the packed 2-bit KV cache.
+
+Same class name, constructor, methods and return conventions as the reference
+(src/kitty/kvcache/kitty.py:24-258): ``update()`` returns ``True`` in prefill and ``False`` in
+decode, the caller runs attention and then calls ``quantize_prefill`` / ``quantize_decode``
+(call order fixed by src/kitty/models/qwen3/modeling_qwen3.py:225-251).
+"""
+from typing import Any, Optional
+
+import torch
+
+try:  # the plugin subclasses HF's Cache when transformers is importable
+    from transformers.cache_utils import Cache as _HFCache
+except Exception:  # pragma: no cover - transformers is optional for the kernels themselves
+    _HFCache = object
+
+from .kernels.kitty_quant_pack import quantize_pack_k, quantize_pack_v
+from .utils_kv_per_layer import KVCache_Layer
+
+
+class KittyCache(_HFCache):
+    """Kitty KV cache: fp16 sink + packed 2-bit pages (25 % of key channels at 4 bit) + fp16
+    residual windows that are flushed into packed pages when full."""
+    is_compileable = False
+
+    def __init__(self, config, max_batch_size: int, max_length: int, *, device="cuda",
+                 select: str = "hip") -> None:
+        if _HFCache is not object:
+            try:
+                super().__init__(layers=[])          # transformers >= 4.54
+            except TypeError:
+                super().__init__()                   # transformers 4.53 (the reference's pin)
+        self.kv_cache: list[KVCache_Layer] = []
+        self.num_hidden_layers = config.num_hidden_layers
+        self.head_dim = getattr(config, "head_dim", None) or config.hidden_size // config.num_attention_heads
+        self.num_key_value_heads = config.num_key_value_heads
+        # Kitty constants (kitty.py:43-47)
+        self.page_size = 128
+        self.d_boosted = self.head_dim // 4
+        self.sink_length = 32
+        self.low_bit = 2
+        self.high_bit = 4
+        self.select = select
+        for _ in range(self.num_hidden_layers):
+            self.kv_cache.append(KVCache_Layer(
+                MAX_BS=max_batch_size, MAX_LEN=max_length, H_KV=self.num_key_value_heads, D=self.head_dim,
+                D_BOOSTED=self.d_boosted, LOW_BIT=self.low_bit, HIGH_BIT=self.high_bit,
+                PAGE_SIZE=self.page_size, S=self.sink_length, device=device))
+
+    def update(self, key_states: torch.Tensor, value_states: torch.Tensor, layer_idx: int,
+               cache_kwargs: Optional[dict[str, Any]] = None) -> bool:
+        """Append to layer ``layer_idx``.  Returns True in prefill (the states are stashed for
+        ``quantize_prefill``), False in decode (one token written to the fp16 windows)."""
+        kvcache = self.kv_cache[layer_idx]
+        if kvcache.Sink_Count == 0:
+            kvcache.key_states = key_states
+            kvcache.value_states = value_states
+            return True
+        assert key_states.shape[-2] == 1 and value_states.shape[-2] == 1, \
+            "Decode: key_states and value_states should have sequence length of 1."
+        B = key_states.shape[0]
+        with torch.no_grad():
+            if kvcache.Sink_Count < kvcache.S:
+                idx = kvcache.Sink_Count
+                kvcache.Sink_Buffer_K[:B, :, idx, :] = key_states[:, :, 0, :]
+                kvcache.Sink_Buffer_V[:B, :, idx, :] = value_states[:, :, 0, :]
+                kvcache.Sink_Count += 1
+            else:
+                assert kvcache.Q_Buffer_Count_K < kvcache.Q_Buffer_K.size(2)
+                kvcache.Q_Buffer_K[:B, :, kvcache.Q_Buffer_Count_K, :] = key_states[:, :, 0, :]
+                kvcache.Q_Buffer_Count_K += 1
+                assert kvcache.Local_Count_V <= kvcache.PAGE_SIZE
+                if kvcache.Local_Count_V < kvcache.PAGE_SIZE:
+                    kvcache.Local_Buffer_V[:B, :, kvcache.Local_Count_V, :] = value_states[:, :, 0, :]
+                    kvcache.Local_Count_V += 1
+                else:   # ring full: the oldest row moves to the V Q-buffer, the new one takes its place
+                    assert kvcache.Q_Buffer_Count_V < kvcache.Q_Buffer_V.size(2)
+                    w = kvcache.Write_Offset_Local_V
+                    kvcache.Q_Buffer_V[:B, :, kvcache.Q_Buffer_Count_V, :] = kvcache.Local_Buffer_V[:B, :, w, :]
+                    kvcache.Q_Buffer_Count_V += 1
+                    kvcache.Local_Buffer_V[:B, :, w, :] = value_states[:, :, 0, :]
+                    kvcache.Write_Offset_Local_V = (w + 1) % kvcache.PAGE_SIZE
+        return False
+
+    def quantize_prefill(self, layer_idx: int = 0) -> None:
+        """Split the stashed prefill into sink / packed pages / fp16 residuals (kitty.py:126-192)."""
+        kvcache = self.kv_cache[layer_idx]
+        if kvcache.key_states is None or kvcache.value_states is None:
+            raise ValueError("No key_states or value_states to quantize. Please call update() first.")
+        K, V = kvcache.key_states, kvcache.value_states
+        B, P = K.shape[0], kvcache.PAGE_SIZE
+        len_prefill = K.shape[-2]
+        len_sink = min(kvcache.S, len_prefill)
+        # K: newest (T-S) % P tokens stay fp16 in the Q-buffer, whole pages in between are packed
+        len_qbuf_k = max(0, len_prefill - len_sink) % P
+        pages_k = (len_prefill - len_sink - len_qbuf_k) // P
+        if pages_k > kvcache.MAX_PAGE:
+            raise ValueError(f"prefill of {len_prefill} tokens exceeds max_length={kvcache.MAX_LEN}")
+        kvcache.Sink_Buffer_K[:B, :, :len_sink, :].copy_(K[:, :, :len_sink, :])
+        kvcache.Sink_Count = len_sink
+        if len_qbuf_k > 0:
+            kvcache.Q_Buffer_K[:B, :, :len_qbuf_k, :].copy_(K[:, :, len_prefill - len_qbuf_k:, :])
+            kvcache.Q_Buffer_Count_K = len_qbuf_k
+        if pages_k > 0:
+            quantize_pack_k(K, len_sink, pages_k, kvcache.PageTable_K, 0, kvcache.KeyCache,
+                            kvcache.KeyCache_metadata, P, kvcache.D_BOOSTED, select=self.select)
+            kvcache.PageCount_K += pages_k
+        # V: newest min(P, T-S) tokens -> local ring, the remainder before them -> Q-buffer, rest packed
+        len_local_v = max(0, min(P, len_prefill - len_sink))
+        len_qbuf_v = max(0, len_prefill - len_sink - len_local_v) % P
+        pages_v = (len_prefill - len_sink - len_local_v - len_qbuf_v) // P
+        kvcache.Sink_Buffer_V[:B, :, :len_sink, :].copy_(V[:, :, :len_sink, :])
+        if len_local_v > 0:
+            kvcache.Local_Buffer_V[:B, :, :len_local_v, :].copy_(V[:, :, len_prefill - len_local_v:, :])
+            kvcache.Local_Count_V = len_local_v
+        if len_qbuf_v > 0:
+            assert len_local_v > 0, "Local buffer must be filled before using Q-buffer."
+            lo = len_prefill - len_local_v - len_qbuf_v
+            kvcache.Q_Buffer_V[:B, :, :len_qbuf_v, :].copy_(V[:, :, lo: lo + len_qbuf_v, :])
+            kvcache.Q_Buffer_Count_V = len_qbuf_v
+        if pages_v > 0:
+            assert len_prefill - len_sink - len_local_v - len_qbuf_v == pages_v * P
+            quantize_pack_v(V, len_sink, pages_v, kvcache.PageTable_V, 0, kvcache.ValueCache,
+                            kvcache.ValueCache_metadata, P)
+            kvcache.PageCount_V += pages_v
+        kvcache.key_states = None
+        kvcache.value_states = None
+
+    def quantize_decode(self, layer_idx: int = 0) -> None:
+        """Flush a full Q-buffer into the next packed page; K and V fill up independently
+        (kitty.py:194-236)."""
+        kvcache = self.kv_cache[layer_idx]
+        if kvcache.Q_Buffer_Count_K == kvcache.PAGE_SIZE:
+            if kvcache.PageCount_K >= kvcache.MAX_PAGE:
+                raise ValueError(f"key cache is full (max_length={kvcache.MAX_LEN})")
+            quantize_pack_k(kvcache.Q_Buffer_K, 0, 1, kvcache.PageTable_K, kvcache.PageCount_K, kvcache.KeyCache,
+                            kvcache.KeyCache_metadata, kvcache.PAGE_SIZE, kvcache.D_BOOSTED, select=self.select)
+            kvcache.PageCount_K += 1
+            kvcache.Q_Buffer_Count_K = 0
+        if kvcache.Q_Buffer_Count_V == kvcache.PAGE_SIZE:
+            if kvcache.PageCount_V >= kvcache.MAX_PAGE:
+                raise ValueError(f"value cache is full (max_length={kvcache.MAX_LEN})")
+            quantize_pack_v(kvcache.Q_Buffer_V, 0, 1, kvcache.PageTable_V, kvcache.PageCount_V, kvcache.ValueCache,
+                            kvcache.ValueCache_metadata, kvcache.PAGE_SIZE)
+            kvcache.PageCount_V += 1
+            kvcache.Q_Buffer_Count_V = 0
+
+    def get_seq_length(self, layer_idx: int = 0) -> int:
+        """Number of cached tokens of a layer."""
+        return self.kv_cache[layer_idx].get_total_length()
+
+
+def get_kvcache_kitty(config, max_batch_size: int, max_length: int, **kwargs) -> KittyCache:
+    """Factory with the reference's signature (kitty.py:244-258)."""
+    return KittyCache(config=config, max_batch_size=max_batch_size, max_length=max_length, **kwargs)

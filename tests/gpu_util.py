@@ -1,0 +1,48 @@
+"""Helpers for the GPU parity tests: build the same cache state in the HIP-backed KittyCache and
+in the CPU oracle from the same seeded inputs."""
+import types
+
+import numpy as np
+import torch
+
+from oracle import kitty_oracle as O
+
+
+def cfg(H_KV, H_Q, layers=1, D=128):
+    return types.SimpleNamespace(num_hidden_layers=layers, head_dim=D, num_key_value_heads=H_KV,
+                                 num_attention_heads=H_Q, hidden_size=H_Q * D)
+
+
+def module(H_KV, H_Q):
+    return types.SimpleNamespace(num_attention_heads=H_Q, num_key_value_heads=H_KV)
+
+
+def to_dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def layer_bytes_equal(layer, ol: O.OracleLayer):
+    """Bit-exact comparison of every tensor of a layer with the oracle's; returns list of mismatches."""
+    bad = []
+
+    def cmp(name, t, a):
+        got = t.detach().cpu().numpy()
+        if got.dtype == np.float16:
+            got, a = got.view(np.uint16), a.view(np.uint16)
+        if not np.array_equal(got, a):
+            bad.append((name, int((got != a).sum())))
+
+    cmp("KeyCache", layer.KeyCache, ol.KeyCache)
+    cmp("KeyCache_metadata", layer.KeyCache_metadata, ol.KeyCache_metadata)
+    cmp("ValueCache", layer.ValueCache, ol.ValueCache)
+    cmp("ValueCache_metadata", layer.ValueCache_metadata, ol.ValueCache_metadata)
+    cmp("Sink_Buffer_K", layer.Sink_Buffer_K, ol.Sink_Buffer_K)
+    cmp("Sink_Buffer_V", layer.Sink_Buffer_V, ol.Sink_Buffer_V)
+    cmp("Q_Buffer_K", layer.Q_Buffer_K, ol.Q_Buffer_K)
+    cmp("Q_Buffer_V", layer.Q_Buffer_V, ol.Q_Buffer_V)
+    cmp("Local_Buffer_V", layer.Local_Buffer_V, ol.Local_Buffer_V)
+    for f in ("Sink_Count", "PageCount_K", "PageCount_V", "Q_Buffer_Count_K", "Q_Buffer_Count_V",
+              "Local_Count_V", "Write_Offset_Local_V"):
+        if getattr(layer, f) != getattr(ol, f):
+            bad.append((f, getattr(layer, f), getattr(ol, f)))
+    return bad

@@ -1,0 +1,356 @@
+"""GPU parity: the HIP path (through the Python plugin API, which calls the C ABI) against the CPU
+oracle on the same seeded inputs.  Packed bytes, slot maps and scales/zeros must be bit-exact;
+attention outputs within max-abs 2e-3 (fp16)."""
+import glob
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import kitty_oracle as O
+from tests.helpers import make_kv, make_q
+
+pytestmark = pytest.mark.gpu
+ATOL = 2e-3
+
+
+@pytest.fixture(scope="module")
+def K():
+    if not torch.cuda.is_available():
+        pytest.skip("needs a GPU")
+    import kitty_amd
+    from kitty_amd import _lib
+    _lib.lib()                                   # raises if the HIP library is not built
+    from kitty_amd.kvcache.kernels import kitty_attention_forward, quantize_pack_k, quantize_pack_v, select_boost_k
+    from tests import gpu_util
+    ns = dict(KittyCache=kitty_amd.KittyCache, attn=kitty_attention_forward, qk=quantize_pack_k,
+              qv=quantize_pack_v, sel=select_boost_k, u=gpu_util)
+    return type("NS", (), ns)
+
+
+def _np16(t):
+    return t.detach().cpu().numpy()
+
+
+# ---------------------------------------------------------------------------------------------
+# quantizer
+# ---------------------------------------------------------------------------------------------
+GOLDEN = sorted(glob.glob(os.path.join(os.path.dirname(__file__), "golden", "quant_*.npz")))
+
+
+@pytest.mark.parametrize("path", GOLDEN, ids=[os.path.basename(p) for p in GOLDEN])
+def test_quantizer_against_reference_golden(K, path):
+    """The HIP kernels on the golden inputs reproduce what the reference's kernels wrote."""
+    g = np.load(path)
+    x = K.u.to_dev(g["x"])
+    B, H, _, D = x.shape
+    P, t0, po = int(g["pages"]), int(g["t_offset"]), int(g["page_offset"])
+    pt = K.u.to_dev(g["page_table"])
+    lay = O.Layout(H_KV=H)
+    gk = g["key_cache"].reshape(-1, H, lay.k_stride_h)
+    sm = np.zeros((B, H, P, D), np.uint8)
+    for b in range(B):
+        for p in range(P):
+            sm[b, :, p] = gk[g["page_table"][b, po + p], :, lay.k_off_idx:]
+    kc = torch.zeros_like(K.u.to_dev(g["key_cache"]))
+    km = torch.zeros_like(K.u.to_dev(g["key_meta"]))
+    vc = torch.zeros_like(K.u.to_dev(g["value_cache"]))
+    vm = torch.zeros_like(K.u.to_dev(g["value_meta"]))
+    K.qk(x, t0, P, pt, po, kc, km, 128, 32, slot_map=K.u.to_dev(sm))
+    K.qv(x, t0, P, pt, po, vc, vm, 128)
+    torch.cuda.synchronize()
+    assert np.array_equal(_np16(vc), g["value_cache"])
+    assert np.array_equal(_np16(vm).view(np.uint16), g["value_meta"].view(np.uint16))
+    assert np.array_equal(_np16(km).view(np.uint16), g["key_meta"].view(np.uint16))
+    ok = _np16(kc).reshape(-1, H, lay.k_stride_h)
+    assert np.array_equal(ok[:, :, : lay.k_off_hi], gk[:, :, : lay.k_off_hi])
+    assert np.array_equal(ok[:, :, lay.k_off_idx:], gk[:, :, lay.k_off_idx:])
+    # whole pages (high plane included) against the oracle, which stores slot s in row s
+    okc, okm = np.zeros_like(g["key_cache"]), np.zeros_like(g["key_meta"])
+    O.quantize_pack_k(g["x"], t0, P, g["page_table"], po, okc, okm, 128, 32, slot_map=sm)
+    assert np.array_equal(_np16(kc), okc)
+    if "spread" in path:     # tie-free scores: the fused selection must give the reference's map
+        kc2, km2 = torch.zeros_like(kc), torch.zeros_like(km)
+        K.qk(x, t0, P, pt, po, kc2, km2, 128, 32)
+        torch.cuda.synchronize()
+        assert np.array_equal(_np16(kc2), okc)
+
+
+@pytest.mark.parametrize("student_t", [False, True])
+def test_quantize_pack_bit_exact_random(K, student_t):
+    B, H, P, t0 = 2, 3, 5, 32
+    T = t0 + P * 128 + 17
+    k, v = make_kv(B, H, T, seed=21 + student_t, student_t=student_t)
+    MAXP = 8
+    rng = np.random.default_rng(3)
+    pt = rng.permutation(B * MAXP).reshape(B, MAXP).astype(np.int64)
+    lay = O.Layout(H_KV=H)
+    okc = np.zeros((B * MAXP, lay.bytes_per_page_K), np.uint8)
+    okm = np.zeros((B * MAXP, H, 128, 2), np.float16)
+    ovc = np.zeros((B * MAXP, lay.bytes_per_page_V), np.uint8)
+    ovm = np.zeros((B * MAXP, H, 128, 2), np.float16)
+    used = O.quantize_pack_k(k, t0, P, pt, 2, okc, okm, 128, 32)
+    O.quantize_pack_v(v, t0, P, pt, 2, ovc, ovm, 128)
+    kc, km = K.u.to_dev(np.zeros_like(okc)), K.u.to_dev(np.zeros_like(okm))
+    vc, vm = K.u.to_dev(np.zeros_like(ovc)), K.u.to_dev(np.zeros_like(ovm))
+    kd, vd, ptd = K.u.to_dev(k), K.u.to_dev(v), K.u.to_dev(pt)
+    K.qk(kd, t0, P, ptd, 2, kc, km, 128, 32)            # fused selection (canonical tie rule)
+    K.qv(vd, t0, P, ptd, 2, vc, vm, 128)
+    sm = K.sel(kd, t0, P, 128, 32)
+    torch.cuda.synchronize()
+    assert np.array_equal(_np16(sm), used)
+    assert np.array_equal(_np16(kc), okc)
+    assert np.array_equal(_np16(km).view(np.uint16), okm.view(np.uint16))
+    assert np.array_equal(_np16(vc), ovc)
+    assert np.array_equal(_np16(vm).view(np.uint16), ovm.view(np.uint16))
+    # given-map mode with a map that is NOT the selection (random slots, fewer than 32 boosted)
+    sm2 = np.full((B, H, P, 128), 32, np.uint8)
+    for idx in np.ndindex(B, H, P):
+        ch = rng.permutation(128)[:20]
+        sm2[idx][ch] = rng.permutation(32)[:20]
+    okc2 = np.full_like(okc, 0x5A)
+    O.quantize_pack_k(k, t0, P, pt, 2, okc2, okm.copy(), 128, 32, slot_map=sm2)
+    kc2 = K.u.to_dev(np.full_like(okc, 0x5A))
+    K.qk(kd, t0, P, ptd, 2, kc2, km, 128, 32, slot_map=K.u.to_dev(sm2))
+    torch.cuda.synchronize()
+    assert np.array_equal(_np16(kc2), okc2)      # unmapped high-plane rows keep their old bytes
+
+
+def test_quantize_strided_source_no_copy(K):
+    """[B, T, H, D] projections transposed to [B, H, T, D] are read through their strides."""
+    B, H, T = 1, 2, 128 * 2
+    k, v = make_kv(B, H, T, seed=4)
+    kd = K.u.to_dev(k.transpose(0, 2, 1, 3)).transpose(1, 2)       # non-contiguous view
+    assert not kd.is_contiguous()
+    lay = O.Layout(H_KV=H)
+    pt = np.arange(2, dtype=np.int64).reshape(1, 2)
+    okc, okm = np.zeros((2, lay.bytes_per_page_K), np.uint8), np.zeros((2, H, 128, 2), np.float16)
+    O.quantize_pack_k(k, 0, 2, pt, 0, okc, okm, 128, 32)
+    kc, km = K.u.to_dev(np.zeros_like(okc)), K.u.to_dev(np.zeros_like(okm))
+    K.qk(kd, 0, 2, K.u.to_dev(pt), 0, kc, km, 128, 32)
+    torch.cuda.synchronize()
+    assert np.array_equal(_np16(kc), okc)
+
+
+def test_select_torch_mode_and_topk_agreement(K):
+    """select='torch' consumes torch.topk's map; where scores are tie-free it equals the fused one."""
+    B, H, P = 1, 4, 4
+    k, _ = make_kv(B, H, P * 128, seed=8)
+    kd = K.u.to_dev(k)
+    lay = O.Layout(H_KV=H)
+    pt = K.u.to_dev(np.arange(P, dtype=np.int64).reshape(1, P))
+    kc_t = torch.zeros((P, lay.bytes_per_page_K), dtype=torch.uint8, device="cuda")
+    kc_h = torch.zeros_like(kc_t)
+    km = torch.zeros((P, H, 128, 2), dtype=torch.float16, device="cuda")
+    K.qk(kd, 0, P, pt, 0, kc_t, km, 128, 32, select="torch")
+    K.qk(kd, 0, P, pt, 0, kc_h, km, 128, 32)
+    torch.cuda.synchronize()
+    a = _np16(kc_t).reshape(P, H, lay.k_stride_h)[:, :, lay.k_off_idx:]
+    b = _np16(kc_h).reshape(P, H, lay.k_stride_h)[:, :, lay.k_off_idx:]
+    same = tie_free = 0
+    for p in range(P):
+        for h in range(H):
+            xx = k[0, h, p * 128:(p + 1) * 128]
+            # the set of boosted channels may differ only among channels tied at the boundary score
+            sc = O.boost_score(xx).astype(np.float64)
+            assert np.array_equal(np.sort(sc[a[p, h] < 32]), np.sort(sc[b[p, h] < 32]))
+            if O.boost_is_tie_free(xx, 32):
+                tie_free += 1
+                assert np.array_equal(a[p, h], b[p, h])
+            same += np.array_equal(a[p, h], b[p, h])
+    print(f"torch.topk == canonical on {same}/{P * H} page-heads ({tie_free} tie-free)")
+
+
+def test_quantizer_rejects_bad_arguments(K):
+    x = torch.zeros(1, 1, 128, 128, dtype=torch.float16, device="cuda")
+    pt = torch.zeros(1, 1, dtype=torch.int64, device="cuda")
+    kc = torch.zeros(1, 5248, dtype=torch.uint8, device="cuda")
+    km = torch.zeros(1, 1, 128, 2, dtype=torch.float16, device="cuda")
+    with pytest.raises(ValueError):
+        K.qk(x, 64, 1, pt, 0, kc, km, 128, 32)                 # pages run past T
+    with pytest.raises(ValueError):
+        K.qk(x, 0, 1, pt, 0, kc, km, 64, 32)                   # unsupported page size
+    with pytest.raises(AssertionError):
+        K.qk(x, 0, 1, pt, 0, kc, km, 128, 200)                 # d_boost out of [0, D]
+    with pytest.raises(RuntimeError):
+        K.qk(x.cpu(), 0, 1, pt, 0, kc, km, 128, 32)            # no CPU path
+
+
+# ---------------------------------------------------------------------------------------------
+# cache plugin + decode attention
+# ---------------------------------------------------------------------------------------------
+def _build(K, B, H_KV, H_Q, T, max_len, seed, student_t=False):
+    k, v = make_kv(B, H_KV, T, seed=seed, student_t=student_t)
+    cache = K.KittyCache(K.u.cfg(H_KV, H_Q), B, max_len)
+    assert cache.update(K.u.to_dev(k), K.u.to_dev(v), 0) is True
+    cache.quantize_prefill(0)
+    ol = O.OracleLayer(B, max_len, H_KV)
+    assert ol.update(k, v) is True
+    ol.quantize_prefill()
+    return cache, ol
+
+
+def _attend_both(K, cache, ol, H_KV, H_Q, q, **kw):
+    out, w = K.attn(K.u.module(H_KV, H_Q), K.u.to_dev(q), cache.kv_cache[0], 128 ** -0.5, **kw)
+    assert w is None
+    torch.cuda.synchronize()
+    ref = O.decode_attention(ol, q, 128 ** -0.5)
+    return _np16(out).astype(np.float64), ref.astype(np.float64)
+
+
+@pytest.mark.parametrize("variant", [0, 1])
+def test_config0_roundtrip_and_decode(K, variant):
+    """BASELINE config 0: B=1, 8 KV / 32 Q heads, D=128, 4096 cached tokens."""
+    B, H_KV, H_Q, T = 1, 8, 32, 4096
+    cache, ol = _build(K, B, H_KV, H_Q, T, 4352, seed=1000)
+    L = cache.kv_cache[0]
+    assert (L.PageCount_K, L.PageCount_V, L.Q_Buffer_Count_K, L.Q_Buffer_Count_V, L.Local_Count_V) == (31, 30, 96, 96, 128)
+    assert K.u.layer_bytes_equal(L, ol) == []
+    assert cache.get_seq_length(0) == T
+    q = make_q(B, H_Q, seed=1000)
+    got, ref = _attend_both(K, cache, ol, H_KV, H_Q, q, variant=variant)
+    assert got.shape == (B, 1, H_Q, 128)
+    assert np.abs(got - ref).max() <= ATOL
+    exact = O.decode_attention(ol, q, 128 ** -0.5, reference_rounding=False)
+    assert np.abs(got - exact).max() <= ATOL
+
+
+@pytest.mark.parametrize("variant", [0, 1])
+@pytest.mark.parametrize("splits", [1, 3, 7, 64])
+def test_split_counts_agree(K, variant, splits):
+    B, H_KV, H_Q, T = 2, 2, 8, 32 + 128 * 9 + 50
+    cache, ol = _build(K, B, H_KV, H_Q, T, 2048, seed=5)
+    q = make_q(B, H_Q, seed=5)
+    got, ref = _attend_both(K, cache, ol, H_KV, H_Q, q, variant=variant, num_splits=splits)
+    assert np.abs(got - ref).max() <= ATOL
+
+
+@pytest.mark.parametrize("variant", [0, 1])
+@pytest.mark.parametrize("T", [1, 7, 32, 33, 100, 160, 161, 288, 289, 416])
+def test_short_and_boundary_prompts(K, variant, T):
+    """Prompts shorter than the sink, exactly the sink, first Q-buffer token, first page, ..."""
+    B, H_KV, H_Q = 2, 2, 4
+    cache, ol = _build(K, B, H_KV, H_Q, T, 1024, seed=100 + T)
+    assert K.u.layer_bytes_equal(cache.kv_cache[0], ol) == []
+    q = make_q(B, H_Q, seed=T)
+    got, ref = _attend_both(K, cache, ol, H_KV, H_Q, q, variant=variant)
+    assert np.abs(got - ref).max() <= ATOL
+
+
+@pytest.mark.parametrize("G", [1, 2, 4, 8, 16])
+def test_group_sizes(K, G):
+    B, H_KV, T = 1, 2, 32 + 128 * 3 + 5
+    H_Q = H_KV * G
+    cache, ol = _build(K, B, H_KV, H_Q, T, 1024, seed=40 + G)
+    q = make_q(B, H_Q, seed=G)
+    for variant in (0, 1):
+        got, ref = _attend_both(K, cache, ol, H_KV, H_Q, q, variant=variant)
+        assert np.abs(got - ref).max() <= ATOL
+
+
+def test_decode_steps_cross_flushes(K):
+    """Prefill, then 300 decode steps (update -> attend -> quantize_decode, the caller's order):
+    sink fill, ring wrap, K and V flushes at different steps.  State bit-exact at every step,
+    attention checked at the steps around each transition."""
+    B, H_KV, H_Q, T0 = 2, 2, 8, 20                      # prompt shorter than the sink
+    steps = 300
+    k, v = make_kv(B, H_KV, T0 + steps, seed=77)
+    cache = K.KittyCache(K.u.cfg(H_KV, H_Q), B, 1024)
+    ol = O.OracleLayer(B, 1024, H_KV)
+    kd, vd = K.u.to_dev(k), K.u.to_dev(v)
+    assert cache.update(kd[:, :, :T0], vd[:, :, :T0], 0) and ol.update(k[:, :, :T0], v[:, :, :T0])
+    cache.quantize_prefill(0)
+    ol.quantize_prefill()
+    mod = K.u.module(H_KV, H_Q)
+    checked = 0
+    for s in range(steps):
+        t = T0 + s
+        assert cache.update(kd[:, :, t:t + 1], vd[:, :, t:t + 1], 0) is False
+        assert ol.update(k[:, :, t:t + 1], v[:, :, t:t + 1]) is False
+        L = cache.kv_cache[0]
+        interesting = (ol.Q_Buffer_Count_K in (1, 127, 128) or ol.Q_Buffer_Count_V in (1, 127, 128)
+                       or ol.Sink_Count < 32 or s % 41 == 0 or ol.Local_Count_V in (127,))
+        if interesting:
+            q = make_q(B, H_Q, seed=s)
+            out, _ = K.attn(mod, K.u.to_dev(q), L, 128 ** -0.5)
+            ref = O.decode_attention(ol, q, 128 ** -0.5).astype(np.float64)
+            assert np.abs(_np16(out).astype(np.float64) - ref).max() <= ATOL, f"step {s}"
+            checked += 1
+        cache.quantize_decode(0)
+        ol.quantize_decode()
+        assert cache.get_seq_length(0) == t + 1
+    assert K.u.layer_bytes_equal(cache.kv_cache[0], ol) == []
+    assert checked > 20 and ol.PageCount_K == 2 and ol.PageCount_V == 1 and ol.Write_Offset_Local_V != 0
+
+
+def test_ragged_batch_per_sequence_counts(K):
+    """Per-sequence occupancy (BASELINE config 2, scaled down): every row of the batch has its own
+    page counts, residual fill and ring offset; the oracle attends each row with its own counts."""
+    B, H_KV, H_Q = 5, 2, 8
+    rng = np.random.default_rng(123)
+    max_len = 32 + 128 * 12
+    cache = K.KittyCache(K.u.cfg(H_KV, H_Q), B, max_len)
+    L = cache.kv_cache[0]
+    ols, counts = [], []
+    for b in range(B):
+        T = int(rng.integers(40, max_len - 130))
+        k, v = make_kv(1, H_KV, T + 150, seed=500 + b)
+        ol = O.OracleLayer(1, max_len, H_KV)
+        ol.update(k[:, :, :T], v[:, :, :T])
+        ol.quantize_prefill()
+        for s in range(int(rng.integers(0, 150))):           # some decode steps: ring offset != 0
+            ol.update(k[:, :, T + s:T + s + 1], v[:, :, T + s:T + s + 1])
+            ol.quantize_decode()
+        ols.append(ol)
+        # copy the oracle-built sequence into row b of the device cache (tests the kernel, not the quantizer)
+        for name in ("Sink_Buffer_K", "Sink_Buffer_V", "Q_Buffer_K", "Q_Buffer_V", "Local_Buffer_V"):
+            getattr(L, name)[b].copy_(K.u.to_dev(getattr(ol, name)[0]))
+        for name in ("KeyCache", "KeyCache_metadata", "ValueCache", "ValueCache_metadata"):
+            getattr(L, name)[b * L.MAX_PAGE:(b + 1) * L.MAX_PAGE].copy_(K.u.to_dev(getattr(ol, name)))
+        counts.append([ol.Sink_Count, ol.PageCount_K, ol.Q_Buffer_Count_K, ol.PageCount_V, ol.Q_Buffer_Count_V,
+                       ol.Local_Count_V, ol.Write_Offset_Local_V, 0])
+    L.seq_counts = torch.tensor(counts, dtype=torch.int32, device="cuda")
+    q = make_q(B, H_Q, seed=9)
+    for variant in (0, 1):
+        out, _ = K.attn(K.u.module(H_KV, H_Q), K.u.to_dev(q), L, 128 ** -0.5, variant=variant)
+        got = _np16(out).astype(np.float64)
+        for b in range(B):
+            ref = O.decode_attention(ols[b], q[b:b + 1], 128 ** -0.5).astype(np.float64)
+            assert np.abs(got[b] - ref[0]).max() <= ATOL, (variant, b)
+
+
+def test_all_equal_keys_give_mean_of_values(K):
+    """Closed form: identical keys -> uniform weights -> output = mean of the dequantized values."""
+    B, H_KV, H_Q, T = 1, 1, 4, 32 + 128 * 3
+    k, v = make_kv(B, H_KV, T, seed=31)
+    k[:] = k[:, :, :1, :]
+    cache = K.KittyCache(K.u.cfg(H_KV, H_Q), B, 1024)
+    cache.update(K.u.to_dev(k), K.u.to_dev(v), 0)
+    cache.quantize_prefill(0)
+    ol = O.OracleLayer(B, 1024, H_KV)
+    ol.update(k, v)
+    ol.quantize_prefill()
+    _, Vd = O.gather_dense_kv(ol, 0)
+    q = make_q(B, H_Q, seed=2)
+    for variant in (0, 1):
+        out, _ = K.attn(K.u.module(H_KV, H_Q), K.u.to_dev(q), cache.kv_cache[0], 128 ** -0.5, variant=variant)
+        got = _np16(out).astype(np.float64)[0, 0]
+        want = Vd[0].astype(np.float64).mean(axis=0)
+        assert np.abs(got - want[None, :]).max() <= ATOL
+
+
+def test_attention_rejects_bad_arguments(K):
+    cache = K.KittyCache(K.u.cfg(2, 8), 1, 512)
+    L = cache.kv_cache[0]
+    q = torch.zeros(1, 8, 1, 128, dtype=torch.float16, device="cuda")
+    with pytest.raises(AssertionError):
+        K.attn(K.u.module(2, 8), torch.zeros(1, 8, 2, 128, dtype=torch.float16, device="cuda"), L, 0.1)
+    with pytest.raises(AssertionError):
+        K.attn(K.u.module(1, 32), torch.zeros(1, 32, 1, 128, dtype=torch.float16, device="cuda"), L, 0.1)
+    L.Q_Buffer_Count_K = 5                                   # K and V lengths disagree
+    with pytest.raises(AssertionError):
+        K.attn(K.u.module(2, 8), q, L, 0.1)
+    L.Q_Buffer_Count_K = 0
+    with pytest.raises(ValueError):
+        cache.quantize_prefill(0)                            # update() was never called
