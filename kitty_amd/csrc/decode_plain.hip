@@ -1,6 +1,7 @@
 // Decode attention, plain variant: the reference's order of operations (dequantize a tile to fp16
-// with fp16 arithmetic, fp32 dot products, logits rounded to fp16) in one fused split-K pass on
-// the vector ALUs.  It is the readable baseline the matrix-core kernel is checked against on the
+// with fp16 arithmetic, fp32 dot products) in one fused split-K pass on the vector ALUs.  Logits
+// and probabilities stay fp32 (the reference rounds both to fp16, kitty_attention.py:169,473,
+// which costs it accuracy and nothing else).  It is the readable baseline the matrix-core kernel is checked against on the
 // GPU and it accepts every boost count; it is not the fast path.
 #include "decode_common.h"
 
@@ -11,12 +12,19 @@ namespace kitty {
 constexpr int kMaxGroup = 16;                        // kitty_attention.py:418
 constexpr int kMaxHeadBytes = kRowBytes * (kD + kD) + kD;   // d_boost up to D
 
-#pragma clang fp contract(off)
+// fp16(code) * scale + zero with BOTH operations rounded to fp16, as eager torch and the Triton
+// interpreter evaluate kitty_attention.py:162-165 and :317-320.  Written on _Float16 with
+// contraction switched off for this function: a fused multiply-add would round once and move
+// large-magnitude channels by up to an fp16 ulp.
 __device__ inline float dequant_ref(uint32_t code, __half scale, __half zero) {
-  // fp16(code) * scale + zero with both operations rounded to fp16 (kitty_attention.py:162-165)
-  return __half2float(__hadd(__hmul(__ushort2half_rn((unsigned short)code), scale), zero));
+#pragma clang fp contract(off)
+  const _Float16 s = static_cast<__half_raw>(scale).data;
+  const _Float16 z = static_cast<__half_raw>(zero).data;
+  const _Float16 c = (_Float16)(float)code;
+  const _Float16 prod = c * s;
+  const _Float16 r = prod + z;
+  return (float)r;
 }
-#pragma clang fp contract(fast)
 
 __global__ __launch_bounds__(256) void decode_plain_kernel(kitty_kv_layer L, const __half* __restrict__ q, int H_Q,
                                                            float scaling, float* __restrict__ ws_ml,
@@ -96,9 +104,8 @@ __global__ __launch_bounds__(256) void decode_plain_kernel(kitty_kv_layer L, con
     // ---- online softmax: one wave per query head ---------------------------------------------
     for (int g = wave; g < G; g += 4) {
       float v0 = -INFINITY, v1 = -INFINITY;
-      if (lane < ntok) v0 = __half2float(__float2half_rn((s_part[0][g][lane] + s_part[1][g][lane]) * scaling));
-      if (lane + 64 < ntok)
-        v1 = __half2float(__float2half_rn((s_part[0][g][lane + 64] + s_part[1][g][lane + 64]) * scaling));
+      if (lane < ntok) v0 = (s_part[0][g][lane] + s_part[1][g][lane]) * scaling;
+      if (lane + 64 < ntok) v1 = (s_part[0][g][lane + 64] + s_part[1][g][lane + 64]) * scaling;
       float mx = fmaxf(v0, v1);
 #pragma unroll
       for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o));

@@ -234,17 +234,36 @@ def k_codes_from_page(by: np.ndarray, lay: Layout) -> np.ndarray:
     return (lo | (hi << 2)).T.copy()
 
 
-def dequant_k_page(by: np.ndarray, meta: np.ndarray, lay: Layout) -> np.ndarray:
-    """fp16 [PAGE, D]: fp16(code) * scale + zero, each operation rounded to fp16."""
-    codes = k_codes_from_page(by, lay).astype(F16)
-    scale, zero = meta[:, 0][None, :], meta[:, 1][None, :]
-    return ((codes * scale).astype(F16) + zero).astype(F16)
+DEQUANT_MODES = ("two", "fma", "affine")
 
 
-def dequant_v_page(by: np.ndarray, meta: np.ndarray, lay: Layout) -> np.ndarray:
-    codes = unpack2(by.reshape(lay.PAGE_SIZE, lay.v_stride_t)).astype(F16)        # [PAGE, D]
-    scale, zero = meta[:, 0][:, None], meta[:, 1][:, None]
-    return ((codes * scale).astype(F16) + zero).astype(F16)
+def _dequant(codes: np.ndarray, scale: np.ndarray, zero: np.ndarray, mode: str) -> np.ndarray:
+    """``code * scale + zero`` on the stored fp16 scale / zero, in one of three roundings:
+
+    ``"two"``    product and sum each rounded to fp16 - how eager torch and the Triton interpreter
+                 evaluate kitty_attention.py:162-165 / :317-320 (the reference semantics; fp16 out);
+    ``"fma"``    rounded once - what a compiled kernel that contracts the expression produces (fp16);
+    ``"affine"`` not rounded at all - the value both of the above approximate (float64 out).
+    """
+    c64, s64, z64 = codes.astype(np.float64), scale.astype(np.float64), zero.astype(np.float64)
+    if mode == "two":
+        return ((codes.astype(F16) * scale).astype(F16) + zero).astype(F16)
+    if mode == "fma":
+        return (c64 * s64 + z64).astype(F16)          # exact in float64, then one rounding
+    if mode == "affine":
+        return c64 * s64 + z64
+    raise ValueError(mode)
+
+
+def dequant_k_page(by: np.ndarray, meta: np.ndarray, lay: Layout, mode: str = "two") -> np.ndarray:
+    """[PAGE, D] dequantized keys of one page-head (see ``_dequant`` for ``mode``)."""
+    codes = k_codes_from_page(by, lay)
+    return _dequant(codes, meta[:, 0][None, :], meta[:, 1][None, :], mode)
+
+
+def dequant_v_page(by: np.ndarray, meta: np.ndarray, lay: Layout, mode: str = "two") -> np.ndarray:
+    codes = unpack2(by.reshape(lay.PAGE_SIZE, lay.v_stride_t))                    # [PAGE, D]
+    return _dequant(codes, meta[:, 0][:, None], meta[:, 1][:, None], mode)
 
 
 # ----------------------------------------------------------------------------------------------
@@ -378,8 +397,9 @@ class OracleLayer:
 # ----------------------------------------------------------------------------------------------
 # decode attention (kitty_attention.py:403-526; qk_kernel :16-207; softmax :473; sv_kernel :210-399)
 # ----------------------------------------------------------------------------------------------
-def gather_dense_kv(layer: OracleLayer, b: int, counts: Optional[dict] = None):
-    """fp16 K̂ [H_KV, T, D] and V̂ [H_KV, T, D] of sequence ``b`` in chronological order:
+def gather_dense_kv(layer: OracleLayer, b: int, counts: Optional[dict] = None, dequant: str = "two"):
+    """K̂ [H_KV, T, D] and V̂ [H_KV, T, D] of sequence ``b`` in chronological order (fp16, or
+    float64 for ``dequant="affine"``):
     K = [sink | pages | Q-buffer], V = [sink | pages | Q-buffer | local ring in age order].
     ``counts`` overrides the layer-wide counters (ragged batches: per-sequence occupancy)."""
     c = dict(sink=layer.Sink_Count, pk=layer.PageCount_K, rk=layer.Q_Buffer_Count_K,
@@ -395,19 +415,20 @@ def gather_dense_kv(layer: OracleLayer, b: int, counts: Optional[dict] = None):
             pg = int(layer.PageTable_K[b, p])
             o = h * lay.k_stride_h
             kparts.append(dequant_k_page(layer.KeyCache[pg, o: o + lay.k_stride_h],
-                                         layer.KeyCache_metadata[pg, h], lay))
+                                         layer.KeyCache_metadata[pg, h], lay, dequant))
         kparts.append(layer.Q_Buffer_K[b, h, : c["rk"]])
         vparts = [layer.Sink_Buffer_V[b, h, : c["sink"]]]
         for p in range(c["pv"]):
             pg = int(layer.PageTable_V[b, p])
             o = h * lay.v_stride_h
             vparts.append(dequant_v_page(layer.ValueCache[pg, o: o + lay.v_stride_h],
-                                         layer.ValueCache_metadata[pg, h], lay))
+                                         layer.ValueCache_metadata[pg, h], lay, dequant))
         vparts.append(layer.Q_Buffer_V[b, h, : c["rv"]])
         ring = (np.arange(c["lv"]) + c["off"]) % P
         vparts.append(layer.Local_Buffer_V[b, h, ring])
-        Ks.append(np.concatenate(kparts, axis=0))
-        Vs.append(np.concatenate(vparts, axis=0))
+        dt = np.float64 if dequant == "affine" else F16
+        Ks.append(np.concatenate([p_.astype(dt) for p_ in kparts], axis=0))
+        Vs.append(np.concatenate([p_.astype(dt) for p_ in vparts], axis=0))
     return np.stack(Ks), np.stack(Vs)
 
 
@@ -440,8 +461,14 @@ def attend_dense(q: np.ndarray, K: np.ndarray, V: np.ndarray, scaling: float,
 
 
 def decode_attention(layer: OracleLayer, query: np.ndarray, scaling: float,
-                     seq_counts: Optional[list] = None, reference_rounding: bool = True) -> np.ndarray:
+                     seq_counts: Optional[list] = None, reference_rounding: bool = True,
+                     dequant: str = "two") -> np.ndarray:
     """query fp16 [B, H_Q, 1, D] -> [B, 1, H_Q, D] (fp16, or float64 without reference rounding).
+
+    ``dequant`` picks how the packed pages are turned into numbers (``_dequant``);
+    ``reference_rounding`` additionally applies the reference's fp16 roundings of logits,
+    probabilities and output.  ``reference_rounding=False`` is plain dequantize-then-attend in
+    float64.
 
     Uses the runtime ``Sink_Count`` for the probability offsets on the V side as well (the
     reference's sv_kernel uses the constant S there, kitty_attention.py:327,343,368, which only
@@ -450,8 +477,10 @@ def decode_attention(layer: OracleLayer, query: np.ndarray, scaling: float,
     assert tq == 1
     outs = []
     for b in range(B):
-        K, V = gather_dense_kv(layer, b, None if seq_counts is None else seq_counts[b])
+        K, V = gather_dense_kv(layer, b, None if seq_counts is None else seq_counts[b], dequant)
         assert K.shape[1] == V.shape[1]
+        if reference_rounding:
+            K, V = K.astype(F16), V.astype(F16)
         outs.append(attend_dense(query[b, :, 0, :], K, V, scaling, reference_rounding))
     return np.stack(outs)[:, None, :, :]
 
