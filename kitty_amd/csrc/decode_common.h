@@ -13,6 +13,8 @@
 
 namespace kitty {
 
+__host__ __device__ inline int c_div_up(int a, int b) { return (a + b - 1) / b; }
+
 struct SeqCounts {
   int sink, pk, rk, pv, rv, lv, off;
   int nbody;    // tokens after the sink

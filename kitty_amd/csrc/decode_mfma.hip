@@ -1,7 +1,477 @@
-// Decode attention, matrix-core variant (placeholder until the kernel lands).
+// Decode attention over packed KV on the gfx950 matrix cores: the split pass of split-K.
+//
+// One wavefront (64 lanes) per workgroup walks a range of 128-token tiles of one (batch row,
+// kv head) and leaves an un-normalised partial (running max, running sum, output) per query head.
+//
+// Formulation.  With lane = 16*kg + n, v_mfma_f32_16x16x32_f16 takes A[row n][k 8kg..8kg+7],
+// B[k 8kg..8kg+7][col n] and returns C[rows 4kg..4kg+3][col n].  Both products are computed
+// transposed so that the accumulator of the first is, lane for lane, the B operand of the second:
+//
+//   S^T[token][col] = sum_ch  code[token][ch]            * (q[col][ch] * scale_k[ch])     (QK)
+//   O^T[ch][col]    = sum_tok code[tok][ch]               * (p[tok][col] * scale_v[tok])   (PV)
+//
+// The 16 columns hold the G query heads of the kv head (col n -> head n % G, replicated).  The
+// zero points never touch the codes: sum_ch q*zero_k is one dot product per page and column,
+// sum_tok p*zero_v one scalar per column, both on the vector ALU.
+//
+// Codes as operands.  A 32-bit word of a packed plane holds 16 two-bit codes of ONE row (K: one
+// channel, 16 tokens; V: one token, 16 channels) but an MFMA register must hold two consecutive k
+// (K: two channels, V: two tokens) of one row of A.  Lanes n and n^1 each load one word of two
+// neighbouring plane rows, swap them with one DPP move and v_perm the matching 16-bit halves
+// together: X = [8 codes of row r | 8 codes of row r+1].  `X & (3 << 2u | 3 << 2u+16)` is then
+// already a valid operand: fp16 SUBNORMALS code * 4^u * 2^-24 (the matrix cores do not flush
+// them), so unpacking costs one v_and_b32 per register and the factor is undone per tile after
+// the contraction.  Codes above bit 9 are reached through X >> 10.
+//
+// Index maps (all bijections chosen so that every load is 64 contiguous bytes per 16 lanes):
+//   K plane word of lane (kg, n) in 256-byte chunk c (= 8 plane rows):   row 2kg + (n&1), word n>>1
+//     -> channel 8c + 2kg + (n&1), tokens 16(n>>1) .. +15; lane n keeps tokens 8n .. 8n+7
+//     -> MFMA tile u (0..7) = tokens {8n + u}; k-slot (kg, 2pi + h) of chunk kc = channel
+//        32kc + 8pi + 2kg + h.
+//   C[u][j] of lane (kg, n) = token 32kg + 8j + u, column n.
+//   V plane rows are tokens: lane group kg owns rows 32kg .. 32kg+31 (its own tokens), k-chunk j
+//   = rows 32kg + 8j .. +7, d-tile u = channels {8n + u}; O^T[u][j] = channel 32kg + 8j + u.
 #include "decode_common.h"
 
 namespace kitty {
-bool decode_mfma_supported(const kitty_kv_layer&, int) { return false; }
-void launch_decode_mfma(const kitty_kv_layer&, const void*, int, int, float, float*, float*, int, hipStream_t) {}
+namespace {
+
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+typedef float float4v __attribute__((ext_vector_type(4)));
+typedef uint32_t uint4v __attribute__((ext_vector_type(4)));
+
+constexpr float kLog2e = 1.44269504088896340736f;
+constexpr int kQPad = 136;   // q_nat row length in halves: 128 channels + a zero entry at 128
+
+struct WaveLds {
+  _Float16 q_nat[16][kQPad];          // [column][channel]; [..][128] = 0 (the "no channel" slot)
+  uint32_t ks_perm[64], kz_perm[64];  // K scale / zero pairs in operand order (see stage_k_meta)
+  _Float16 ks4_nat[kQPad];            // 4 * K scale by channel; [128] = 0
+  uint32_t vs_nat[64], vz_nat[64];    // V scale / zero pairs by token pair
+  uint8_t inv[32];                    // high-plane slot -> channel (128 = slot unused)
+};
+
+__device__ __forceinline__ float4v mfma16(const uint32_t (&a)[4], const uint32_t (&b)[4], float4v c) {
+  const uint4v av = {a[0], a[1], a[2], a[3]}, bv = {b[0], b[1], b[2], b[3]};
+  return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, av), __builtin_bit_cast(half8, bv), c, 0,
+                                                0, 0);
+}
+__device__ __forceinline__ half2v as_h2(uint32_t u) { return __builtin_bit_cast(half2v, u); }
+__device__ __forceinline__ uint32_t as_u32(half2v h) { return __builtin_bit_cast(uint32_t, h); }
+__device__ __forceinline__ uint32_t swap_pair(uint32_t v) {   // value of lane n^1
+  return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0xB1 /* quad_perm [1,0,3,2] */, 0xf, 0xf, false);
+}
+__device__ __forceinline__ float xor_lanes(float v, int mask) { return __shfl_xor(v, mask); }
+
+// Mask of tile / d-tile u inside X (u < 5) or X >> 10 (u >= 5), and the factor that undoes the
+// subnormal encoding code * 4^u' * 2^-24.
+__device__ __forceinline__ constexpr uint32_t code_mask(int u) { return 0x00030003u << (2 * (u < 5 ? u : u - 5)); }
+__device__ __forceinline__ constexpr float code_unscale(int u) {
+  return 16777216.0f / (float)(1 << (2 * (u < 5 ? u : u - 5)));
+}
+
+struct Acc {
+  float4v out[8];     // O^T accumulators, d-tile u: channel 32kg + 8j + u, column n
+  float m;            // running max of the column's logits, log2 units
+  float l, z;         // lane-local sums over this lane's tokens of p and p * zero_v
+  bool first;         // nothing accumulated yet
+  bool true_units;    // out[] already multiplied by code_unscale (fp16-V tiles accumulate directly)
+};
+
+struct Ctx {
+  const kitty_kv_layer* L;
+  SeqCounts c;
+  int b, h, lane, kg, n;
+  uint32_t lane_off;    // byte offset of this lane's word inside a 256-byte plane chunk
+  uint32_t sel;         // v_perm selector merging own / partner halves
+  float sc2;            // scaling * log2(e)
+  uint32_t qpair[16];   // q[col][32kc + 8pi + 2kg + {0,1}] as an fp16 pair, index 4kc + pi
+};
+
+// ---------------------------------------------------------------------------------------------
+// K side
+// ---------------------------------------------------------------------------------------------
+// Stage one K page-head's (scale, zero) pairs and slot map in LDS in the order the operands need:
+// channel pair (2l, 2l+1) of lane l belongs to chunk kc = l/16, pair pi = (l/4)%4, lane group
+// l%4 and is stored at word 16kc + 4kg + pi, so that a lane reads the four pairs of a chunk with
+// one 128-bit LDS read.
+template <bool BOOST>
+__device__ __forceinline__ void stage_k_meta(WaveLds& S, const Ctx& x, const uint8_t* page, const uint8_t* meta) {
+  const int l = x.lane;
+  const uint2 km = *(const uint2*)(meta + l * 8);                       // [s0|z0], [s1|z1]
+  const uint32_t ss = __builtin_amdgcn_perm(km.y, km.x, 0x05040100u);   // (s0, s1)
+  const uint32_t zz = __builtin_amdgcn_perm(km.y, km.x, 0x07060302u);   // (z0, z1)
+  const int pos = (l >> 4) * 16 + (l & 3) * 4 + ((l >> 2) & 3);
+  S.ks_perm[pos] = ss;
+  S.kz_perm[pos] = zz;
+  if (BOOST) {
+    const half2v four = {(_Float16)4.0f, (_Float16)4.0f};
+    ((uint32_t*)S.ks4_nat)[l] = as_u32(as_h2(ss) * four);
+    if (l < 8) ((uint32_t*)S.inv)[l] = 0x80808080u;
+    __syncthreads();
+    const uint32_t ib = *(const uint16_t*)(page + kRowBytes * (kD + 32) + 2 * l);
+    const uint32_t i0 = ib & 0xffu, i1 = ib >> 8;
+    if (i0 < 32) S.inv[i0] = (uint8_t)(2 * l);
+    if (i1 < 32) S.inv[i1] = (uint8_t)(2 * l + 1);
+  }
+  __syncthreads();
+}
+
+// logits of one packed K page: C[u][j] = sum_ch code * q * scale (subnormal-scaled), cz = q . zero
+template <bool BOOST>
+__device__ __forceinline__ void qk_packed(WaveLds& S, const Ctx& x, int page_index, float4v (&C)[8], float& cz) {
+  const kitty_kv_layer& L = *x.L;
+  const int64_t pg = L.page_table_k[(int64_t)x.b * L.page_table_k_stride_b + page_index];
+  const uint8_t* page = L.key_cache + pg * L.key_cache_stride_page + (int64_t)x.h * k_head_bytes(BOOST ? 32 : 0);
+  const uint8_t* meta = (const uint8_t*)L.key_meta + pg * L.key_meta_stride_page + (int64_t)x.h * kD * 4;
+  uint32_t klo[16], khi[4];
+#pragma unroll
+  for (int c = 0; c < 16; ++c) klo[c] = *(const uint32_t*)(page + c * 256 + x.lane_off);
+  if (BOOST) {
+#pragma unroll
+    for (int c = 0; c < 4; ++c) khi[c] = *(const uint32_t*)(page + kLoBytes + c * 256 + x.lane_off);
+  }
+  stage_k_meta<BOOST>(S, x, page, meta);
+
+  float czl = 0.f;
+#pragma unroll
+  for (int u = 0; u < 8; ++u) C[u] = float4v{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int kc = 0; kc < 4; ++kc) {
+    const uint4v sp = *(const uint4v*)&S.ks_perm[kc * 16 + x.kg * 4];
+    const uint4v zp = *(const uint4v*)&S.kz_perm[kc * 16 + x.kg * 4];
+    uint32_t bh[4], bl[4], X[4], Y[4];
+#pragma unroll
+    for (int pi = 0; pi < 4; ++pi) {
+      const half2v qq = as_h2(x.qpair[kc * 4 + pi]), s2 = as_h2(sp[pi]);
+      const half2v hi = qq * s2;                                   // q*scale rounded to fp16 ...
+      const half2v lo = __builtin_elementwise_fma(qq, s2, -hi);    // ... and its exact remainder
+      bh[pi] = as_u32(hi);
+      bl[pi] = as_u32(lo);
+      czl = __builtin_amdgcn_fdot2(qq, as_h2(zp[pi]), czl, false);
+      const uint32_t own = klo[kc * 4 + pi];
+      X[pi] = __builtin_amdgcn_perm(swap_pair(own), own, x.sel);
+      Y[pi] = X[pi] >> 10;
+    }
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      uint32_t a[4];
+#pragma unroll
+      for (int pi = 0; pi < 4; ++pi) a[pi] = (u < 5 ? X[pi] : Y[pi]) & code_mask(u);
+      C[u] = mfma16(a, bh, C[u]);
+      C[u] = mfma16(a, bl, C[u]);
+    }
+  }
+  if (BOOST) {
+    // fifth chunk: the 32 high-plane slots; slot 8pi + 2kg + h carries bits 3:2 of the channel
+    // inv[slot], weight 4 * scale
+    uint32_t bh[4], bl[4], X[4], Y[4];
+#pragma unroll
+    for (int pi = 0; pi < 4; ++pi) {
+      const uint32_t cc = *(const uint16_t*)&S.inv[8 * pi + 2 * x.kg];
+      const uint32_t c0 = cc & 0xffu, c1 = cc >> 8;
+      const half2v qq = {S.q_nat[x.n][c0], S.q_nat[x.n][c1]};
+      const half2v s2 = {S.ks4_nat[c0], S.ks4_nat[c1]};
+      const half2v hi = qq * s2;
+      const half2v lo = __builtin_elementwise_fma(qq, s2, -hi);
+      bh[pi] = as_u32(hi);
+      bl[pi] = as_u32(lo);
+      const uint32_t own = khi[pi];
+      X[pi] = __builtin_amdgcn_perm(swap_pair(own), own, x.sel);
+      Y[pi] = X[pi] >> 10;
+    }
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      uint32_t a[4];
+#pragma unroll
+      for (int pi = 0; pi < 4; ++pi) a[pi] = (u < 5 ? X[pi] : Y[pi]) & code_mask(u);
+      C[u] = mfma16(a, bh, C[u]);
+      C[u] = mfma16(a, bl, C[u]);
+    }
+  }
+  czl += xor_lanes(czl, 16);
+  czl += xor_lanes(czl, 32);
+  cz = czl;
+#pragma unroll
+  for (int u = 0; u < 8; ++u) C[u] *= code_unscale(u);
+}
+
+// logits of up to 128 fp16 rows (sink or K Q-buffer): A = the rows themselves, B = q
+__device__ __forceinline__ void qk_fp16(const Ctx& x, const uint8_t* rows, int nrows_alloc, float4v (&C)[8]) {
+#pragma unroll
+  for (int u = 0; u < 8; ++u) {
+    C[u] = float4v{0.f, 0.f, 0.f, 0.f};
+    const int row = min(8 * x.n + u, nrows_alloc - 1);     // A row of this lane; clamped rows are masked later
+    const uint8_t* rp = rows + (int64_t)row * (kD * 2) + 4 * x.kg;
+#pragma unroll
+    for (int kc = 0; kc < 4; ++kc) {
+      uint32_t a[4], bq[4];
+#pragma unroll
+      for (int pi = 0; pi < 4; ++pi) {
+        a[pi] = *(const uint32_t*)(rp + (32 * kc + 8 * pi) * 2);   // channels 32kc + 8pi + 2kg + {0,1}
+        bq[pi] = x.qpair[kc * 4 + pi];
+      }
+      C[u] = mfma16(a, bq, C[u]);
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// softmax bookkeeping: C holds logits * (1/sc2) on entry, probabilities on exit
+// ---------------------------------------------------------------------------------------------
+__device__ __forceinline__ void softmax_tile(const Ctx& x, Acc& A, float4v (&C)[8], float cz, int ntok) {
+  const float cst = cz * x.sc2 - A.m;
+  float mt = -INFINITY;
+#pragma unroll
+  for (int u = 0; u < 8; ++u)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      float v = C[u][j] * x.sc2 + cst;                       // log2-logit relative to the running max
+      if (ntok < kPage && 32 * x.kg + 8 * j + u >= ntok) v = -INFINITY;
+      C[u][j] = v;
+      mt = fmaxf(mt, v);
+    }
+  mt = fmaxf(mt, xor_lanes(mt, 16));
+  mt = fmaxf(mt, xor_lanes(mt, 32));
+  if (__any(A.first || mt > 0.f)) {
+    // the column's max moves: shift this tile's logits and rescale what is accumulated
+    const float dm = A.first ? mt : fmaxf(mt, 0.f);
+#pragma unroll
+    for (int u = 0; u < 8; ++u)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) C[u][j] -= dm;
+    if (!A.first) {
+      const float alpha = __builtin_amdgcn_exp2f(-dm);
+      A.l *= alpha;
+      A.z *= alpha;
+#pragma unroll
+      for (int u = 0; u < 8; ++u) A.out[u] *= alpha;
+    }
+    A.m += dm;
+    A.first = false;
+  }
+#pragma unroll
+  for (int u = 0; u < 8; ++u)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) C[u][j] = __builtin_amdgcn_exp2f(C[u][j]);
+}
+
+// ---------------------------------------------------------------------------------------------
+// V side
+// ---------------------------------------------------------------------------------------------
+__device__ __forceinline__ void pv_packed(WaveLds& S, const Ctx& x, Acc& A, int page_index, const float4v (&P)[8]) {
+  const kitty_kv_layer& L = *x.L;
+  const int64_t pg = L.page_table_v[(int64_t)x.b * L.page_table_v_stride_b + page_index];
+  const uint8_t* page = L.value_cache + pg * L.value_cache_stride_page + (int64_t)x.h * kVBytes;
+  const uint8_t* meta = (const uint8_t*)L.value_meta + pg * L.value_meta_stride_page + (int64_t)x.h * kPage * 4;
+  uint32_t vw[16];
+  const uint32_t v_off = (32 * x.kg + (x.n & 1)) * kRowBytes + (x.n >> 1) * 4;
+#pragma unroll
+  for (int c = 0; c < 16; ++c) vw[c] = *(const uint32_t*)(page + v_off + c * 64);   // rows 32kg + 2c + (n&1)
+  {
+    const uint2 vm = *(const uint2*)(meta + x.lane * 8);                  // tokens 2l, 2l+1
+    __syncthreads();
+    S.vs_nat[x.lane] = __builtin_amdgcn_perm(vm.y, vm.x, 0x05040100u);
+    S.vz_nat[x.lane] = __builtin_amdgcn_perm(vm.y, vm.x, 0x07060302u);
+    __syncthreads();
+  }
+  const half2v ones = {(_Float16)1.0f, (_Float16)1.0f};
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const uint4v sp = *(const uint4v*)&S.vs_nat[16 * x.kg + 4 * j];
+    const uint4v zp = *(const uint4v*)&S.vz_nat[16 * x.kg + 4 * j];
+    uint32_t bp[4], X[4], Y[4];
+#pragma unroll
+    for (int pi = 0; pi < 4; ++pi) {
+      const half2v p2 = {(_Float16)P[2 * pi][j], (_Float16)P[2 * pi + 1][j]};   // tokens 32kg + 8j + 2pi + {0,1}
+      A.l = __builtin_amdgcn_fdot2(p2, ones, A.l, false);
+      A.z = __builtin_amdgcn_fdot2(p2, as_h2(zp[pi]), A.z, false);
+      bp[pi] = as_u32(p2 * as_h2(sp[pi]));
+      const uint32_t own = vw[4 * j + pi];
+      X[pi] = __builtin_amdgcn_perm(swap_pair(own), own, x.sel);
+      Y[pi] = X[pi] >> 10;
+    }
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      uint32_t a[4];
+#pragma unroll
+      for (int pi = 0; pi < 4; ++pi) a[pi] = (u < 5 ? X[pi] : Y[pi]) & code_mask(u);
+      A.out[u] = mfma16(a, bp, A.out[u]);
+    }
+  }
+}
+
+// fp16 V rows (sink, V Q-buffer, local ring): A gathered column-wise, accumulators in true units
+template <bool SINK>
+__device__ __forceinline__ void pv_fp16(const Ctx& x, Acc& A, int tail_first_row, int ntok, const float4v (&P)[8]) {
+  const kitty_kv_layer& L = *x.L;
+  const half2v ones = {(_Float16)1.0f, (_Float16)1.0f};
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    uint32_t bp[4];
+    const __half* rp[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      // rows past the tile's end carry p = 0; read a valid row instead so that 0 * value stays 0
+      const int t = min(32 * x.kg + 8 * j + i, ntok - 1);
+      if (SINK)
+        rp[i] = (const __half*)((const uint8_t*)L.sink_v + (int64_t)x.b * L.sink_stride_b +
+                                (int64_t)x.h * L.sink_stride_h) + (int64_t)t * kD;
+      else
+        rp[i] = v_tail_row(L, x.c, x.b, x.h, tail_first_row + t);
+    }
+#pragma unroll
+    for (int pi = 0; pi < 4; ++pi) {
+      const half2v p2 = {(_Float16)P[2 * pi][j], (_Float16)P[2 * pi + 1][j]};
+      A.l = __builtin_amdgcn_fdot2(p2, ones, A.l, false);
+      bp[pi] = as_u32(p2);
+    }
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      uint32_t a[4];
+#pragma unroll
+      for (int pi = 0; pi < 4; ++pi) {
+        const uint32_t lo = __half_as_ushort(rp[2 * pi][8 * x.n + u]);
+        const uint32_t hi = __half_as_ushort(rp[2 * pi + 1][8 * x.n + u]);
+        a[pi] = lo | (hi << 16);
+      }
+      A.out[u] = mfma16(a, bp, A.out[u]);
+    }
+  }
+}
+
+__device__ __forceinline__ void to_true_units(Acc& A) {
+  if (!A.true_units) {
+#pragma unroll
+    for (int u = 0; u < 8; ++u) A.out[u] *= code_unscale(u);
+    A.true_units = true;
+  }
+}
+
+template <bool BOOST>
+__global__ __launch_bounds__(64) void decode_mfma_kernel(kitty_kv_layer L, const __half* __restrict__ q, int H_Q,
+                                                         float scaling, float* __restrict__ ws_ml,
+                                                         float* __restrict__ ws_acc, int num_splits) {
+  __shared__ WaveLds S;
+  Ctx x;
+  x.L = &L;
+  x.b = blockIdx.z;
+  x.h = blockIdx.y;
+  const int split = blockIdx.x;
+  x.lane = threadIdx.x;
+  x.kg = x.lane >> 4;
+  x.n = x.lane & 15;
+  x.c = load_counts(L, x.b);
+  x.lane_off = (2 * x.kg + (x.n & 1)) * kRowBytes + (x.n >> 1) * 4;
+  x.sel = (x.n & 1) ? 0x03020706u : 0x05040100u;
+  x.sc2 = scaling * kLog2e;
+  const int G = H_Q / L.H_KV;
+  const int g = x.n % G;
+
+  // q of this column: operand-order pairs in registers, natural order in LDS for the slot gather
+  const __half* qrow = q + ((int64_t)x.b * H_Q + (int64_t)x.h * G + g) * kD;
+#pragma unroll
+  for (int kc = 0; kc < 4; ++kc)
+#pragma unroll
+    for (int pi = 0; pi < 4; ++pi) x.qpair[kc * 4 + pi] = *(const uint32_t*)(qrow + 32 * kc + 8 * pi + 2 * x.kg);
+  {
+    const uint4* src = (const uint4*)(qrow + 32 * x.kg);
+    uint4* dst = (uint4*)&S.q_nat[x.n][32 * x.kg];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) dst[i] = src[i];
+    if (x.kg == 0) S.q_nat[x.n][128] = (_Float16)0.0f;
+    if (x.lane == 0) S.ks4_nat[128] = (_Float16)0.0f;
+  }
+  __syncthreads();
+
+  Acc A;
+#pragma unroll
+  for (int u = 0; u < 8; ++u) A.out[u] = float4v{0.f, 0.f, 0.f, 0.f};
+  A.m = 0.f;
+  A.l = 0.f;
+  A.z = 0.f;
+  A.first = true;
+  A.true_units = false;
+
+  // Tiles whose V side is packed are shared by all splits but the last, which takes the rest
+  // (tiles with fp16 V rows and the sink); a single split takes everything.
+  const int nbt = c_div_up(x.c.nbody, kPage);
+  const int nvp = min(x.c.pv, nbt);
+  int t0, t1;
+  bool tail;
+  if (num_splits == 1) {
+    t0 = 0; t1 = nvp; tail = true;
+  } else if (split < num_splits - 1) {
+    const int per = (nvp + num_splits - 2) / (num_splits - 1);
+    t0 = min(nvp, split * per); t1 = min(nvp, t0 + per); tail = false;
+  } else {
+    t0 = t1 = 0; tail = true;
+  }
+  const uint8_t* qbuf_k = (const uint8_t*)L.qbuf_k + (int64_t)x.b * L.win_stride_b + (int64_t)x.h * L.win_stride_h;
+
+  float4v C[8];
+#pragma unroll 1
+  for (int i = t0; i < t1; ++i) {
+    float cz = 0.f;
+    const int ntok = min(kPage, x.c.nbody - i * kPage);
+    if (i < x.c.pk) qk_packed<BOOST>(S, x, i, C, cz);
+    else qk_fp16(x, qbuf_k, kPage, C);
+    softmax_tile(x, A, C, cz, ntok);
+    pv_packed(S, x, A, i, C);
+  }
+  if (tail) {
+    to_true_units(A);
+#pragma unroll 1
+    for (int i = nvp; i < nbt; ++i) {
+      float cz = 0.f;
+      const int ntok = min(kPage, x.c.nbody - i * kPage);
+      if (i < x.c.pk) qk_packed<BOOST>(S, x, i, C, cz);
+      else qk_fp16(x, qbuf_k, kPage, C);
+      softmax_tile(x, A, C, cz, ntok);
+      pv_fp16<false>(x, A, (i - x.c.pv) * kPage, ntok, C);
+    }
+    if (x.c.sink > 0) {
+      const uint8_t* sink_k = (const uint8_t*)L.sink_k + (int64_t)x.b * L.sink_stride_b + (int64_t)x.h * L.sink_stride_h;
+      qk_fp16(x, sink_k, L.S, C);
+      softmax_tile(x, A, C, 0.f, x.c.sink);
+      pv_fp16<true>(x, A, 0, x.c.sink, C);
+    }
+  }
+  to_true_units(A);
+
+  // ---- partial of this split: columns n < G are the G heads -----------------------------------
+  float l = A.l, z = A.z;
+  l += xor_lanes(l, 16); l += xor_lanes(l, 32);
+  z += xor_lanes(z, 16); z += xor_lanes(z, 32);
+  if (x.n < G) {
+    const int64_t row = ((int64_t)x.b * H_Q + (int64_t)x.h * G + x.n) * num_splits + split;
+    if (x.kg == 0) {
+      ws_ml[row * 2] = A.first ? -INFINITY : A.m;
+      ws_ml[row * 2 + 1] = l;
+    }
+#pragma unroll
+    for (int u = 0; u < 8; ++u)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) ws_acc[row * kD + 32 * x.kg + 8 * j + u] = A.out[u][j] + z;
+  }
+}
+
+}  // namespace
+
+bool decode_mfma_supported(const kitty_kv_layer& L, int H_Q) {
+  return (L.D_BOOSTED == 32 || L.D_BOOSTED == 0) && L.D == kD && L.PAGE_SIZE == kPage && H_Q / L.H_KV <= 16;
+}
+
+void launch_decode_mfma(const kitty_kv_layer& L, const void* q, int B, int H_Q, float scaling, float* ws_ml,
+                        float* ws_acc, int num_splits, hipStream_t stream) {
+  const dim3 grid(num_splits, L.H_KV, B), block(64);
+  if (L.D_BOOSTED == 32)
+    hipLaunchKernelGGL(decode_mfma_kernel<true>, grid, block, 0, stream, L, (const __half*)q, H_Q, scaling, ws_ml,
+                       ws_acc, num_splits);
+  else
+    hipLaunchKernelGGL(decode_mfma_kernel<false>, grid, block, 0, stream, L, (const __half*)q, H_Q, scaling, ws_ml,
+                       ws_acc, num_splits);
+}
+
 }  // namespace kitty
