@@ -92,17 +92,41 @@ struct Ctx {
 // ---------------------------------------------------------------------------------------------
 // K side
 // ---------------------------------------------------------------------------------------------
-// Stage one K page-head's (scale, zero) pairs and slot map in LDS in the order the operands need:
+// Everything one packed K page-head contributes, as loaded from HBM: 16 low-plane words, 4
+// high-plane words, this lane's two (scale, zero) pairs and its two slot-map bytes.
+struct KBuf {
+  uint32_t lo[16], hi[4];
+  uint2 meta;
+  uint32_t idx2;
+};
+
+template <bool BOOST>
+__device__ __forceinline__ void k_issue_loads(const Ctx& x, int page_index, KBuf& kb) {
+  const kitty_kv_layer& L = *x.L;
+  const int64_t pg = L.page_table_k[(int64_t)x.b * L.page_table_k_stride_b + page_index];
+  const uint8_t* page = L.key_cache + pg * L.key_cache_stride_page + (int64_t)x.h * k_head_bytes(BOOST ? 32 : 0);
+  const uint8_t* meta = (const uint8_t*)L.key_meta + pg * L.key_meta_stride_page + (int64_t)x.h * kD * 4;
+#pragma unroll
+  for (int c = 0; c < 16; ++c) kb.lo[c] = *(const uint32_t*)(page + c * 256 + x.lane_off);
+  if (BOOST) {
+#pragma unroll
+    for (int c = 0; c < 4; ++c) kb.hi[c] = *(const uint32_t*)(page + kLoBytes + c * 256 + x.lane_off);
+    kb.idx2 = *(const uint16_t*)(page + kRowBytes * (kD + 32) + 2 * x.lane);
+  }
+  kb.meta = *(const uint2*)(meta + x.lane * 8);                          // [s0|z0], [s1|z1]
+}
+
+// Stage the page-head's (scale, zero) pairs and slot map in LDS in the order the operands need:
 // channel pair (2l, 2l+1) of lane l belongs to chunk kc = l/16, pair pi = (l/4)%4, lane group
 // l%4 and is stored at word 16kc + 4kg + pi, so that a lane reads the four pairs of a chunk with
 // one 128-bit LDS read.
 template <bool BOOST>
-__device__ __forceinline__ void stage_k_meta(WaveLds& S, const Ctx& x, const uint8_t* page, const uint8_t* meta) {
+__device__ __forceinline__ void stage_k_meta(WaveLds& S, const Ctx& x, const KBuf& kb) {
   const int l = x.lane;
-  const uint2 km = *(const uint2*)(meta + l * 8);                       // [s0|z0], [s1|z1]
-  const uint32_t ss = __builtin_amdgcn_perm(km.y, km.x, 0x05040100u);   // (s0, s1)
-  const uint32_t zz = __builtin_amdgcn_perm(km.y, km.x, 0x07060302u);   // (z0, z1)
+  const uint32_t ss = __builtin_amdgcn_perm(kb.meta.y, kb.meta.x, 0x05040100u);   // (s0, s1)
+  const uint32_t zz = __builtin_amdgcn_perm(kb.meta.y, kb.meta.x, 0x07060302u);   // (z0, z1)
   const int pos = (l >> 4) * 16 + (l & 3) * 4 + ((l >> 2) & 3);
+  __syncthreads();
   S.ks_perm[pos] = ss;
   S.kz_perm[pos] = zz;
   if (BOOST) {
@@ -110,30 +134,18 @@ __device__ __forceinline__ void stage_k_meta(WaveLds& S, const Ctx& x, const uin
     ((uint32_t*)S.ks4_nat)[l] = as_u32(as_h2(ss) * four);
     if (l < 8) ((uint32_t*)S.inv)[l] = 0x80808080u;
     __syncthreads();
-    const uint32_t ib = *(const uint16_t*)(page + kRowBytes * (kD + 32) + 2 * l);
-    const uint32_t i0 = ib & 0xffu, i1 = ib >> 8;
+    const uint32_t i0 = kb.idx2 & 0xffu, i1 = kb.idx2 >> 8;
     if (i0 < 32) S.inv[i0] = (uint8_t)(2 * l);
     if (i1 < 32) S.inv[i1] = (uint8_t)(2 * l + 1);
   }
   __syncthreads();
 }
 
-// logits of one packed K page: C[u][j] = sum_ch code * q * scale (subnormal-scaled), cz = q . zero
+// logits of one packed K page: C[u][j] = sum_ch code * q * scale, still in subnormal units
+// (multiply by code_unscale(u)); cz = q . zero
 template <bool BOOST>
-__device__ __forceinline__ void qk_packed(WaveLds& S, const Ctx& x, int page_index, float4v (&C)[8], float& cz) {
-  const kitty_kv_layer& L = *x.L;
-  const int64_t pg = L.page_table_k[(int64_t)x.b * L.page_table_k_stride_b + page_index];
-  const uint8_t* page = L.key_cache + pg * L.key_cache_stride_page + (int64_t)x.h * k_head_bytes(BOOST ? 32 : 0);
-  const uint8_t* meta = (const uint8_t*)L.key_meta + pg * L.key_meta_stride_page + (int64_t)x.h * kD * 4;
-  uint32_t klo[16], khi[4];
-#pragma unroll
-  for (int c = 0; c < 16; ++c) klo[c] = *(const uint32_t*)(page + c * 256 + x.lane_off);
-  if (BOOST) {
-#pragma unroll
-    for (int c = 0; c < 4; ++c) khi[c] = *(const uint32_t*)(page + kLoBytes + c * 256 + x.lane_off);
-  }
-  stage_k_meta<BOOST>(S, x, page, meta);
-
+__device__ __forceinline__ void qk_packed(WaveLds& S, const Ctx& x, const KBuf& kb, float4v (&C)[8], float& cz) {
+  stage_k_meta<BOOST>(S, x, kb);
   float czl = 0.f;
 #pragma unroll
   for (int u = 0; u < 8; ++u) C[u] = float4v{0.f, 0.f, 0.f, 0.f};
@@ -150,7 +162,7 @@ __device__ __forceinline__ void qk_packed(WaveLds& S, const Ctx& x, int page_ind
       bh[pi] = as_u32(hi);
       bl[pi] = as_u32(lo);
       czl = __builtin_amdgcn_fdot2(qq, as_h2(zp[pi]), czl, false);
-      const uint32_t own = klo[kc * 4 + pi];
+      const uint32_t own = kb.lo[kc * 4 + pi];
       X[pi] = __builtin_amdgcn_perm(swap_pair(own), own, x.sel);
       Y[pi] = X[pi] >> 10;
     }
@@ -177,7 +189,7 @@ __device__ __forceinline__ void qk_packed(WaveLds& S, const Ctx& x, int page_ind
       const half2v lo = __builtin_elementwise_fma(qq, s2, -hi);
       bh[pi] = as_u32(hi);
       bl[pi] = as_u32(lo);
-      const uint32_t own = khi[pi];
+      const uint32_t own = kb.hi[pi];
       X[pi] = __builtin_amdgcn_perm(swap_pair(own), own, x.sel);
       Y[pi] = X[pi] >> 10;
     }
@@ -193,8 +205,6 @@ __device__ __forceinline__ void qk_packed(WaveLds& S, const Ctx& x, int page_ind
   czl += xor_lanes(czl, 16);
   czl += xor_lanes(czl, 32);
   cz = czl;
-#pragma unroll
-  for (int u = 0; u < 8; ++u) C[u] *= code_unscale(u);
 }
 
 // logits of up to 128 fp16 rows (sink or K Q-buffer): A = the rows themselves, B = q
@@ -218,8 +228,10 @@ __device__ __forceinline__ void qk_fp16(const Ctx& x, const uint8_t* rows, int n
 }
 
 // ---------------------------------------------------------------------------------------------
-// softmax bookkeeping: C holds logits * (1/sc2) on entry, probabilities on exit
+// softmax bookkeeping: C holds raw dot products on entry (SUBNORMAL: in code units, to be
+// multiplied by code_unscale(u)), probabilities on exit
 // ---------------------------------------------------------------------------------------------
+template <bool SUBNORMAL>
 __device__ __forceinline__ void softmax_tile(const Ctx& x, Acc& A, float4v (&C)[8], float cz, int ntok) {
   const float cst = cz * x.sc2 - A.m;
   float mt = -INFINITY;
@@ -227,7 +239,7 @@ __device__ __forceinline__ void softmax_tile(const Ctx& x, Acc& A, float4v (&C)[
   for (int u = 0; u < 8; ++u)
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      float v = C[u][j] * x.sc2 + cst;                       // log2-logit relative to the running max
+      float v = C[u][j] * (SUBNORMAL ? code_unscale(u) * x.sc2 : x.sc2) + cst;   // log2-logit - running max
       if (ntok < kPage && 32 * x.kg + 8 * j + u >= ntok) v = -INFINITY;
       C[u][j] = v;
       mt = fmaxf(mt, v);
@@ -260,22 +272,28 @@ __device__ __forceinline__ void softmax_tile(const Ctx& x, Acc& A, float4v (&C)[
 // ---------------------------------------------------------------------------------------------
 // V side
 // ---------------------------------------------------------------------------------------------
-__device__ __forceinline__ void pv_packed(WaveLds& S, const Ctx& x, Acc& A, int page_index, const float4v (&P)[8]) {
+struct VBuf {
+  uint32_t w[16];
+  uint2 meta;
+};
+
+__device__ __forceinline__ void v_issue_loads(const Ctx& x, int page_index, VBuf& vb) {
   const kitty_kv_layer& L = *x.L;
   const int64_t pg = L.page_table_v[(int64_t)x.b * L.page_table_v_stride_b + page_index];
   const uint8_t* page = L.value_cache + pg * L.value_cache_stride_page + (int64_t)x.h * kVBytes;
   const uint8_t* meta = (const uint8_t*)L.value_meta + pg * L.value_meta_stride_page + (int64_t)x.h * kPage * 4;
-  uint32_t vw[16];
   const uint32_t v_off = (32 * x.kg + (x.n & 1)) * kRowBytes + (x.n >> 1) * 4;
 #pragma unroll
-  for (int c = 0; c < 16; ++c) vw[c] = *(const uint32_t*)(page + v_off + c * 64);   // rows 32kg + 2c + (n&1)
-  {
-    const uint2 vm = *(const uint2*)(meta + x.lane * 8);                  // tokens 2l, 2l+1
-    __syncthreads();
-    S.vs_nat[x.lane] = __builtin_amdgcn_perm(vm.y, vm.x, 0x05040100u);
-    S.vz_nat[x.lane] = __builtin_amdgcn_perm(vm.y, vm.x, 0x07060302u);
-    __syncthreads();
-  }
+  for (int c = 0; c < 16; ++c) vb.w[c] = *(const uint32_t*)(page + v_off + c * 64);   // rows 32kg + 2c + (n&1)
+  vb.meta = *(const uint2*)(meta + x.lane * 8);                                        // tokens 2l, 2l+1
+}
+
+__device__ __forceinline__ void pv_packed(WaveLds& S, const Ctx& x, float4v (&out)[8], float& l, float& z,
+                                          const VBuf& vb, const float4v (&P)[8]) {
+  __syncthreads();
+  S.vs_nat[x.lane] = __builtin_amdgcn_perm(vb.meta.y, vb.meta.x, 0x05040100u);
+  S.vz_nat[x.lane] = __builtin_amdgcn_perm(vb.meta.y, vb.meta.x, 0x07060302u);
+  __syncthreads();
   const half2v ones = {(_Float16)1.0f, (_Float16)1.0f};
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
@@ -285,10 +303,10 @@ __device__ __forceinline__ void pv_packed(WaveLds& S, const Ctx& x, Acc& A, int 
 #pragma unroll
     for (int pi = 0; pi < 4; ++pi) {
       const half2v p2 = {(_Float16)P[2 * pi][j], (_Float16)P[2 * pi + 1][j]};   // tokens 32kg + 8j + 2pi + {0,1}
-      A.l = __builtin_amdgcn_fdot2(p2, ones, A.l, false);
-      A.z = __builtin_amdgcn_fdot2(p2, as_h2(zp[pi]), A.z, false);
+      l = __builtin_amdgcn_fdot2(p2, ones, l, false);
+      z = __builtin_amdgcn_fdot2(p2, as_h2(zp[pi]), z, false);
       bp[pi] = as_u32(p2 * as_h2(sp[pi]));
-      const uint32_t own = vw[4 * j + pi];
+      const uint32_t own = vb.w[4 * j + pi];
       X[pi] = __builtin_amdgcn_perm(swap_pair(own), own, x.sel);
       Y[pi] = X[pi] >> 10;
     }
@@ -297,7 +315,7 @@ __device__ __forceinline__ void pv_packed(WaveLds& S, const Ctx& x, Acc& A, int 
       uint32_t a[4];
 #pragma unroll
       for (int pi = 0; pi < 4; ++pi) a[pi] = (u < 5 ? X[pi] : Y[pi]) & code_mask(u);
-      A.out[u] = mfma16(a, bp, A.out[u]);
+      out[u] = mfma16(a, bp, out[u]);
     }
   }
 }
@@ -350,7 +368,7 @@ __device__ __forceinline__ void to_true_units(Acc& A) {
 }
 
 template <bool BOOST>
-__global__ __launch_bounds__(64) void decode_mfma_kernel(kitty_kv_layer L, const __half* __restrict__ q, int H_Q,
+__global__ __launch_bounds__(64, 2) void decode_mfma_kernel(kitty_kv_layer L, const __half* __restrict__ q, int H_Q,
                                                          float scaling, float* __restrict__ ws_ml,
                                                          float* __restrict__ ws_acc, int num_splits) {
   __shared__ WaveLds S;
@@ -394,47 +412,71 @@ __global__ __launch_bounds__(64) void decode_mfma_kernel(kitty_kv_layer L, const
   A.first = true;
   A.true_units = false;
 
-  // Tiles whose V side is packed are shared by all splits but the last, which takes the rest
-  // (tiles with fp16 V rows and the sink); a single split takes everything.
+  // Tiles with both sides packed are shared by all splits but the last, which takes the rest
+  // (tiles with fp16 rows on either side, and the sink); a single split takes everything.
   const int nbt = c_div_up(x.c.nbody, kPage);
-  const int nvp = min(x.c.pv, nbt);
+  const int npp = min(min(x.c.pv, x.c.pk), nbt);
   int t0, t1;
   bool tail;
   if (num_splits == 1) {
-    t0 = 0; t1 = nvp; tail = true;
+    t0 = 0; t1 = npp; tail = true;
   } else if (split < num_splits - 1) {
-    const int per = (nvp + num_splits - 2) / (num_splits - 1);
-    t0 = min(nvp, split * per); t1 = min(nvp, t0 + per); tail = false;
+    const int per = (npp + num_splits - 2) / (num_splits - 1);
+    t0 = min(npp, split * per); t1 = min(npp, t0 + per); tail = false;
   } else {
     t0 = t1 = 0; tail = true;
   }
   const uint8_t* qbuf_k = (const uint8_t*)L.qbuf_k + (int64_t)x.b * L.win_stride_b + (int64_t)x.h * L.win_stride_h;
 
   float4v C[8];
+  KBuf kb;
+  VBuf vb;
+  // Software pipeline over the packed tiles: the V words of tile i are in flight during its QK
+  // phase, the K words of tile i+1 during its softmax and PV phase.
+  if (t0 < t1) k_issue_loads<BOOST>(x, t0, kb);
 #pragma unroll 1
   for (int i = t0; i < t1; ++i) {
-    float cz = 0.f;
-    const int ntok = min(kPage, x.c.nbody - i * kPage);
-    if (i < x.c.pk) qk_packed<BOOST>(S, x, i, C, cz);
-    else qk_fp16(x, qbuf_k, kPage, C);
-    softmax_tile(x, A, C, cz, ntok);
-    pv_packed(S, x, A, i, C);
+    float cz;
+    v_issue_loads(x, i, vb);
+    qk_packed<BOOST>(S, x, kb, C, cz);
+    // unconditional (the last iteration re-loads its own tile) so that the number of loads in
+    // flight is static and the PV phase only waits for the V words, not for this prefetch
+    k_issue_loads<BOOST>(x, min(i + 1, t1 - 1), kb);
+    softmax_tile<true>(x, A, C, cz, kPage);
+    pv_packed(S, x, A.out, A.l, A.z, vb, C);
   }
   if (tail) {
     to_true_units(A);
 #pragma unroll 1
-    for (int i = nvp; i < nbt; ++i) {
+    for (int i = npp; i < nbt; ++i) {
       float cz = 0.f;
       const int ntok = min(kPage, x.c.nbody - i * kPage);
-      if (i < x.c.pk) qk_packed<BOOST>(S, x, i, C, cz);
-      else qk_fp16(x, qbuf_k, kPage, C);
-      softmax_tile(x, A, C, cz, ntok);
-      pv_fp16<false>(x, A, (i - x.c.pv) * kPage, ntok, C);
+      if (i < x.c.pk) {
+        k_issue_loads<BOOST>(x, i, kb);
+        qk_packed<BOOST>(S, x, kb, C, cz);
+        softmax_tile<true>(x, A, C, cz, ntok);
+      } else {
+        qk_fp16(x, qbuf_k, kPage, C);
+        softmax_tile<false>(x, A, C, 0.f, ntok);
+      }
+      if (i < x.c.pv) {
+        // a packed V page under fp16 keys (only reachable with hand-made counters): accumulate in
+        // code units on the side, then fold in
+        float4v tmp[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) tmp[u] = float4v{0.f, 0.f, 0.f, 0.f};
+        v_issue_loads(x, i, vb);
+        pv_packed(S, x, tmp, A.l, A.z, vb, C);
+#pragma unroll
+        for (int u = 0; u < 8; ++u) A.out[u] += tmp[u] * code_unscale(u);
+      } else {
+        pv_fp16<false>(x, A, (i - x.c.pv) * kPage, ntok, C);
+      }
     }
     if (x.c.sink > 0) {
       const uint8_t* sink_k = (const uint8_t*)L.sink_k + (int64_t)x.b * L.sink_stride_b + (int64_t)x.h * L.sink_stride_h;
       qk_fp16(x, sink_k, L.S, C);
-      softmax_tile(x, A, C, 0.f, x.c.sink);
+      softmax_tile<false>(x, A, C, 0.f, x.c.sink);
       pv_fp16<true>(x, A, 0, x.c.sink, C);
     }
   }
