@@ -49,6 +49,7 @@ struct WaveLds {
   uint32_t ks_perm[64], kz_perm[64];  // K scale / zero pairs in operand order (see stage_k_meta)
   _Float16 ks4_nat[kQPad];            // 4 * K scale by channel; [128] = 0
   uint32_t vs_nat[64], vz_nat[64];    // V scale / zero pairs by token pair
+  uint32_t ones[64];                  // fp16 (1, 1) pairs: the "row of ones" operand
   uint8_t inv[32];                    // high-plane slot -> channel (128 = slot unused)
 };
 
@@ -71,10 +72,42 @@ __device__ __forceinline__ constexpr float code_unscale(int u) {
   return 16777216.0f / (float)(1 << (2 * (u < 5 ? u : u - 5)));
 }
 
+// The eight tiles of one k-chunk against a two-part B operand; the operand registers of the next
+// tile are masked out while the MFMAs of the current one run (two register sets, no copies).
+__device__ __forceinline__ void unpack_mfma2(const uint32_t (&X)[4], const uint32_t (&Y)[4], const uint32_t (&bh)[4],
+                                             const uint32_t (&bl)[4], float4v (&C)[8]) {
+  uint32_t a0[4], a1[4];
+#pragma unroll
+  for (int pi = 0; pi < 4; ++pi) a0[pi] = X[pi] & code_mask(0);
+#pragma unroll
+  for (int u = 0; u < 8; u += 2) {
+    C[u] = mfma16(a0, bh, C[u]);
+#pragma unroll
+    for (int pi = 0; pi < 4; ++pi) a1[pi] = (u + 1 < 5 ? X[pi] : Y[pi]) & code_mask(u + 1);
+    C[u] = mfma16(a0, bl, C[u]);
+    C[u + 1] = mfma16(a1, bh, C[u + 1]);
+    if (u + 2 < 8) {
+#pragma unroll
+      for (int pi = 0; pi < 4; ++pi) a0[pi] = (u + 2 < 5 ? X[pi] : Y[pi]) & code_mask(u + 2);
+    }
+    C[u + 1] = mfma16(a1, bl, C[u + 1]);
+  }
+}
+__device__ __forceinline__ void unpack_mfma1(const uint32_t (&X)[4], const uint32_t (&Y)[4], const uint32_t (&b)[4],
+                                             float4v (&C)[8]) {
+#pragma unroll
+  for (int u = 0; u < 8; ++u) {
+    uint32_t a[4];
+#pragma unroll
+    for (int pi = 0; pi < 4; ++pi) a[pi] = (u < 5 ? X[pi] : Y[pi]) & code_mask(u);
+    C[u] = mfma16(a, b, C[u]);
+  }
+}
+
 struct Acc {
   float4v out[8];     // O^T accumulators, d-tile u: channel 32kg + 8j + u, column n
   float m;            // running max of the column's logits, log2 units
-  float l, z;         // lane-local sums over this lane's tokens of p and p * zero_v
+  float4v lz;         // [0] = sum of p, [1] = sum of p * zero_v over all tokens seen (whole column)
   bool first;         // nothing accumulated yet
   bool true_units;    // out[] already multiplied by code_unscale (fp16-V tiles accumulate directly)
 };
@@ -146,14 +179,15 @@ __device__ __forceinline__ void stage_k_meta(WaveLds& S, const Ctx& x, const KBu
 template <bool BOOST>
 __device__ __forceinline__ void qk_packed(WaveLds& S, const Ctx& x, const KBuf& kb, float4v (&C)[8], float& cz) {
   stage_k_meta<BOOST>(S, x, kb);
-  float czl = 0.f;
+  // q . zero_k on the matrix core as well: an A tile whose 16 rows all hold the zero points
+  float4v Cz = float4v{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
   for (int u = 0; u < 8; ++u) C[u] = float4v{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
   for (int kc = 0; kc < 4; ++kc) {
     const uint4v sp = *(const uint4v*)&S.ks_perm[kc * 16 + x.kg * 4];
     const uint4v zp = *(const uint4v*)&S.kz_perm[kc * 16 + x.kg * 4];
-    uint32_t bh[4], bl[4], X[4], Y[4];
+    uint32_t bh[4], bl[4], bq[4], az[4], X[4], Y[4];
 #pragma unroll
     for (int pi = 0; pi < 4; ++pi) {
       const half2v qq = as_h2(x.qpair[kc * 4 + pi]), s2 = as_h2(sp[pi]);
@@ -161,19 +195,14 @@ __device__ __forceinline__ void qk_packed(WaveLds& S, const Ctx& x, const KBuf& 
       const half2v lo = __builtin_elementwise_fma(qq, s2, -hi);    // ... and its exact remainder
       bh[pi] = as_u32(hi);
       bl[pi] = as_u32(lo);
-      czl = __builtin_amdgcn_fdot2(qq, as_h2(zp[pi]), czl, false);
+      bq[pi] = x.qpair[kc * 4 + pi];
+      az[pi] = zp[pi];
       const uint32_t own = kb.lo[kc * 4 + pi];
       X[pi] = __builtin_amdgcn_perm(swap_pair(own), own, x.sel);
       Y[pi] = X[pi] >> 10;
     }
-#pragma unroll
-    for (int u = 0; u < 8; ++u) {
-      uint32_t a[4];
-#pragma unroll
-      for (int pi = 0; pi < 4; ++pi) a[pi] = (u < 5 ? X[pi] : Y[pi]) & code_mask(u);
-      C[u] = mfma16(a, bh, C[u]);
-      C[u] = mfma16(a, bl, C[u]);
-    }
+    Cz = mfma16(az, bq, Cz);
+    unpack_mfma2(X, Y, bh, bl, C);
   }
   if (BOOST) {
     // fifth chunk: the 32 high-plane slots; slot 8pi + 2kg + h carries bits 3:2 of the channel
@@ -193,18 +222,9 @@ __device__ __forceinline__ void qk_packed(WaveLds& S, const Ctx& x, const KBuf& 
       X[pi] = __builtin_amdgcn_perm(swap_pair(own), own, x.sel);
       Y[pi] = X[pi] >> 10;
     }
-#pragma unroll
-    for (int u = 0; u < 8; ++u) {
-      uint32_t a[4];
-#pragma unroll
-      for (int pi = 0; pi < 4; ++pi) a[pi] = (u < 5 ? X[pi] : Y[pi]) & code_mask(u);
-      C[u] = mfma16(a, bh, C[u]);
-      C[u] = mfma16(a, bl, C[u]);
-    }
+    unpack_mfma2(X, Y, bh, bl, C);
   }
-  czl += xor_lanes(czl, 16);
-  czl += xor_lanes(czl, 32);
-  cz = czl;
+  cz = Cz[0];
 }
 
 // logits of up to 128 fp16 rows (sink or K Q-buffer): A = the rows themselves, B = q
@@ -242,8 +262,9 @@ __device__ __forceinline__ void softmax_tile(const Ctx& x, Acc& A, float4v (&C)[
       float v = C[u][j] * (SUBNORMAL ? code_unscale(u) * x.sc2 : x.sc2) + cst;   // log2-logit - running max
       if (ntok < kPage && 32 * x.kg + 8 * j + u >= ntok) v = -INFINITY;
       C[u][j] = v;
-      mt = fmaxf(mt, v);
     }
+#pragma unroll
+  for (int u = 0; u < 8; ++u) mt = fmaxf(fmaxf(mt, fmaxf(C[u][0], C[u][1])), fmaxf(C[u][2], C[u][3]));
   mt = fmaxf(mt, xor_lanes(mt, 16));
   mt = fmaxf(mt, xor_lanes(mt, 32));
   if (__any(A.first || mt > 0.f)) {
@@ -255,8 +276,7 @@ __device__ __forceinline__ void softmax_tile(const Ctx& x, Acc& A, float4v (&C)[
       for (int j = 0; j < 4; ++j) C[u][j] -= dm;
     if (!A.first) {
       const float alpha = __builtin_amdgcn_exp2f(-dm);
-      A.l *= alpha;
-      A.z *= alpha;
+      A.lz *= alpha;
 #pragma unroll
       for (int u = 0; u < 8; ++u) A.out[u] *= alpha;
     }
@@ -288,35 +308,32 @@ __device__ __forceinline__ void v_issue_loads(const Ctx& x, int page_index, VBuf
   vb.meta = *(const uint2*)(meta + x.lane * 8);                                        // tokens 2l, 2l+1
 }
 
-__device__ __forceinline__ void pv_packed(WaveLds& S, const Ctx& x, float4v (&out)[8], float& l, float& z,
-                                          const VBuf& vb, const float4v (&P)[8]) {
+__device__ __forceinline__ void pv_packed(WaveLds& S, const Ctx& x, float4v (&out)[8], float4v& lz, const VBuf& vb,
+                                          const float4v (&P)[8]) {
   __syncthreads();
   S.vs_nat[x.lane] = __builtin_amdgcn_perm(vb.meta.y, vb.meta.x, 0x05040100u);
   S.vz_nat[x.lane] = __builtin_amdgcn_perm(vb.meta.y, vb.meta.x, 0x07060302u);
   __syncthreads();
-  const half2v ones = {(_Float16)1.0f, (_Float16)1.0f};
+  // sum p and sum p*zero_v ride along as one more A tile: even rows are ones, odd rows the zero
+  // points, so row 0 of the product is the column's sum of p and row 1 its sum of p * zero_v
+  const uint32_t* lz_rows = (x.n & 1) ? S.vz_nat : S.ones;
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
     const uint4v sp = *(const uint4v*)&S.vs_nat[16 * x.kg + 4 * j];
-    const uint4v zp = *(const uint4v*)&S.vz_nat[16 * x.kg + 4 * j];
-    uint32_t bp[4], X[4], Y[4];
+    const uint4v zr = *(const uint4v*)&lz_rows[16 * x.kg + 4 * j];
+    uint32_t bp[4], p16[4], alz[4], X[4], Y[4];
 #pragma unroll
     for (int pi = 0; pi < 4; ++pi) {
       const half2v p2 = {(_Float16)P[2 * pi][j], (_Float16)P[2 * pi + 1][j]};   // tokens 32kg + 8j + 2pi + {0,1}
-      l = __builtin_amdgcn_fdot2(p2, ones, l, false);
-      z = __builtin_amdgcn_fdot2(p2, as_h2(zp[pi]), z, false);
+      p16[pi] = as_u32(p2);
+      alz[pi] = zr[pi];
       bp[pi] = as_u32(p2 * as_h2(sp[pi]));
       const uint32_t own = vb.w[4 * j + pi];
       X[pi] = __builtin_amdgcn_perm(swap_pair(own), own, x.sel);
       Y[pi] = X[pi] >> 10;
     }
-#pragma unroll
-    for (int u = 0; u < 8; ++u) {
-      uint32_t a[4];
-#pragma unroll
-      for (int pi = 0; pi < 4; ++pi) a[pi] = (u < 5 ? X[pi] : Y[pi]) & code_mask(u);
-      out[u] = mfma16(a, bp, out[u]);
-    }
+    lz = mfma16(alz, p16, lz);
+    unpack_mfma1(X, Y, bp, out);
   }
 }
 
@@ -324,10 +341,10 @@ __device__ __forceinline__ void pv_packed(WaveLds& S, const Ctx& x, float4v (&ou
 template <bool SINK>
 __device__ __forceinline__ void pv_fp16(const Ctx& x, Acc& A, int tail_first_row, int ntok, const float4v (&P)[8]) {
   const kitty_kv_layer& L = *x.L;
-  const half2v ones = {(_Float16)1.0f, (_Float16)1.0f};
+  const uint32_t one_or_zero = (x.n & 1) ? 0u : 0x3C003C00u;    // even rows sum p, odd rows stay 0
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
-    uint32_t bp[4];
+    uint32_t bp[4], alz[4];
     const __half* rp[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
@@ -342,9 +359,10 @@ __device__ __forceinline__ void pv_fp16(const Ctx& x, Acc& A, int tail_first_row
 #pragma unroll
     for (int pi = 0; pi < 4; ++pi) {
       const half2v p2 = {(_Float16)P[2 * pi][j], (_Float16)P[2 * pi + 1][j]};
-      A.l = __builtin_amdgcn_fdot2(p2, ones, A.l, false);
       bp[pi] = as_u32(p2);
+      alz[pi] = one_or_zero;
     }
+    A.lz = mfma16(alz, bp, A.lz);
 #pragma unroll
     for (int u = 0; u < 8; ++u) {
       uint32_t a[4];
@@ -400,6 +418,7 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(kitty_kv_layer L, co
     for (int i = 0; i < 4; ++i) dst[i] = src[i];
     if (x.kg == 0) S.q_nat[x.n][128] = (_Float16)0.0f;
     if (x.lane == 0) S.ks4_nat[128] = (_Float16)0.0f;
+    S.ones[x.lane] = 0x3C003C00u;
   }
   __syncthreads();
 
@@ -407,8 +426,7 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(kitty_kv_layer L, co
 #pragma unroll
   for (int u = 0; u < 8; ++u) A.out[u] = float4v{0.f, 0.f, 0.f, 0.f};
   A.m = 0.f;
-  A.l = 0.f;
-  A.z = 0.f;
+  A.lz = float4v{0.f, 0.f, 0.f, 0.f};
   A.first = true;
   A.true_units = false;
 
@@ -443,7 +461,7 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(kitty_kv_layer L, co
     // flight is static and the PV phase only waits for the V words, not for this prefetch
     k_issue_loads<BOOST>(x, min(i + 1, t1 - 1), kb);
     softmax_tile<true>(x, A, C, cz, kPage);
-    pv_packed(S, x, A.out, A.l, A.z, vb, C);
+    pv_packed(S, x, A.out, A.lz, vb, C);
   }
   if (tail) {
     to_true_units(A);
@@ -466,7 +484,7 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(kitty_kv_layer L, co
 #pragma unroll
         for (int u = 0; u < 8; ++u) tmp[u] = float4v{0.f, 0.f, 0.f, 0.f};
         v_issue_loads(x, i, vb);
-        pv_packed(S, x, tmp, A.l, A.z, vb, C);
+        pv_packed(S, x, tmp, A.lz, vb, C);
 #pragma unroll
         for (int u = 0; u < 8; ++u) A.out[u] += tmp[u] * code_unscale(u);
       } else {
@@ -483,9 +501,7 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(kitty_kv_layer L, co
   to_true_units(A);
 
   // ---- partial of this split: columns n < G are the G heads -----------------------------------
-  float l = A.l, z = A.z;
-  l += xor_lanes(l, 16); l += xor_lanes(l, 32);
-  z += xor_lanes(z, 16); z += xor_lanes(z, 32);
+  const float l = A.lz[0], z = A.lz[1];
   if (x.n < G) {
     const int64_t row = ((int64_t)x.b * H_Q + (int64_t)x.h * G + x.n) * num_splits + split;
     if (x.kg == 0) {
