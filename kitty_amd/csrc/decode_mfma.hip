@@ -44,13 +44,32 @@ typedef uint32_t uint4v __attribute__((ext_vector_type(4)));
 constexpr float kLog2e = 1.44269504088896340736f;
 constexpr int kQPad = 136;   // q_nat row length in halves: 128 channels + a zero entry at 128
 
-struct WaveLds {
-  _Float16 q_nat[16][kQPad];          // [column][channel]; [..][128] = 0 (the "no channel" slot)
+// A packed K page-head as it sits in LDS after the global->LDS loads: low plane, high plane, slot
+// map (128 bytes, loaded twice), (scale, zero) pairs.  A V page-head: codes (16-byte pieces
+// swizzled, see dma_v) and (scale, zero) pairs.
+constexpr int kKOffHi = 4096, kKOffIdx = 5120, kKOffMeta = 5376, kKTile = 5888;
+constexpr int kVOffMeta = 4096, kVTile = 4608;
+
+struct Tables {
   uint32_t ks_perm[64], kz_perm[64];  // K scale / zero pairs in operand order (see stage_k_meta)
   _Float16 ks4_nat[kQPad];            // 4 * K scale by channel; [128] = 0
   uint32_t vs_nat[64], vz_nat[64];    // V scale / zero pairs by token pair
   uint32_t ones[64];                  // fp16 (1, 1) pairs: the "row of ones" operand
   uint8_t inv[32];                    // high-plane slot -> channel (128 = slot unused)
+};
+// LDS of one wave.  With tiles streamed through LDS (DMA) the budget is 160 KB / 8 waves per CU,
+// which leaves room for the q rows of 8 heads; larger groups use the register-fed variant.
+template <bool DMA>
+struct WaveLds;
+template <>
+struct WaveLds<true> : Tables {
+  __attribute__((aligned(16))) uint8_t kbuf[2][kKTile];
+  __attribute__((aligned(16))) uint8_t vbuf[kVTile];
+  __attribute__((aligned(16))) _Float16 q_nat[8][kQPad];   // [head][channel]; [..][128] = 0 ("no channel")
+};
+template <>
+struct WaveLds<false> : Tables {
+  __attribute__((aligned(16))) _Float16 q_nat[16][kQPad];
 };
 
 __device__ __forceinline__ float4v mfma16(const uint32_t (&a)[4], const uint32_t (&b)[4], float4v c) {
@@ -61,7 +80,7 @@ __device__ __forceinline__ float4v mfma16(const uint32_t (&a)[4], const uint32_t
 __device__ __forceinline__ half2v as_h2(uint32_t u) { return __builtin_bit_cast(half2v, u); }
 __device__ __forceinline__ uint32_t as_u32(half2v h) { return __builtin_bit_cast(uint32_t, h); }
 __device__ __forceinline__ uint32_t swap_pair(uint32_t v) {   // value of lane n^1
-  return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0xB1 /* quad_perm [1,0,3,2] */, 0xf, 0xf, false);
+  return (uint32_t)__builtin_amdgcn_mov_dpp((int)v, 0xB1 /* quad_perm [1,0,3,2] */, 0xf, 0xf, true);
 }
 __device__ __forceinline__ float xor_lanes(float v, int mask) { return __shfl_xor(v, mask); }
 
@@ -118,6 +137,9 @@ struct Ctx {
   int b, h, lane, kg, n;
   uint32_t lane_off;    // byte offset of this lane's word inside a 256-byte plane chunk
   uint32_t sel;         // v_perm selector merging own / partner halves
+  int g;                // query head of this column (n % G)
+  uint32_t kb0;         // LDS: byte offset of this lane's 16-bit piece in plane row 2kg (K tiles)
+  uint32_t vb[4];       // LDS: same for V rows 32kg + 2pi, swizzled (V tiles)
   float sc2;            // scaling * log2(e)
   uint32_t qpair[16];   // q[col][32kc + 8pi + 2kg + {0,1}] as an fp16 pair, index 4kc + pi
 };
@@ -125,16 +147,40 @@ struct Ctx {
 // ---------------------------------------------------------------------------------------------
 // K side
 // ---------------------------------------------------------------------------------------------
-// Everything one packed K page-head contributes, as loaded from HBM: 16 low-plane words, 4
-// high-plane words, this lane's two (scale, zero) pairs and its two slot-map bytes.
-struct KBuf {
+// Two ways a packed K page-head reaches the operands.  Both hand out, per 256-byte plane chunk,
+// X = [8 codes of plane row 2kg | 8 codes of row 2kg+1] for this lane's token octet.
+//
+// KRegs: 20 words in registers, loaded straight from HBM; halves swapped between lanes n, n^1.
+struct KRegs {
   uint32_t lo[16], hi[4];
   uint2 meta;
   uint32_t idx2;
+  __device__ __forceinline__ uint32_t x_lo(const Ctx& x, int c) const {
+    return __builtin_amdgcn_perm(swap_pair(lo[c]), lo[c], x.sel);
+  }
+  __device__ __forceinline__ uint32_t x_hi(const Ctx& x, int c) const {
+    return __builtin_amdgcn_perm(swap_pair(hi[c]), hi[c], x.sel);
+  }
+  __device__ __forceinline__ uint2 meta2(const Ctx&) const { return meta; }
+  __device__ __forceinline__ uint32_t idx(const Ctx&) const { return idx2; }
+};
+// KLds: the whole page-head in LDS; the two 16-bit pieces are read where they lie and merged.
+struct KLds {
+  const uint8_t* base;
+  __device__ __forceinline__ uint32_t x_lo(const Ctx& x, int c) const {
+    const uint16_t* p = (const uint16_t*)(base + c * 256 + x.kb0);
+    return __builtin_amdgcn_perm(p[16], p[0], 0x05040100u);     // [row 2kg piece | row 2kg+1 piece]
+  }
+  __device__ __forceinline__ uint32_t x_hi(const Ctx& x, int c) const {
+    const uint16_t* p = (const uint16_t*)(base + kKOffHi + c * 256 + x.kb0);
+    return __builtin_amdgcn_perm(p[16], p[0], 0x05040100u);
+  }
+  __device__ __forceinline__ uint2 meta2(const Ctx& x) const { return *(const uint2*)(base + kKOffMeta + x.lane * 8); }
+  __device__ __forceinline__ uint32_t idx(const Ctx& x) const { return *(const uint16_t*)(base + kKOffIdx + 2 * x.lane); }
 };
 
 template <bool BOOST>
-__device__ __forceinline__ void k_issue_loads(const Ctx& x, int page_index, KBuf& kb) {
+__device__ __forceinline__ void k_load_regs(const Ctx& x, int page_index, KRegs& kb) {
   const kitty_kv_layer& L = *x.L;
   const int64_t pg = L.page_table_k[(int64_t)x.b * L.page_table_k_stride_b + page_index];
   const uint8_t* page = L.key_cache + pg * L.key_cache_stride_page + (int64_t)x.h * k_head_bytes(BOOST ? 32 : 0);
@@ -149,15 +195,50 @@ __device__ __forceinline__ void k_issue_loads(const Ctx& x, int page_index, KBuf
   kb.meta = *(const uint2*)(meta + x.lane * 8);                          // [s0|z0], [s1|z1]
 }
 
+// Global -> LDS loads of one K page-head (no registers involved): scalar base + per-lane offset,
+// the LDS destination is M0 + instruction offset + lane * size.  8 instructions with the high
+// plane, 6 without.
+template <bool BOOST>
+constexpr int kDmaK = BOOST ? 8 : 6;
+constexpr int kDmaV = 6;
+
+template <bool BOOST>
+__device__ __forceinline__ void dma_k(const Ctx& x, int page_index, uint32_t lds) {
+  const kitty_kv_layer& L = *x.L;
+  const int64_t pg = L.page_table_k[(int64_t)x.b * L.page_table_k_stride_b + page_index];
+  const uint8_t* page = L.key_cache + pg * L.key_cache_stride_page + (int64_t)x.h * k_head_bytes(BOOST ? 32 : 0);
+  const uint8_t* meta = (const uint8_t*)L.key_meta + pg * L.key_meta_stride_page + (int64_t)x.h * kD * 4;
+  const uint32_t off16 = x.lane * 16, off4 = x.lane * 4, off4dup = (x.lane & 31) * 4;
+  asm volatile(
+      "s_mov_b32 m0, %2\n\t"
+      "global_load_lds_dwordx4 %0, %1\n\t"
+      "global_load_lds_dwordx4 %0, %1 offset:1024\n\t"
+      "global_load_lds_dwordx4 %0, %1 offset:2048\n\t"
+      "global_load_lds_dwordx4 %0, %1 offset:3072"
+      :: "v"(off16), "s"(page), "s"(lds) : "memory", "m0");
+  if (BOOST) {
+    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1"
+                 :: "v"(off16), "s"(page + kLoBytes), "s"(lds + kKOffHi) : "memory", "m0");
+    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dword %0, %1"
+                 :: "v"(off4dup), "s"(page + kLoBytes + 1024), "s"(lds + kKOffIdx) : "memory", "m0");
+  }
+  asm volatile(
+      "s_mov_b32 m0, %2\n\t"
+      "global_load_lds_dword %0, %1\n\t"
+      "global_load_lds_dword %0, %1 offset:256"
+      :: "v"(off4), "s"(meta), "s"(lds + kKOffMeta) : "memory", "m0");
+}
+
 // Stage the page-head's (scale, zero) pairs and slot map in LDS in the order the operands need:
 // channel pair (2l, 2l+1) of lane l belongs to chunk kc = l/16, pair pi = (l/4)%4, lane group
 // l%4 and is stored at word 16kc + 4kg + pi, so that a lane reads the four pairs of a chunk with
 // one 128-bit LDS read.
-template <bool BOOST>
-__device__ __forceinline__ void stage_k_meta(WaveLds& S, const Ctx& x, const KBuf& kb) {
+template <bool BOOST, class LDS, class KSRC>
+__device__ __forceinline__ void stage_k_meta(LDS& S, const Ctx& x, const KSRC& kb) {
   const int l = x.lane;
-  const uint32_t ss = __builtin_amdgcn_perm(kb.meta.y, kb.meta.x, 0x05040100u);   // (s0, s1)
-  const uint32_t zz = __builtin_amdgcn_perm(kb.meta.y, kb.meta.x, 0x07060302u);   // (z0, z1)
+  const uint2 km = kb.meta2(x);
+  const uint32_t ss = __builtin_amdgcn_perm(km.y, km.x, 0x05040100u);   // (s0, s1)
+  const uint32_t zz = __builtin_amdgcn_perm(km.y, km.x, 0x07060302u);   // (z0, z1)
   const int pos = (l >> 4) * 16 + (l & 3) * 4 + ((l >> 2) & 3);
   __syncthreads();
   S.ks_perm[pos] = ss;
@@ -167,7 +248,8 @@ __device__ __forceinline__ void stage_k_meta(WaveLds& S, const Ctx& x, const KBu
     ((uint32_t*)S.ks4_nat)[l] = as_u32(as_h2(ss) * four);
     if (l < 8) ((uint32_t*)S.inv)[l] = 0x80808080u;
     __syncthreads();
-    const uint32_t i0 = kb.idx2 & 0xffu, i1 = kb.idx2 >> 8;
+    const uint32_t ib = kb.idx(x);
+    const uint32_t i0 = ib & 0xffu, i1 = ib >> 8;
     if (i0 < 32) S.inv[i0] = (uint8_t)(2 * l);
     if (i1 < 32) S.inv[i1] = (uint8_t)(2 * l + 1);
   }
@@ -176,8 +258,8 @@ __device__ __forceinline__ void stage_k_meta(WaveLds& S, const Ctx& x, const KBu
 
 // logits of one packed K page: C[u][j] = sum_ch code * q * scale, still in subnormal units
 // (multiply by code_unscale(u)); cz = q . zero
-template <bool BOOST>
-__device__ __forceinline__ void qk_packed(WaveLds& S, const Ctx& x, const KBuf& kb, float4v (&C)[8], float& cz) {
+template <bool BOOST, class LDS, class KSRC>
+__device__ __forceinline__ void qk_packed(LDS& S, const Ctx& x, const KSRC& kb, float4v (&C)[8], float& cz) {
   stage_k_meta<BOOST>(S, x, kb);
   // q . zero_k on the matrix core as well: an A tile whose 16 rows all hold the zero points
   float4v Cz = float4v{0.f, 0.f, 0.f, 0.f};
@@ -197,8 +279,7 @@ __device__ __forceinline__ void qk_packed(WaveLds& S, const Ctx& x, const KBuf& 
       bl[pi] = as_u32(lo);
       bq[pi] = x.qpair[kc * 4 + pi];
       az[pi] = zp[pi];
-      const uint32_t own = kb.lo[kc * 4 + pi];
-      X[pi] = __builtin_amdgcn_perm(swap_pair(own), own, x.sel);
+      X[pi] = kb.x_lo(x, kc * 4 + pi);
       Y[pi] = X[pi] >> 10;
     }
     Cz = mfma16(az, bq, Cz);
@@ -212,14 +293,13 @@ __device__ __forceinline__ void qk_packed(WaveLds& S, const Ctx& x, const KBuf& 
     for (int pi = 0; pi < 4; ++pi) {
       const uint32_t cc = *(const uint16_t*)&S.inv[8 * pi + 2 * x.kg];
       const uint32_t c0 = cc & 0xffu, c1 = cc >> 8;
-      const half2v qq = {S.q_nat[x.n][c0], S.q_nat[x.n][c1]};
+      const half2v qq = {S.q_nat[x.g][c0], S.q_nat[x.g][c1]};
       const half2v s2 = {S.ks4_nat[c0], S.ks4_nat[c1]};
       const half2v hi = qq * s2;
       const half2v lo = __builtin_elementwise_fma(qq, s2, -hi);
       bh[pi] = as_u32(hi);
       bl[pi] = as_u32(lo);
-      const uint32_t own = kb.hi[pi];
-      X[pi] = __builtin_amdgcn_perm(swap_pair(own), own, x.sel);
+      X[pi] = kb.x_hi(x, pi);
       Y[pi] = X[pi] >> 10;
     }
     unpack_mfma2(X, Y, bh, bl, C);
@@ -292,12 +372,24 @@ __device__ __forceinline__ void softmax_tile(const Ctx& x, Acc& A, float4v (&C)[
 // ---------------------------------------------------------------------------------------------
 // V side
 // ---------------------------------------------------------------------------------------------
-struct VBuf {
+struct VRegs {
   uint32_t w[16];
   uint2 meta;
+  __device__ __forceinline__ uint32_t xv(const Ctx& x, int j, int pi) const {
+    return __builtin_amdgcn_perm(swap_pair(w[4 * j + pi]), w[4 * j + pi], x.sel);
+  }
+  __device__ __forceinline__ uint2 meta2(const Ctx&) const { return meta; }
+};
+struct VLds {
+  const uint8_t* base;
+  __device__ __forceinline__ uint32_t xv(const Ctx& x, int j, int pi) const {
+    const uint16_t* p = (const uint16_t*)(base + j * 256 + x.vb[pi]);
+    return __builtin_amdgcn_perm(p[16], p[0], 0x05040100u);
+  }
+  __device__ __forceinline__ uint2 meta2(const Ctx& x) const { return *(const uint2*)(base + kVOffMeta + x.lane * 8); }
 };
 
-__device__ __forceinline__ void v_issue_loads(const Ctx& x, int page_index, VBuf& vb) {
+__device__ __forceinline__ void v_load_regs(const Ctx& x, int page_index, VRegs& vb) {
   const kitty_kv_layer& L = *x.L;
   const int64_t pg = L.page_table_v[(int64_t)x.b * L.page_table_v_stride_b + page_index];
   const uint8_t* page = L.value_cache + pg * L.value_cache_stride_page + (int64_t)x.h * kVBytes;
@@ -308,11 +400,38 @@ __device__ __forceinline__ void v_issue_loads(const Ctx& x, int page_index, VBuf
   vb.meta = *(const uint2*)(meta + x.lane * 8);                                        // tokens 2l, 2l+1
 }
 
-__device__ __forceinline__ void pv_packed(WaveLds& S, const Ctx& x, float4v (&out)[8], float4v& lz, const VBuf& vb,
+// Global -> LDS loads of one V page-head.  Lane group kg reads rows 32kg .. 32kg+31, i.e. the
+// four groups would hit the same LDS banks 1 KB apart; so instruction q (which fills LDS bytes
+// 1024q ..) fetches its 16-byte pieces in the order lane ^ 4q, which rotates the 64-byte windows
+// of the four groups apart (see Ctx::vb for the matching read offsets).
+__device__ __forceinline__ void dma_v(const Ctx& x, int page_index, uint32_t lds) {
+  const kitty_kv_layer& L = *x.L;
+  const int64_t pg = L.page_table_v[(int64_t)x.b * L.page_table_v_stride_b + page_index];
+  const uint8_t* page = L.value_cache + pg * L.value_cache_stride_page + (int64_t)x.h * kVBytes;
+  const uint8_t* meta = (const uint8_t*)L.value_meta + pg * L.value_meta_stride_page + (int64_t)x.h * kPage * 4;
+  const uint32_t o0 = x.lane * 16, o1 = (x.lane ^ 4) * 16, o2 = (x.lane ^ 8) * 16, o3 = (x.lane ^ 12) * 16;
+  asm volatile(
+      "s_mov_b32 m0, %5\n\t"
+      "global_load_lds_dwordx4 %0, %4\n\t"
+      "global_load_lds_dwordx4 %1, %4 offset:1024\n\t"
+      "global_load_lds_dwordx4 %2, %4 offset:2048\n\t"
+      "global_load_lds_dwordx4 %3, %4 offset:3072"
+      :: "v"(o0), "v"(o1), "v"(o2), "v"(o3), "s"(page), "s"(lds) : "memory", "m0");
+  const uint32_t off4 = x.lane * 4;
+  asm volatile(
+      "s_mov_b32 m0, %2\n\t"
+      "global_load_lds_dword %0, %1\n\t"
+      "global_load_lds_dword %0, %1 offset:256"
+      :: "v"(off4), "s"(meta), "s"(lds + kVOffMeta) : "memory", "m0");
+}
+
+template <class LDS, class VSRC>
+__device__ __forceinline__ void pv_packed(LDS& S, const Ctx& x, float4v (&out)[8], float4v& lz, const VSRC& vb,
                                           const float4v (&P)[8]) {
+  const uint2 vm = vb.meta2(x);
   __syncthreads();
-  S.vs_nat[x.lane] = __builtin_amdgcn_perm(vb.meta.y, vb.meta.x, 0x05040100u);
-  S.vz_nat[x.lane] = __builtin_amdgcn_perm(vb.meta.y, vb.meta.x, 0x07060302u);
+  S.vs_nat[x.lane] = __builtin_amdgcn_perm(vm.y, vm.x, 0x05040100u);
+  S.vz_nat[x.lane] = __builtin_amdgcn_perm(vm.y, vm.x, 0x07060302u);
   __syncthreads();
   // sum p and sum p*zero_v ride along as one more A tile: even rows are ones, odd rows the zero
   // points, so row 0 of the product is the column's sum of p and row 1 its sum of p * zero_v
@@ -328,8 +447,7 @@ __device__ __forceinline__ void pv_packed(WaveLds& S, const Ctx& x, float4v (&ou
       p16[pi] = as_u32(p2);
       alz[pi] = zr[pi];
       bp[pi] = as_u32(p2 * as_h2(sp[pi]));
-      const uint32_t own = vb.w[4 * j + pi];
-      X[pi] = __builtin_amdgcn_perm(swap_pair(own), own, x.sel);
+      X[pi] = vb.xv(x, j, pi);
       Y[pi] = X[pi] >> 10;
     }
     lz = mfma16(alz, p16, lz);
@@ -385,11 +503,17 @@ __device__ __forceinline__ void to_true_units(Acc& A) {
   }
 }
 
-template <bool BOOST>
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+  asm volatile("s_waitcnt vmcnt(%0)" :: "n"(N) : "memory");
+}
+
+// DMA: packed tiles are streamed global -> LDS (G <= 8); otherwise they are loaded into registers.
+template <bool BOOST, bool DMA>
 __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(kitty_kv_layer L, const __half* __restrict__ q, int H_Q,
-                                                         float scaling, float* __restrict__ ws_ml,
-                                                         float* __restrict__ ws_acc, int num_splits) {
-  __shared__ WaveLds S;
+                                                            float scaling, float* __restrict__ ws_ml,
+                                                            float* __restrict__ ws_acc, int num_splits) {
+  __shared__ WaveLds<DMA> S;
   Ctx x;
   x.L = &L;
   x.b = blockIdx.z;
@@ -403,23 +527,26 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(kitty_kv_layer L, co
   x.sel = (x.n & 1) ? 0x03020706u : 0x05040100u;
   x.sc2 = scaling * kLog2e;
   const int G = H_Q / L.H_KV;
-  const int g = x.n % G;
+  x.g = x.n % G;
+  x.kb0 = x.kg * 64 + 2 * x.n;
+#pragma unroll
+  for (int pi = 0; pi < 4; ++pi) x.vb[pi] = x.kg * 1024 + ((pi ^ x.kg) * 64) + 2 * x.n;
 
   // q of this column: operand-order pairs in registers, natural order in LDS for the slot gather
-  const __half* qrow = q + ((int64_t)x.b * H_Q + (int64_t)x.h * G + g) * kD;
+  const __half* qrow = q + ((int64_t)x.b * H_Q + (int64_t)x.h * G + x.g) * kD;
 #pragma unroll
   for (int kc = 0; kc < 4; ++kc)
 #pragma unroll
     for (int pi = 0; pi < 4; ++pi) x.qpair[kc * 4 + pi] = *(const uint32_t*)(qrow + 32 * kc + 8 * pi + 2 * x.kg);
-  {
+  if (x.n < G) {   // one copy per head
     const uint4* src = (const uint4*)(qrow + 32 * x.kg);
-    uint4* dst = (uint4*)&S.q_nat[x.n][32 * x.kg];
+    uint4* dst = (uint4*)&S.q_nat[x.g][32 * x.kg];
 #pragma unroll
     for (int i = 0; i < 4; ++i) dst[i] = src[i];
-    if (x.kg == 0) S.q_nat[x.n][128] = (_Float16)0.0f;
-    if (x.lane == 0) S.ks4_nat[128] = (_Float16)0.0f;
-    S.ones[x.lane] = 0x3C003C00u;
+    if (x.kg == 0) S.q_nat[x.g][128] = (_Float16)0.0f;
   }
+  if (x.lane == 0) S.ks4_nat[128] = (_Float16)0.0f;
+  S.ones[x.lane] = 0x3C003C00u;
   __syncthreads();
 
   Acc A;
@@ -447,30 +574,63 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(kitty_kv_layer L, co
   const uint8_t* qbuf_k = (const uint8_t*)L.qbuf_k + (int64_t)x.b * L.win_stride_b + (int64_t)x.h * L.win_stride_h;
 
   float4v C[8];
-  KBuf kb;
-  VBuf vb;
-  // Software pipeline over the packed tiles: the V words of tile i are in flight during its QK
-  // phase, the K words of tile i+1 during its softmax and PV phase.
-  if (t0 < t1) k_issue_loads<BOOST>(x, t0, kb);
+  if constexpr (DMA) {
+    // Tiles stream through LDS: two K buffers, one V buffer.  Issue order
+    //   K(t0) K(t0+1) V(t0) | QK(i) -> K(i+2) -> softmax -> PV(i) -> V(i+1) | ...
+    // so K(i) has a lead of one and a half iterations and V(i) of half an iteration.  Loads past
+    // the end re-read the last tile, which keeps the number in flight static: the waits below
+    // count instructions issued AFTER the tile that is needed.
+    if (t0 < t1) {
+      constexpr int nK = kDmaK<BOOST>;
+      const uint32_t lk0 = (uint32_t)(uintptr_t)&S.kbuf[0][0], lk1 = (uint32_t)(uintptr_t)&S.kbuf[1][0];
+      const uint32_t lv = (uint32_t)(uintptr_t)&S.vbuf[0];
+      dma_k<BOOST>(x, t0, lk0);
+      dma_k<BOOST>(x, min(t0 + 1, t1 - 1), lk1);
+      dma_v(x, t0, lv);
 #pragma unroll 1
-  for (int i = t0; i < t1; ++i) {
-    float cz;
-    v_issue_loads(x, i, vb);
-    qk_packed<BOOST>(S, x, kb, C, cz);
-    // unconditional (the last iteration re-loads its own tile) so that the number of loads in
-    // flight is static and the PV phase only waits for the V words, not for this prefetch
-    k_issue_loads<BOOST>(x, min(i + 1, t1 - 1), kb);
-    softmax_tile<true>(x, A, C, cz, kPage);
-    pv_packed(S, x, A.out, A.lz, vb, C);
+      for (int i = t0; i < t1; ++i) {
+        float cz;
+        const int buf = (i - t0) & 1;
+        if (i == t0) wait_vmcnt<nK + kDmaV>(); else wait_vmcnt<nK + 2 * kDmaV>();
+        qk_packed<BOOST>(S, x, KLds{S.kbuf[buf]}, C, cz);
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        dma_k<BOOST>(x, min(i + 2, t1 - 1), buf ? lk1 : lk0);
+        softmax_tile<true>(x, A, C, cz, kPage);
+        wait_vmcnt<nK>();
+        pv_packed(S, x, A.out, A.lz, VLds{S.vbuf}, C);
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        dma_v(x, min(i + 1, t1 - 1), lv);
+      }
+      wait_vmcnt<0>();
+    }
+  } else {
+    // Register-fed software pipeline: the V words of tile i are in flight during its QK phase,
+    // the K words of tile i+1 during its softmax and PV phase.
+    KRegs kb;
+    VRegs vb;
+    if (t0 < t1) k_load_regs<BOOST>(x, t0, kb);
+#pragma unroll 1
+    for (int i = t0; i < t1; ++i) {
+      float cz;
+      v_load_regs(x, i, vb);
+      qk_packed<BOOST>(S, x, kb, C, cz);
+      // unconditional (the last iteration re-loads its own tile) so that the number of loads in
+      // flight is static and the PV phase only waits for the V words, not for this prefetch
+      k_load_regs<BOOST>(x, min(i + 1, t1 - 1), kb);
+      softmax_tile<true>(x, A, C, cz, kPage);
+      pv_packed(S, x, A.out, A.lz, vb, C);
+    }
   }
   if (tail) {
     to_true_units(A);
+    KRegs kb;
+    VRegs vb;
 #pragma unroll 1
     for (int i = npp; i < nbt; ++i) {
       float cz = 0.f;
       const int ntok = min(kPage, x.c.nbody - i * kPage);
       if (i < x.c.pk) {
-        k_issue_loads<BOOST>(x, i, kb);
+        k_load_regs<BOOST>(x, i, kb);
         qk_packed<BOOST>(S, x, kb, C, cz);
         softmax_tile<true>(x, A, C, cz, ntok);
       } else {
@@ -483,7 +643,7 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(kitty_kv_layer L, co
         float4v tmp[8];
 #pragma unroll
         for (int u = 0; u < 8; ++u) tmp[u] = float4v{0.f, 0.f, 0.f, 0.f};
-        v_issue_loads(x, i, vb);
+        v_load_regs(x, i, vb);
         pv_packed(S, x, tmp, A.lz, vb, C);
 #pragma unroll
         for (int u = 0; u < 8; ++u) A.out[u] += tmp[u] * code_unscale(u);
@@ -524,12 +684,15 @@ bool decode_mfma_supported(const kitty_kv_layer& L, int H_Q) {
 void launch_decode_mfma(const kitty_kv_layer& L, const void* q, int B, int H_Q, float scaling, float* ws_ml,
                         float* ws_acc, int num_splits, hipStream_t stream) {
   const dim3 grid(num_splits, L.H_KV, B), block(64);
-  if (L.D_BOOSTED == 32)
-    hipLaunchKernelGGL(decode_mfma_kernel<true>, grid, block, 0, stream, L, (const __half*)q, H_Q, scaling, ws_ml,
-                       ws_acc, num_splits);
-  else
-    hipLaunchKernelGGL(decode_mfma_kernel<false>, grid, block, 0, stream, L, (const __half*)q, H_Q, scaling, ws_ml,
-                       ws_acc, num_splits);
+  const bool boost = L.D_BOOSTED == 32, dma = H_Q / L.H_KV <= 8;
+#define KITTY_LAUNCH(BOOST, DMA)                                                                            \
+  hipLaunchKernelGGL((decode_mfma_kernel<BOOST, DMA>), grid, block, 0, stream, L, (const __half*)q, H_Q, scaling, \
+                     ws_ml, ws_acc, num_splits)
+  if (boost && dma) KITTY_LAUNCH(true, true);
+  else if (boost) KITTY_LAUNCH(true, false);
+  else if (dma) KITTY_LAUNCH(false, true);
+  else KITTY_LAUNCH(false, false);
+#undef KITTY_LAUNCH
 }
 
 }  // namespace kitty
