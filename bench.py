@@ -26,6 +26,20 @@ WORKLOADS = {
     "c4": (1, 64, 8, 131072, "long-context decode B=1 64Q/8KV D=128 ctx=131072 (configs[4])"),
 }
 HBM_PEAK_GBPS = 8000.0
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "decode_split_pmc_traffic.txt")
+
+
+def measured_traffic(workload, splits):
+    """HBM bytes per launch of the split pass as measured with rocprofv3 --pmc FETCH_SIZE /
+    WRITE_SIZE on this workload (summary committed under profiles/); None when there is no
+    measurement for this workload."""
+    try:
+        with open(TRAFFIC_FILE) as f:
+            rec = json.load(f).get(workload)
+        return None if rec is None else rec["fetch_bytes"] + rec["write_bytes"]
+    except (OSError, ValueError, KeyError):
+        return None
+
 
 
 def synth_kv(B, H, T, D, seed, device, student_t=False):
@@ -91,6 +105,9 @@ def main():
     ap.add_argument("--splits", type=int, default=0)
     ap.add_argument("--variant", type=int, default=0)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run a plain 1 GiB device copy a few times, so that a counter run of this command "
+                         "holds a kernel of known traffic to scale FETCH_SIZE / WRITE_SIZE by")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build measures the one-GPU kernel path only; run with --gpus 1 "
@@ -178,6 +195,13 @@ def main():
     torch.cuda.synchronize()
     hot_us = sorted(a.elapsed_time(b) * 1e3 for a, b in hot_ev)[len(hot_ev) // 2]
 
+    if args.copy_calibration:
+        src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).fill_(3)
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+
     result = {
         "metric": "packed_kv_decode_attention_us_per_step",
         "value": ms_per_step * 1e3,
@@ -196,7 +220,7 @@ def main():
                    "variant": args.variant, "cache_copies_rotated": len(caches)},
         "roofline": {
             "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-            "frac": achieved / HBM_PEAK_GBPS, "traffic": None,
+            "frac": achieved / HBM_PEAK_GBPS, "traffic": measured_traffic(args.workload, splits),
             "kernel": "decode split pass", "kernel_avg_us": kern_avg_us, "kernel_median_us": kern_us[len(kern_us) // 2],
             "algorithmic_bytes_per_launch": total_bytes, "packed_bytes_per_launch": packed_bytes,
             "packed_gbps": packed_bytes / (kern_avg_us * 1e-6) / 1e9,
