@@ -143,6 +143,23 @@ int kitty_decode_attn_split(const kitty_kv_layer* layer, const void* q, int B, i
 int kitty_decode_attn_merge(const void* workspace, size_t workspace_bytes, int B, int H_Q, int D,
                             int num_splits, void* out, void* stream);
 
+/*
+ * Chunked-prefill attention: T_q new tokens attend to everything the layer already holds (sink
+ * rows, packed pages, fp16 windows, in the token order of decode) and, causally, to the keys and
+ * values of the chunk itself, which are still fp16 and not yet appended.  An extension: the
+ * reference asserts t_query == 1 (kernels/kitty_attention.py:411) and prefills an empty cache
+ * with dense attention (benchmark_kitty.py:302); the arithmetic per cached token is that of
+ * qk_kernel / sv_kernel (kitty_attention.py:162-165, 317-320).  With an empty layer this is plain
+ * causal attention.
+ * q: fp16 [B,H_Q,T_q,D], k_new / v_new: fp16 [B,H_KV,T_q,D] (one set of strides for both), D
+ * contiguous, byte strides as given.  out: fp16 [B,T_q,H_Q,D] contiguous.  No workspace.
+ */
+int kitty_prefill_attn(const kitty_kv_layer* layer,
+                       const void* q, int64_t q_stride_b, int64_t q_stride_h, int64_t q_stride_t,
+                       const void* k_new, const void* v_new,
+                       int64_t new_stride_b, int64_t new_stride_h, int64_t new_stride_t,
+                       int B, int H_Q, int T_q, float scaling, void* out, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

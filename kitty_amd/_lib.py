@@ -54,6 +54,8 @@ _SIGNATURES = {
     "kitty_decode_attn_merge": (c_int, [c_void_p, c_size_t, c_int, c_int, c_int, c_int, c_void_p, c_void_p]),
     "kitty_decode_attn": (c_int, [POINTER(KittyKVLayer), c_void_p, c_int, c_int, c_float, c_void_p, c_void_p,
                                   c_size_t, c_int, c_int, c_void_p]),
+    "kitty_prefill_attn": (c_int, [POINTER(KittyKVLayer), c_void_p, c_int64, c_int64, c_int64, c_void_p, c_void_p,
+                                   c_int64, c_int64, c_int64, c_int, c_int, c_int, c_float, c_void_p, c_void_p]),
 }
 
 EXPORTS = tuple(_SIGNATURES)

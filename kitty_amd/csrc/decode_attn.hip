@@ -10,6 +10,10 @@ void launch_decode_merge(const float* ws_ml, const float* ws_acc, void* out, int
 bool decode_mfma_supported(const kitty_kv_layer& L, int H_Q);
 void launch_decode_mfma(const kitty_kv_layer& L, const void* q, int B, int H_Q, float scaling, float* ws_ml,
                         float* ws_acc, int num_splits, hipStream_t stream);
+void launch_prefill_attn(const kitty_kv_layer& L, const void* q, int64_t q_stride_b, int64_t q_stride_h,
+                         int64_t q_stride_t, const void* k_new, const void* v_new, int64_t new_stride_b,
+                         int64_t new_stride_h, int64_t new_stride_t, int B, int H_Q, int Tq, float scaling,
+                         void* out, hipStream_t stream);
 }  // namespace kitty
 
 using namespace kitty;
@@ -131,4 +135,24 @@ extern "C" int kitty_decode_attn(const kitty_kv_layer* layer, const void* q, int
                                        stream))
     return rc;
   return kitty_decode_attn_merge(workspace, workspace_bytes, B, H_Q, layer->D, num_splits, out, stream);
+}
+
+extern "C" int kitty_prefill_attn(const kitty_kv_layer* layer, const void* q, int64_t q_stride_b,
+                                  int64_t q_stride_h, int64_t q_stride_t, const void* k_new, const void* v_new,
+                                  int64_t new_stride_b, int64_t new_stride_h, int64_t new_stride_t, int B, int H_Q,
+                                  int T_q, float scaling, void* out, void* stream) {
+  int max_tiles = 0;
+  if (int rc = check_layer(layer, q, B, H_Q, &max_tiles)) return rc;
+  KITTY_REQUIRE(k_new && v_new && out, KITTY_E_NULL, "k_new / v_new / out is NULL");
+  KITTY_REQUIRE(T_q >= 1 && T_q <= (1 << 24), KITTY_E_RANGE, "T_q=%d out of range", T_q);
+  KITTY_REQUIRE(layer->D_BOOSTED % 4 == 0, KITTY_E_SHAPE, "unsupported D_BOOSTED=%d", layer->D_BOOSTED);
+  KITTY_REQUIRE(((uintptr_t)k_new % 16) == 0 && ((uintptr_t)v_new % 16) == 0 && ((uintptr_t)out % 16) == 0 &&
+                    q_stride_b % 16 == 0 && q_stride_h % 16 == 0 && q_stride_t % 16 == 0 &&
+                    new_stride_b % 16 == 0 && new_stride_h % 16 == 0 && new_stride_t % 16 == 0,
+                KITTY_E_ALIGN, "q, k_new, v_new and out need 16-byte aligned bases and strides");
+  KITTY_REQUIRE(q_stride_t >= kD * 2 && new_stride_t >= kD * 2, KITTY_E_ALIGN,
+                "a token stride is smaller than one row of D fp16 values");
+  launch_prefill_attn(*layer, q, q_stride_b, q_stride_h, q_stride_t, k_new, v_new, new_stride_b, new_stride_h,
+                      new_stride_t, B, H_Q, T_q, scaling, out, (hipStream_t)stream);
+  return check_launch("kitty_prefill_attn");
 }

@@ -1,0 +1,515 @@
+// Chunked-prefill attention: T_q new tokens attend, causally among themselves, to everything the
+// cache already holds (sink rows, packed pages, fp16 windows) and to the new chunk's own keys
+// and values.  The reference has no such kernel (its prefill runs dense flash attention on an
+// empty cache, benchmark_kitty.py:302, and kitty_attention.py:411 asserts t_query == 1); the
+// arithmetic is the same as decode: softmax(q . k^ * scaling) . v^ with
+// k^ = fp16(code) * scale + zero evaluated in fp16 (kitty_attention.py:162-165, 317-320).
+//
+// The work is a dense contraction (G * T_q query rows per KV head), so it runs on the matrix
+// cores, flash-attention style.  One workgroup of 4 wavefronts owns 256 query rows of one
+// (batch row, KV head): PB = 256 / G consecutive chunk positions times the G query heads of the
+// group; wavefront w owns rows 64w .. 64w+63.  The workgroup walks the sequence in 128-token
+// tiles.  Each tile is brought into LDS once, as fp16, by all 256 threads: packed pages are
+// dequantized on the way (exactly the reference's two fp16 roundings), fp16 rows are copied.
+// Two tile buffers alternate: the global loads of tile t+1 are issued before the arithmetic on
+// tile t and its dequantization follows it, one barrier per tile.
+//
+// Matrix-core formulation (v_mfma_f32_16x16x32_f16; lane = 16 kg + n holds A[n][8 k-slots],
+// B[8 k-slots][n], C[4kg .. 4kg+3][n]):
+//   S^T[pos][row]  = sum_ch  K[pos][ch]  * Q[row][ch]      A = keys,   B = queries (registers)
+//   O^T[cp][row]   = sum_pos V[pos][cp]  * P^T[pos][row]   A = values, B = probabilities
+// The accumulator of the first product is, lane for lane, the B operand of the second: k-slot j
+// of lane group kg stands for position 32 m2 + 16 (j / 4) + 4 kg + j % 4.
+//
+// LDS layouts, chosen so that dequantization writes 128-bit rows and the matrix-core operands
+// come out of `ds_read_b64_tr_b16` (a 16-lane block reads 4 rows x 16 columns and lane i
+// receives column i of the 4 rows):
+//   K tile: [channel][position]       V tile: [position][channel slot]      row pitch 288 bytes
+// "position" and "channel slot" are the order in which codes fall out of a plane word when it is
+// masked with 0x00030003 << 2u: slot 2u + e of a 16-block is element u + 8e.  Keys and values use
+// the same token permutation, the output undoes the channel permutation.
+#include "decode_common.h"
+
+namespace kitty {
+namespace {
+
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef _Float16 half4 __attribute__((ext_vector_type(4)));
+typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+typedef float float4v __attribute__((ext_vector_type(4)));
+typedef short short4v __attribute__((ext_vector_type(4)));
+
+constexpr int kPitch = 288;                   // bytes per LDS row: 128 fp16 + 32 bytes of padding
+constexpr int kTile = kPage * kPitch;         // 36864 bytes, one K or V tile
+constexpr int kLdsBytes = 4 * kTile;          // K and V, two buffers each
+constexpr int kRows = 256;                    // query rows per workgroup
+constexpr int kThreads = 256;
+constexpr float kLog2e = 1.4426950408889634f;
+
+enum SrcKind : int { SRC_PACKED = 0, SRC_ROWS = 1, SRC_VTAIL = 2 };
+
+// where the keys and the values of one 128-token tile come from
+struct TileSrc {
+  int k_kind, v_kind;
+  const uint8_t* k_ptr;   // packed: the page-head;  rows: first row
+  const uint8_t* k_meta;
+  const uint8_t* v_ptr;
+  const uint8_t* v_meta;
+  int64_t k_stride, v_stride;   // rows: bytes between tokens
+  int v_u0;                     // v-tail: index of the tile's first token in [Q_Buffer_V | ring]
+  int ntok;                     // valid tokens
+  int chunk_t0;                 // >= 0: tile of the new chunk starting at this chunk position
+};
+
+// what issue() leaves in flight for a packed tile (fp16 rows are few and are copied by finish())
+struct Stage {
+  uint4 klo, khi, v;
+  uint32_t kmeta, vmeta;
+};
+
+__device__ __forceinline__ int slot_of(int e) {   // element (token or channel) -> LDS slot
+  return (e & ~15) | ((e & 7) << 1) | ((e >> 3) & 1);
+}
+__device__ __forceinline__ int elem_of(int s) {   // LDS slot -> element
+  return (s & ~15) | ((s & 15) >> 1) | ((s & 1) << 3);
+}
+
+__device__ __forceinline__ half4 lds_tr(const uint8_t* p) {
+  short4v r = __builtin_amdgcn_ds_read_tr16_b64_v4i16((short4v __attribute__((address_space(3)))*)p);
+  return __builtin_bit_cast(half4, r);
+}
+
+// matrix-core A operand: k-slots 0..3 from the 4 LDS rows at p, k-slots 4..7 from 16 rows further
+__device__ __forceinline__ half8 load_a(const uint8_t* p) {
+  const half4 a0 = lds_tr(p), a1 = lds_tr(p + 16 * kPitch);
+  return __builtin_shufflevector(a0, a1, 0, 1, 2, 3, 4, 5, 6, 7);
+}
+
+__device__ __forceinline__ float xor_lanes(float v, int mask) { return __shfl_xor(v, mask); }
+
+// fp16(code) * scale + zero with both roundings, for two codes at a time; `c` holds the codes as
+// integers in its two halves.
+__device__ __forceinline__ uint32_t dequant_pair(uint32_t c, half2v scale, half2v zero) {
+#pragma clang fp contract(off)
+  const half2v magic = {(_Float16)1024.f, (_Float16)1024.f};
+  half2v f = __builtin_bit_cast(half2v, c | 0x64006400u) - magic;   // exact: 1024 + code - 1024
+  half2v m = f * scale;
+  half2v r = m + zero;
+  return __builtin_bit_cast(uint32_t, r);
+}
+
+template <bool BOOST>
+struct Prefill {
+  const kitty_kv_layer& L;
+  const SeqCounts c;
+  const int b, h, tid;
+  const uint8_t* k_new;
+  const uint8_t* v_new;
+  int64_t new_stride_t;
+  int kv_chunk;      // chunk tokens this workgroup can see
+  int n_body;        // body tiles
+  int n_tiles;       // sink + body + chunk tiles actually walked
+  int first_body, first_chunk;
+
+  __device__ TileSrc tile(int t) const {
+    TileSrc s;
+    s.chunk_t0 = -1;
+    s.k_meta = s.v_meta = nullptr;
+    s.v_u0 = 0;
+    const int64_t win = (int64_t)b * L.win_stride_b + (int64_t)h * L.win_stride_h;
+    if (t < first_body) {   // the sink rows
+      const int64_t off = (int64_t)b * L.sink_stride_b + (int64_t)h * L.sink_stride_h;
+      s.k_kind = s.v_kind = SRC_ROWS;
+      s.k_ptr = (const uint8_t*)L.sink_k + off;
+      s.v_ptr = (const uint8_t*)L.sink_v + off;
+      s.k_stride = s.v_stride = kD * 2;
+      s.ntok = c.sink;
+    } else if (t < first_chunk) {
+      const int i = t - first_body;
+      s.ntok = min(kPage, c.nbody - i * kPage);
+      if (i < c.pk) {
+        const int64_t pg = L.page_table_k[(int64_t)b * L.page_table_k_stride_b + i];
+        s.k_kind = SRC_PACKED;
+        s.k_ptr = L.key_cache + pg * L.key_cache_stride_page + (int64_t)h * k_head_bytes(L.D_BOOSTED);
+        s.k_meta = (const uint8_t*)L.key_meta + pg * L.key_meta_stride_page + (int64_t)h * kD * 4;
+      } else {
+        s.k_kind = SRC_ROWS;
+        s.k_ptr = (const uint8_t*)L.qbuf_k + win;
+        s.k_stride = kD * 2;
+      }
+      if (i < c.pv) {
+        const int64_t pg = L.page_table_v[(int64_t)b * L.page_table_v_stride_b + i];
+        s.v_kind = SRC_PACKED;
+        s.v_ptr = L.value_cache + pg * L.value_cache_stride_page + (int64_t)h * kVBytes;
+        s.v_meta = (const uint8_t*)L.value_meta + pg * L.value_meta_stride_page + (int64_t)h * kPage * 4;
+      } else {
+        s.v_kind = SRC_VTAIL;
+        s.v_ptr = nullptr;
+        s.v_u0 = (i - c.pv) * kPage;
+      }
+      s.v_stride = 0;
+    } else {
+      const int t0 = (t - first_chunk) * kPage;
+      s.k_kind = s.v_kind = SRC_ROWS;
+      s.k_ptr = k_new + (int64_t)t0 * new_stride_t;
+      s.v_ptr = v_new + (int64_t)t0 * new_stride_t;
+      s.k_stride = s.v_stride = new_stride_t;
+      s.ntok = min(kPage, kv_chunk - t0);
+      s.chunk_t0 = t0;
+    }
+    return s;
+  }
+
+  // ---- stage 1: global loads of a packed tile into registers ----------------------------------
+  __device__ __forceinline__ void issue(const TileSrc& s, Stage& g) const {
+    const int e = tid >> 1, half = tid & 1;   // element (channel or token) and 64-wide half
+    if (s.k_kind == SRC_PACKED) {
+      g.klo = *(const uint4*)(s.k_ptr + e * kRowBytes + half * 16);
+      g.kmeta = *(const uint32_t*)(s.k_meta + e * 4);
+      g.khi = uint4{0u, 0u, 0u, 0u};
+      if (BOOST) {
+        const int slot = s.k_ptr[kLoBytes + L.D_BOOSTED * kRowBytes + e];
+        if (slot < L.D_BOOSTED) g.khi = *(const uint4*)(s.k_ptr + kLoBytes + slot * kRowBytes + half * 16);
+      }
+    }
+    if (s.v_kind == SRC_PACKED) {
+      g.v = *(const uint4*)(s.v_ptr + e * kRowBytes + half * 16);
+      g.vmeta = *(const uint32_t*)(s.v_meta + e * 4);
+    }
+  }
+
+  // ---- stage 2: registers -> fp16 tile in LDS -----------------------------------------------
+  __device__ __forceinline__ void finish(const TileSrc& s, const Stage& g, uint8_t* kt, uint8_t* vt) const {
+    const int e = tid >> 1, half = tid & 1;
+    if (s.k_kind == SRC_PACKED) {
+      // thread = one channel, 64 tokens: four plane words of 16 tokens each
+      const half2v m2 = __builtin_bit_cast(half2v, g.kmeta);
+      const half2v scale = {m2[0], m2[0]}, zero = {m2[1], m2[1]};
+      const uint32_t lo[4] = {g.klo.x, g.klo.y, g.klo.z, g.klo.w};
+      const uint32_t hi[4] = {g.khi.x, g.khi.y, g.khi.z, g.khi.w};
+      uint8_t* row = kt + e * kPitch + half * 128;
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {
+        uint32_t o[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          uint32_t code = (lo[w] >> (2 * u)) & 0x00030003u;
+          if (BOOST) code |= ((hi[w] >> (2 * u)) & 0x00030003u) << 2;
+          o[u] = dequant_pair(code, scale, zero);
+        }
+        *(uint4*)(row + w * 32) = uint4{o[0], o[1], o[2], o[3]};
+        *(uint4*)(row + w * 32 + 16) = uint4{o[4], o[5], o[6], o[7]};
+      }
+    } else if (e < s.ntok) {
+      // thread = one token, 64 channels: transpose into [channel][slot] with 16-bit stores
+      uint8_t* col = kt + (half * 64) * kPitch + slot_of(e) * 2;
+      const uint4* src = (const uint4*)(s.k_ptr + (int64_t)e * s.k_stride + half * 128);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const uint4 x = src[i];
+        const uint32_t w4[4] = {x.x, x.y, x.z, x.w};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          *(uint16_t*)(col + (8 * i + 2 * j) * kPitch) = (uint16_t)(w4[j] & 0xffffu);
+          *(uint16_t*)(col + (8 * i + 2 * j + 1) * kPitch) = (uint16_t)(w4[j] >> 16);
+        }
+      }
+    }
+    uint8_t* vrow = vt + slot_of(e) * kPitch + half * 128;
+    if (s.v_kind == SRC_PACKED) {
+      // thread = one token, 64 channels: four words of 16 channels each
+      const half2v m2 = __builtin_bit_cast(half2v, g.vmeta);
+      const half2v scale = {m2[0], m2[0]}, zero = {m2[1], m2[1]};
+      const uint32_t wv[4] = {g.v.x, g.v.y, g.v.z, g.v.w};
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {
+        uint32_t o[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) o[u] = dequant_pair((wv[w] >> (2 * u)) & 0x00030003u, scale, zero);
+        *(uint4*)(vrow + w * 32) = uint4{o[0], o[1], o[2], o[3]};
+        *(uint4*)(vrow + w * 32 + 16) = uint4{o[4], o[5], o[6], o[7]};
+      }
+    } else {
+      // 16 channels at a time: slot 2u + e' takes channel u + 8e'; dead rows must be finite
+      const bool ok = e < s.ntok;
+      const uint4* src = nullptr;
+      if (ok)
+        src = s.v_kind == SRC_VTAIL
+                  ? (const uint4*)((const uint8_t*)v_tail_row(L, c, b, h, s.v_u0 + e) + half * 128)
+                  : (const uint4*)(s.v_ptr + (int64_t)e * s.v_stride + half * 128);
+      const uint4 zero4 = uint4{0u, 0u, 0u, 0u};
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {
+        const uint4 a = ok ? src[2 * w] : zero4, bb = ok ? src[2 * w + 1] : zero4;   // channels 0..7, 8..15
+        const uint32_t a4[4] = {a.x, a.y, a.z, a.w}, b4[4] = {bb.x, bb.y, bb.z, bb.w};
+        uint32_t o[8];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          o[2 * j] = __builtin_amdgcn_perm(b4[j], a4[j], 0x05040100u);
+          o[2 * j + 1] = __builtin_amdgcn_perm(b4[j], a4[j], 0x07060302u);
+        }
+        *(uint4*)(vrow + w * 32) = uint4{o[0], o[1], o[2], o[3]};
+        *(uint4*)(vrow + w * 32 + 16) = uint4{o[4], o[5], o[6], o[7]};
+      }
+    }
+  }
+};
+
+// One wavefront's state: 64 query rows (4 column tiles of 16) against the tiles in LDS.
+struct WaveAcc {
+  float4v o[8][4];    // O^T: [channel-slot tile][row tile]
+  float m[4], l[4];   // running max (log2 units) per row tile column, per-lane partial sums
+  bool first;
+};
+
+// 64 positions [64 sub, 64 sub + 64) of the tile in (kt, vt) against this wavefront's rows.
+// limit[nt]: tokens of the tile with index < limit are visible to the row of column tile nt.
+__device__ __forceinline__ void attend_sub(const uint8_t* kt, const uint8_t* vt, int sub, const half8 (&q)[4][4],
+                                           WaveAcc& A, float sc2, bool masked, const int (&limit)[4], int kg,
+                                           int n) {
+  float4v S[4][4];
+#pragma unroll
+  for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+    for (int nt = 0; nt < 4; ++nt) S[mt][nt] = float4v{0.f, 0.f, 0.f, 0.f};
+  // lane's corner inside a 16-lane transposing read: row n / 4 of 4, columns 4 (n % 4) ..
+  const int lane_off = (4 * kg + (n >> 2)) * kPitch + (n & 3) * 8;
+  const uint8_t* kbase = kt + lane_off + sub * 128;
+  // channel chunk c+1 is fetched while chunk c is multiplied; the fences keep the scheduler from
+  // hoisting every operand load to the top (which costs more registers than the wave has)
+  half8 a_cur[4], a_nxt[4];
+#pragma unroll
+  for (int mt = 0; mt < 4; ++mt) a_cur[mt] = load_a(kbase + mt * 32);
+#pragma unroll
+  for (int c = 0; c < 4; ++c) {
+    if (c < 3) {
+#pragma unroll
+      for (int mt = 0; mt < 4; ++mt) a_nxt[mt] = load_a(kbase + (32 * (c + 1)) * kPitch + mt * 32);
+    }
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+      for (int nt = 0; nt < 4; ++nt)
+        S[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a_cur[mt], q[c][nt], S[mt][nt], 0, 0, 0);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt) a_cur[mt] = a_nxt[mt];
+  }
+
+  // online softmax, column by column (a column = one query row, spread over the 4 lane groups)
+  float mt_[4];
+#pragma unroll
+  for (int nt = 0; nt < 4; ++nt) {
+    const float cst = -A.m[nt];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        float v = S[mt][nt][i] * sc2 + cst;
+        if (masked) {
+          const int tok = 64 * sub + 16 * mt + 2 * kg + (i >> 1) + 8 * (i & 1);
+          if (tok >= limit[nt]) v = -INFINITY;
+        }
+        S[mt][nt][i] = v;
+        mx = fmaxf(mx, v);
+      }
+    mx = fmaxf(mx, xor_lanes(mx, 16));
+    mx = fmaxf(mx, xor_lanes(mx, 32));
+    mt_[nt] = mx;
+  }
+  const bool move = A.first || mt_[0] > 0.f || mt_[1] > 0.f || mt_[2] > 0.f || mt_[3] > 0.f;
+  if (__any(move)) {
+#pragma unroll
+    for (int nt = 0; nt < 4; ++nt) {
+      const float dm = A.first ? mt_[nt] : fmaxf(mt_[nt], 0.f);
+#pragma unroll
+      for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) S[mt][nt][i] -= dm;
+      if (!A.first) {
+        const float alpha = __builtin_amdgcn_exp2f(-dm);
+        A.l[nt] *= alpha;
+#pragma unroll
+        for (int ct = 0; ct < 8; ++ct) A.o[ct][nt] *= alpha;
+      }
+      A.m[nt] += dm;
+    }
+    A.first = false;
+  }
+  half8 p[2][4];
+#pragma unroll
+  for (int nt = 0; nt < 4; ++nt) {
+    float sum = 0.f;
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float e = __builtin_amdgcn_exp2f(S[mt][nt][i]);
+        S[mt][nt][i] = e;
+        sum += e;
+      }
+    A.l[nt] += sum;
+#pragma unroll
+    for (int m2 = 0; m2 < 2; ++m2) {
+      const float4v x0 = S[2 * m2][nt], x1 = S[2 * m2 + 1][nt];
+      p[m2][nt] = half8{(_Float16)x0[0], (_Float16)x0[1], (_Float16)x0[2], (_Float16)x0[3],
+                        (_Float16)x1[0], (_Float16)x1[1], (_Float16)x1[2], (_Float16)x1[3]};
+    }
+  }
+  const uint8_t* vbase = vt + lane_off + (64 * sub) * kPitch;
+  // 8 groups of (m2, two channel-slot tiles); group i+1 is fetched while group i is multiplied
+  half8 v_cur[2], v_nxt[2];
+  v_cur[0] = load_a(vbase);
+  v_cur[1] = load_a(vbase + 32);
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int m2 = i >> 2, ct = 2 * (i & 3);
+    if (i < 7) {
+      const int m2n = (i + 1) >> 2, ctn = 2 * ((i + 1) & 3);
+      v_nxt[0] = load_a(vbase + (32 * m2n) * kPitch + ctn * 32);
+      v_nxt[1] = load_a(vbase + (32 * m2n) * kPitch + (ctn + 1) * 32);
+    }
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int nt = 0; nt < 4; ++nt)
+        A.o[ct + j][nt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(v_cur[j], p[m2][nt], A.o[ct + j][nt], 0, 0, 0);
+    __builtin_amdgcn_sched_barrier(0);
+    v_cur[0] = v_nxt[0];
+    v_cur[1] = v_nxt[1];
+  }
+}
+
+template <bool BOOST>
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))) void prefill_attn_kernel(
+    kitty_kv_layer L, const uint8_t* __restrict__ q, int64_t q_stride_b, int64_t q_stride_h, int64_t q_stride_t,
+    const uint8_t* __restrict__ k_new, const uint8_t* __restrict__ v_new, int64_t new_stride_b,
+    int64_t new_stride_h, int64_t new_stride_t, int H_Q, int Tq, float scaling, __half* __restrict__ out) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+  const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, kg = lane >> 4, n = lane & 15;
+  const int b = blockIdx.z, h = blockIdx.y;
+  const int G = H_Q / L.H_KV;
+  const int PB = kRows / G;                              // chunk positions per workgroup
+  const int blk = (int)gridDim.x - 1 - (int)blockIdx.x;   // longest causal extent first
+  const int p0 = blk * PB;
+
+  const SeqCounts cnt = load_counts(L, b);
+  Prefill<BOOST> P{L, cnt, b, h, tid,
+                   k_new + (int64_t)b * new_stride_b + (int64_t)h * new_stride_h,
+                   v_new + (int64_t)b * new_stride_b + (int64_t)h * new_stride_h,
+                   new_stride_t, min(Tq, p0 + PB), 0, 0, 0, 0};
+  P.n_body = c_div_up(cnt.nbody, kPage);
+  P.first_body = cnt.sink > 0 ? 1 : 0;
+  P.first_chunk = P.first_body + P.n_body;
+  P.n_tiles = P.first_chunk + c_div_up(P.kv_chunk, kPage);
+
+  // this lane's query rows: column n of row tile nt is row 64 w + 16 nt + n
+  half8 qreg[4][4];
+  int qpos[4];
+#pragma unroll
+  for (int nt = 0; nt < 4; ++nt) {
+    const int r = 64 * w + 16 * nt + n;
+    const int g = r / PB, pos = p0 + r % PB;
+    const bool ok = g < G && pos < Tq;
+    qpos[nt] = ok ? pos : -1;
+    const uint8_t* row = q + (int64_t)b * q_stride_b + (int64_t)(h * G + (ok ? g : 0)) * q_stride_h +
+                         (int64_t)(ok ? pos : 0) * q_stride_t;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      // k-slots 0..3 = channels 32c + 4kg .., k-slots 4..7 = channels 32c + 16 + 4kg ..
+      uint2 x0 = *(const uint2*)(row + (32 * c + 4 * kg) * 2);
+      uint2 x1 = *(const uint2*)(row + (32 * c + 16 + 4 * kg) * 2);
+      if (!ok) x0 = x1 = uint2{0u, 0u};
+      const uint4 x = uint4{x0.x, x0.y, x1.x, x1.y};
+      qreg[c][nt] = __builtin_bit_cast(half8, x);
+    }
+  }
+
+  WaveAcc A;
+#pragma unroll
+  for (int ct = 0; ct < 8; ++ct)
+#pragma unroll
+    for (int nt = 0; nt < 4; ++nt) A.o[ct][nt] = float4v{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int nt = 0; nt < 4; ++nt) A.m[nt] = 0.f, A.l[nt] = 0.f;
+  A.first = true;
+  const float sc2 = scaling * kLog2e;
+
+  Stage g;
+  TileSrc cur = P.tile(0);
+  P.issue(cur, g);
+  P.finish(cur, g, lds, lds + 2 * kTile);
+  __syncthreads();
+#pragma unroll 1
+  for (int t = 0; t < P.n_tiles; ++t) {
+    const int buf = t & 1;
+    const bool more = t + 1 < P.n_tiles;
+    TileSrc nxt = cur;
+    if (more) {
+      nxt = P.tile(t + 1);
+      P.issue(nxt, g);
+    }
+    const uint8_t* kt = lds + buf * kTile;
+    const uint8_t* vt = lds + (2 + buf) * kTile;
+    int limit[4];
+#pragma unroll
+    for (int nt = 0; nt < 4; ++nt)
+      limit[nt] = cur.chunk_t0 >= 0 ? min(cur.ntok, qpos[nt] - cur.chunk_t0 + 1) : cur.ntok;
+    const bool masked = cur.chunk_t0 >= 0 || cur.ntok < kPage;
+    attend_sub(kt, vt, 0, qreg, A, sc2, masked, limit, kg, n);
+    if (cur.ntok > 64) attend_sub(kt, vt, 1, qreg, A, sc2, masked, limit, kg, n);
+    if (more) P.finish(nxt, g, lds + (buf ^ 1) * kTile, lds + (2 + (buf ^ 1)) * kTile);
+    cur = nxt;
+    __syncthreads();
+  }
+
+  // normalise and store: O^T[ct][nt][i] is channel slot 16 ct + 4 kg + i of row 64 w + 16 nt + n
+#pragma unroll
+  for (int nt = 0; nt < 4; ++nt) {
+    float l = A.l[nt];
+    l += xor_lanes(l, 16);
+    l += xor_lanes(l, 32);
+    if (qpos[nt] < 0) continue;
+    const float inv = 1.f / l;
+    const int r = 64 * w + 16 * nt + n;
+    const int g_ = r / PB;
+    __half* orow = out + (((int64_t)b * Tq + qpos[nt]) * H_Q + (h * G + g_)) * kD;
+#pragma unroll
+    for (int ct = 0; ct < 8; ++ct) {
+      const float4v o = A.o[ct][nt] * inv;
+      // slots 4kg + {0, 2} are channels 2kg, 2kg + 1; slots 4kg + {1, 3} are channels 2kg + 8, 2kg + 9
+      *(__half2*)(orow + 16 * ct + 2 * kg) = __floats2half2_rn(o[0], o[2]);
+      *(__half2*)(orow + 16 * ct + 2 * kg + 8) = __floats2half2_rn(o[1], o[3]);
+    }
+  }
+}
+
+}  // namespace
+
+int prefill_lds_bytes() { return kLdsBytes; }
+
+void launch_prefill_attn(const kitty_kv_layer& L, const void* q, int64_t q_stride_b, int64_t q_stride_h,
+                         int64_t q_stride_t, const void* k_new, const void* v_new, int64_t new_stride_b,
+                         int64_t new_stride_h, int64_t new_stride_t, int B, int H_Q, int Tq, float scaling,
+                         void* out, hipStream_t stream) {
+  const int G = H_Q / L.H_KV;
+  const int PB = kRows / G;
+  dim3 grid(c_div_up(Tq, PB), L.H_KV, B), block(kThreads);
+#define KITTY_LAUNCH_PREFILL(BOOST)                                                                              \
+  do {                                                                                                           \
+    /* more LDS than the default per-workgroup limit; per device, so set on every launch */                      \
+    (void)hipFuncSetAttribute((const void*)prefill_attn_kernel<BOOST>,                                           \
+                              hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);                            \
+    hipLaunchKernelGGL((prefill_attn_kernel<BOOST>), grid, block, kLdsBytes, stream, L, (const uint8_t*)q,       \
+                       q_stride_b, q_stride_h, q_stride_t, (const uint8_t*)k_new, (const uint8_t*)v_new,         \
+                       new_stride_b, new_stride_h, new_stride_t, H_Q, Tq, scaling, (__half*)out);                \
+  } while (0)
+  if (L.D_BOOSTED > 0)
+    KITTY_LAUNCH_PREFILL(true);
+  else
+    KITTY_LAUNCH_PREFILL(false);
+#undef KITTY_LAUNCH_PREFILL
+}
+
+}  // namespace kitty

@@ -57,3 +57,53 @@ def kitty_attention_forward(
                                _lib.current_stream_ptr(query.device))
     _lib.check(rc, "kitty_attention_forward")
     return attn_output, None
+
+
+def kitty_prefill_attention(
+    module: nn.Module,
+    query: torch.Tensor,
+    key_states: torch.Tensor,
+    value_states: torch.Tensor,
+    kv_cache: KVCache_Layer,
+    scaling: float,
+):
+    """Chunked-prefill attention: ``query [B, H_Q, T_q, D]`` attends to everything ``kv_cache``
+    holds and, causally, to the chunk's own ``key_states`` / ``value_states [B, H_KV, T_q, D]``
+    (fp16, not yet appended).  Returns ``(attn_output [B, T_q, H_Q, D] fp16, None)``.
+
+    An extension of the reference's interface, whose attention asserts ``t_query == 1``
+    (kitty_attention.py:411) and whose prefill is dense attention on an empty cache
+    (benchmark_kitty.py:302); cached tokens enter exactly as in decode.  Append the chunk afterwards
+    with ``KittyCache.update`` (empty cache) or ``KittyCache.append``.
+    """
+    B, H_Q, T_q, D = query.size()
+    assert H_Q == module.num_attention_heads, "H_Q must match num_attention_heads."
+    H_KV = module.num_key_value_heads
+    KV_GROUP = H_Q // H_KV
+    assert KV_GROUP <= MAX_KV_GROUP, f"KV_GROUP ({KV_GROUP}) exceeds MAX_KV_GROUP ({MAX_KV_GROUP})."
+    for name, t in (("query", query), ("key_states", key_states), ("value_states", value_states)):
+        _lib.require_hip(t, name)
+        if t.dtype != torch.float16:
+            raise ValueError(f"{name} must be float16, got {t.dtype}")
+    if key_states.shape != (B, H_KV, T_q, D) or value_states.shape != key_states.shape:
+        raise ValueError(f"key_states / value_states must be [B, H_KV, T_q, D] = {(B, H_KV, T_q, D)}, got "
+                         f"{tuple(key_states.shape)} / {tuple(value_states.shape)}")
+    if H_KV != kv_cache.H_KV or B > kv_cache.MAX_BS:
+        raise ValueError("query does not match the cache (H_KV or batch size)")
+    if query.stride(-1) != 1:
+        query = query.contiguous()
+    if key_states.stride(-1) != 1:
+        key_states = key_states.contiguous()
+    if value_states.stride() != key_states.stride():
+        value_states = value_states.contiguous()
+        key_states = key_states.contiguous()
+
+    lib = _lib.lib()
+    attn_output = torch.empty((B, T_q, H_Q, D), dtype=query.dtype, device=query.device)
+    desc = kv_cache.descriptor()
+    qs, ks = [x * 2 for x in query.stride()], [x * 2 for x in key_states.stride()]
+    rc = lib.kitty_prefill_attn(desc, query.data_ptr(), qs[0], qs[1], qs[2], key_states.data_ptr(),
+                                value_states.data_ptr(), ks[0], ks[1], ks[2], B, H_Q, T_q, float(scaling),
+                                attn_output.data_ptr(), _lib.current_stream_ptr(query.device))
+    _lib.check(rc, "kitty_prefill_attention")
+    return attn_output, None

@@ -501,3 +501,23 @@ def prefill_attention(query: np.ndarray, K: np.ndarray, V: np.ndarray, scaling: 
         e = np.exp(s - s.max(axis=1, keepdims=True))
         out[hq] = (e / e.sum(axis=1, keepdims=True)) @ V[h].astype(np.float64)
     return out
+
+
+def chunk_attention(layer: OracleLayer, query: np.ndarray, key_chunk: np.ndarray, value_chunk: np.ndarray,
+                    scaling: float, seq_counts: Optional[list] = None, dequant: str = "two") -> np.ndarray:
+    """Chunked-prefill attention over a cache (an extension; the reference attends one token at a
+    time, kitty_attention.py:411).  query [B, H_Q, Tq, D]; key_chunk / value_chunk [B, H_KV, Tq, D]
+    are the chunk's own fp16 keys / values, not yet appended.  Query i sees every cached token (in
+    decode's order, dequantized as decode does) and chunk tokens 0..i.  Float64 throughout after the
+    dequantization.  Returns [B, Tq, H_Q, D] float64.  Pinned by: reduction to `prefill_attention`
+    (textbook causal attention) over `gather_dense_kv`, both pinned on their own; with Tq == 1 it
+    equals decode attention after appending the token."""
+    B, H_Q, Tq, D = query.shape
+    out = np.zeros((B, Tq, H_Q, D), np.float64)
+    for b in range(B):
+        K, V = gather_dense_kv(layer, b, None if seq_counts is None else seq_counts[b], dequant)   # [H_KV, T0, D]
+        T0 = K.shape[1]
+        Kc = np.concatenate([K.astype(np.float64), key_chunk[b].astype(np.float64)], axis=1)
+        Vc = np.concatenate([V.astype(np.float64), value_chunk[b].astype(np.float64)], axis=1)
+        out[b] = prefill_attention(query[b], Kc, Vc, scaling, T0).transpose(1, 0, 2)
+    return out

@@ -46,3 +46,18 @@ def layer_bytes_equal(layer, ol: O.OracleLayer):
         if getattr(layer, f) != getattr(ol, f):
             bad.append((f, getattr(layer, f), getattr(ol, f)))
     return bad
+
+
+def oracle_from_layer(layer, max_len) -> O.OracleLayer:
+    """An OracleLayer holding a copy of a device layer's bytes and counters (to check attention at
+    sizes where quantizing again on the CPU would take minutes; the quantizer is checked elsewhere)."""
+    ol = O.OracleLayer(layer.MAX_BS, max_len, layer.H_KV)
+    for name in ("KeyCache", "KeyCache_metadata", "ValueCache", "ValueCache_metadata", "PageTable_K",
+                 "PageTable_V", "Sink_Buffer_K", "Sink_Buffer_V", "Q_Buffer_K", "Q_Buffer_V", "Local_Buffer_V"):
+        a = getattr(layer, name).detach().cpu().numpy()
+        assert a.shape == getattr(ol, name).shape, name
+        setattr(ol, name, a)
+    for f in ("Sink_Count", "PageCount_K", "PageCount_V", "Q_Buffer_Count_K", "Q_Buffer_Count_V",
+              "Local_Count_V", "Write_Offset_Local_V"):
+        setattr(ol, f, getattr(layer, f))
+    return ol

@@ -1,0 +1,189 @@
+"""GPU parity of chunked-prefill attention (through the Python API, i.e. the C ABI) against the
+oracle: float64 causal attention over [cache dequantized as decode does | the chunk in fp16].
+
+Tolerance: max-abs 2e-3 on fp16 outputs.  The kernel dequantizes a page exactly as the reference's
+expression fp16(code)*scale+zero evaluates eagerly (two fp16 roundings, the oracle's "two" mode),
+so unlike decode there is no dequantization ambiguity in this comparison; what remains is the fp16
+rounding of the probabilities and of the output."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import kitty_oracle as O
+from tests.helpers import make_kv
+
+pytestmark = pytest.mark.gpu
+ATOL = 2e-3
+SC = 128 ** -0.5
+
+
+@pytest.fixture(scope="module")
+def K():
+    if not torch.cuda.is_available():
+        pytest.skip("needs a GPU")
+    import kitty_amd
+    from kitty_amd import _lib
+    _lib.lib()
+    from kitty_amd.kvcache.kernels import kitty_attention_forward, kitty_prefill_attention
+    from tests import gpu_util
+    return type("NS", (), dict(KittyCache=kitty_amd.KittyCache, attn=kitty_attention_forward,
+                               pre=kitty_prefill_attention, u=gpu_util))
+
+
+def _q(B, HQ, Tq, seed):
+    return np.random.default_rng(seed + 31337).standard_normal((B, HQ, Tq, 128)).astype(np.float16)
+
+
+def _state(K, B, H_KV, H_Q, T0, steps, max_len, seed, student_t=False):
+    """Device cache and oracle after a prefill of T0 tokens and `steps` decode steps."""
+    cache = K.KittyCache(K.u.cfg(H_KV, H_Q), B, max_len)
+    ol = O.OracleLayer(B, max_len, H_KV)
+    if T0 == 0:
+        return cache, ol
+    k, v = make_kv(B, H_KV, T0 + steps, seed=seed, student_t=student_t)
+    kd, vd = K.u.to_dev(k), K.u.to_dev(v)
+    cache.update(kd[:, :, :T0], vd[:, :, :T0], 0)
+    cache.quantize_prefill(0)
+    ol.update(k[:, :, :T0], v[:, :, :T0])
+    ol.quantize_prefill()
+    for s in range(steps):
+        t = T0 + s
+        cache.update(kd[:, :, t:t + 1], vd[:, :, t:t + 1], 0)
+        cache.quantize_decode(0)
+        ol.update(k[:, :, t:t + 1], v[:, :, t:t + 1])
+        ol.quantize_decode()
+    assert K.u.layer_bytes_equal(cache.kv_cache[0], ol) == []
+    return cache, ol
+
+
+def _run(K, cache, ol, H_KV, H_Q, B, Tq, seed, student_t=False, what=""):
+    kc, vc = make_kv(B, H_KV, Tq, seed=seed + 1, student_t=student_t)
+    q = _q(B, H_Q, Tq, seed)
+    out, w = K.pre(K.u.module(H_KV, H_Q), K.u.to_dev(q), K.u.to_dev(kc), K.u.to_dev(vc), cache.kv_cache[0], SC)
+    assert w is None and tuple(out.shape) == (B, Tq, H_Q, 128) and out.dtype == torch.float16
+    torch.cuda.synchronize()
+    got = out.cpu().numpy().astype(np.float64)
+    want = O.chunk_attention(ol, q, kc, vc, SC)
+    assert np.isfinite(got).all(), what
+    err = np.abs(got - want).max()
+    assert err <= ATOL, f"{what}: {err:.3e}"
+    return got, q, kc, vc
+
+
+@pytest.mark.parametrize("Tq", [1, 5, 64, 65, 130, 300])
+def test_empty_cache_is_plain_causal_attention(K, Tq):
+    B, H_KV, H_Q = 2, 2, 8
+    cache, ol = _state(K, B, H_KV, H_Q, 0, 0, 1024, seed=1)
+    got, q, kc, vc = _run(K, cache, ol, H_KV, H_Q, B, Tq, seed=Tq, what=f"Tq={Tq}")
+    # the same thing from torch (fp32, CPU): textbook reference independent of the oracle
+    qt, kt, vt = (torch.from_numpy(a).float() for a in (q, kc, vc))
+    ref = torch.nn.functional.scaled_dot_product_attention(
+        qt, kt.repeat_interleave(H_Q // H_KV, 1), vt.repeat_interleave(H_Q // H_KV, 1), is_causal=True, scale=SC)
+    assert np.abs(got - ref.transpose(1, 2).numpy()).max() <= ATOL
+
+
+@pytest.mark.parametrize("T0,steps", [(7, 0), (32, 0), (33, 0), (100, 3), (161, 0), (32 + 128 * 3 + 50, 0),
+                                      (32 + 128 * 2 + 120, 140), (20, 200)])
+@pytest.mark.parametrize("Tq", [1, 33, 200])
+def test_chunk_over_cached_prefix(K, T0, steps, Tq):
+    """Sink only, sink + residual, pages with a mixed K-packed / V-fp16 tile, ring offset != 0."""
+    B, H_KV, H_Q = 2, 2, 8
+    cache, ol = _state(K, B, H_KV, H_Q, T0, steps, 2048, seed=T0 + steps)
+    _run(K, cache, ol, H_KV, H_Q, B, Tq, seed=T0 + Tq, what=f"T0={T0} steps={steps} Tq={Tq}")
+
+
+@pytest.mark.parametrize("G", [1, 2, 3, 4, 8, 16])
+def test_chunk_group_sizes(K, G):
+    B, H_KV, T0, Tq = 1, 2, 32 + 128 * 2 + 77, 150
+    cache, ol = _state(K, B, H_KV, H_KV * G, T0, 0, 1024, seed=G)
+    _run(K, cache, ol, H_KV, H_KV * G, B, Tq, seed=G, what=f"G={G}")
+
+
+def test_one_token_chunk_equals_decode(K):
+    """T_q = 1 is a decode step: same result as appending the token and calling decode attention."""
+    B, H_KV, H_Q, T0 = 2, 2, 8, 32 + 128 * 4 + 9
+    cache, ol = _state(K, B, H_KV, H_Q, T0, 0, 1024, seed=3)
+    got, q, kc, vc = _run(K, cache, ol, H_KV, H_Q, B, 1, seed=3)
+    cache.update(K.u.to_dev(kc), K.u.to_dev(vc), 0)
+    ol.update(kc, vc)
+    kw = dict(reference_rounding=False)
+    d = np.abs(O.decode_attention(ol, q, SC, dequant="two", **kw)
+               - O.decode_attention(ol, q, SC, dequant="affine", **kw)).max()
+    for variant in (0, 1):
+        out, _ = K.attn(K.u.module(H_KV, H_Q), K.u.to_dev(q), cache.kv_cache[0], SC, variant=variant)
+        dec = out.cpu().numpy().astype(np.float64)
+        # two kernels, each within ATOL of its oracle; the matrix-core decode kernel's oracle is the
+        # affine dequantization, d away from the two-rounding one this kernel follows
+        bound = 2 * ATOL + (d if variant == 0 else 0.0)
+        err = np.abs(dec - got).max()
+        assert err <= bound, f"variant {variant}: {err:.3e} > {bound:.3e}"
+
+
+def test_strided_query_and_chunk(K):
+    """[B, T, H, D] projections viewed as [B, H, T, D] (what an attention module holds): no copy."""
+    B, H_KV, H_Q, T0, Tq = 1, 2, 8, 32 + 128 + 40, 70
+    cache, ol = _state(K, B, H_KV, H_Q, T0, 0, 1024, seed=8)
+    kc, vc = make_kv(B, H_KV, Tq, seed=9)
+    q = _q(B, H_Q, Tq, 9)
+    qd = K.u.to_dev(q.transpose(0, 2, 1, 3)).transpose(1, 2)
+    kd = K.u.to_dev(kc.transpose(0, 2, 1, 3)).transpose(1, 2)
+    vd = K.u.to_dev(vc.transpose(0, 2, 1, 3)).transpose(1, 2)
+    assert not qd.is_contiguous() and not kd.is_contiguous()
+    out, _ = K.pre(K.u.module(H_KV, H_Q), qd, kd, vd, cache.kv_cache[0], SC)
+    want = O.chunk_attention(ol, q, kc, vc, SC)
+    assert np.abs(out.cpu().numpy().astype(np.float64) - want).max() <= ATOL
+
+
+def test_ragged_prefix_per_sequence_counts(K):
+    B, H_KV, H_Q, Tq = 3, 2, 8, 90
+    max_len = 32 + 128 * 8
+    cache = K.KittyCache(K.u.cfg(H_KV, H_Q), B, max_len)
+    L = cache.kv_cache[0]
+    rng = np.random.default_rng(5)
+    ols, counts, dicts = [], [], []
+    for b in range(B):
+        T = int(rng.integers(40, max_len - 200))
+        k, v = make_kv(1, H_KV, T + 60, seed=700 + b)
+        ol = O.OracleLayer(1, max_len, H_KV)
+        ol.update(k[:, :, :T], v[:, :, :T])
+        ol.quantize_prefill()
+        for s in range(int(rng.integers(0, 60))):
+            ol.update(k[:, :, T + s:T + s + 1], v[:, :, T + s:T + s + 1])
+            ol.quantize_decode()
+        ols.append(ol)
+        for name in ("Sink_Buffer_K", "Sink_Buffer_V", "Q_Buffer_K", "Q_Buffer_V", "Local_Buffer_V"):
+            getattr(L, name)[b].copy_(K.u.to_dev(getattr(ol, name)[0]))
+        for name in ("KeyCache", "KeyCache_metadata", "ValueCache", "ValueCache_metadata"):
+            getattr(L, name)[b * L.MAX_PAGE:(b + 1) * L.MAX_PAGE].copy_(K.u.to_dev(getattr(ol, name)))
+        counts.append([ol.Sink_Count, ol.PageCount_K, ol.Q_Buffer_Count_K, ol.PageCount_V, ol.Q_Buffer_Count_V,
+                       ol.Local_Count_V, ol.Write_Offset_Local_V, 0])
+    L.seq_counts = torch.tensor(counts, dtype=torch.int32, device="cuda")
+    kc, vc = make_kv(B, H_KV, Tq, seed=55)
+    q = _q(B, H_Q, Tq, 55)
+    out, _ = K.pre(K.u.module(H_KV, H_Q), K.u.to_dev(q), K.u.to_dev(kc), K.u.to_dev(vc), L, SC)
+    got = out.cpu().numpy().astype(np.float64)
+    for b in range(B):
+        want = O.chunk_attention(ols[b], q[b:b + 1], kc[b:b + 1], vc[b:b + 1], SC)
+        assert np.abs(got[b:b + 1] - want).max() <= ATOL, b
+
+
+def test_config3_scaled_down_student_t(K):
+    """BASELINE config 3 at a size the oracle finishes in seconds: heavy-tailed keys, a packed
+    prefix with residual, a chunk of several tiles."""
+    B, H_KV, H_Q, T0, Tq = 2, 2, 8, 32 + 128 * 20 + 96, 512
+    cache, ol = _state(K, B, H_KV, H_Q, T0, 0, 4096, seed=1003, student_t=True)
+    _run(K, cache, ol, H_KV, H_Q, B, Tq, seed=1003, student_t=True, what="config 3 scaled")
+
+
+def test_prefill_rejects_bad_arguments(K):
+    cache = K.KittyCache(K.u.cfg(2, 8), 1, 512)
+    L = cache.kv_cache[0]
+    z = lambda *s: torch.zeros(*s, dtype=torch.float16, device="cuda")
+    with pytest.raises(ValueError):
+        K.pre(K.u.module(2, 8), z(1, 8, 4, 128), z(1, 2, 5, 128), z(1, 2, 5, 128), L, SC)     # chunk length
+    with pytest.raises(ValueError):
+        K.pre(K.u.module(2, 8), z(1, 8, 4, 128).float(), z(1, 2, 4, 128), z(1, 2, 4, 128), L, SC)
+    with pytest.raises(AssertionError):
+        K.pre(K.u.module(1, 32), z(1, 32, 4, 128), z(1, 1, 4, 128), z(1, 1, 4, 128), L, SC)   # group of 32
+    with pytest.raises(RuntimeError):
+        K.pre(K.u.module(2, 8), z(1, 8, 4, 128).cpu(), z(1, 2, 4, 128), z(1, 2, 4, 128), L, SC)
