@@ -145,6 +145,106 @@ class KittyCache(_HFCache):
             kvcache.PageCount_V += 1
             kvcache.Q_Buffer_Count_V = 0
 
+    def append(self, key_states: torch.Tensor, value_states: torch.Tensor, layer_idx: int = 0) -> None:
+        """Append a chunk of T >= 1 tokens ``[B, H_KV, T, D]`` to a layer in one go.
+
+        An extension (the reference's ``update`` takes one token at a time once the cache holds
+        anything, kitty.py:97-98).  The resulting state is the one T calls of ``update`` +
+        ``quantize_decode`` would leave: same counters, same packed pages bit for bit, same fp16
+        rows in the same slots of the sink, the Q-buffers and the local ring.  Pages that lie
+        entirely inside the chunk are quantized straight from it; only pages that start with
+        rows already buffered go through the Q-buffer.  On an empty layer this is
+        ``update`` + ``quantize_prefill``.
+        """
+        L = self.kv_cache[layer_idx]
+        if key_states.shape != value_states.shape or key_states.dim() != 4:
+            raise ValueError("key_states and value_states must both be [B, H_KV, T, D]")
+        if L.get_total_length() == 0:
+            self.update(key_states, value_states, layer_idx)
+            self.quantize_prefill(layer_idx)
+            return
+        B, T, P = key_states.shape[0], key_states.shape[-2], L.PAGE_SIZE
+        a = min(L.S - L.Sink_Count, T)                  # tokens that still go to the sink
+        n = T - a
+        # capacity first, so that a rejected chunk leaves the layer untouched
+        new_pk = (L.Q_Buffer_Count_K + n) // P
+        lv_after = min(P, L.Local_Count_V + n)
+        evicted = L.Local_Count_V + n - lv_after        # rows leaving the ring for the V Q-buffer
+        new_pv = (L.Q_Buffer_Count_V + evicted) // P
+        if L.PageCount_K + new_pk > L.MAX_PAGE or L.PageCount_V + new_pv > L.MAX_PAGE:
+            raise ValueError(f"appending {T} tokens exceeds max_length={L.MAX_LEN}")
+        with torch.no_grad():
+            if a > 0:
+                L.Sink_Buffer_K[:B, :, L.Sink_Count:L.Sink_Count + a, :].copy_(key_states[:, :, :a, :])
+                L.Sink_Buffer_V[:B, :, L.Sink_Count:L.Sink_Count + a, :].copy_(value_states[:, :, :a, :])
+                L.Sink_Count += a
+            if n == 0:
+                return
+            # K: every new row enters the quantize stream
+            self._push_k(L, key_states, a, T, B)
+            # V: the ring keeps the newest P rows; what it evicts, oldest first, enters the stream:
+            # first rows of the old ring (age order = slots from Write_Offset_Local_V), then the head
+            # of the chunk
+            from_ring = min(evicted, L.Local_Count_V)
+            off = L.Write_Offset_Local_V
+            first = min(from_ring, P - off)
+            self._push_v(L, L.Local_Buffer_V, off, off + first, B)
+            self._push_v(L, L.Local_Buffer_V, 0, from_ring - first, B)
+            from_chunk = evicted - from_ring
+            self._push_v(L, value_states, a, a + from_chunk, B)
+            # the newest rows take the slots single steps would have given them
+            base = L.Local_Count_V if L.Local_Count_V < P else off
+            j = from_chunk
+            while j < n:
+                slot = (base + j) % P
+                run = min(n - j, P - slot)
+                L.Local_Buffer_V[:B, :, slot:slot + run, :].copy_(value_states[:, :, a + j:a + j + run, :])
+                j += run
+            L.Local_Count_V = lv_after
+            L.Write_Offset_Local_V = (off + evicted) % P
+
+    def _push_k(self, L: KVCache_Layer, src: torch.Tensor, lo: int, hi: int, B: int) -> None:
+        """Rows ``src[:, :, lo:hi]`` enter the K quantize stream: whole pages straight from ``src``
+        when the Q-buffer is empty, otherwise through the Q-buffer, flushing it when full."""
+        P = L.PAGE_SIZE
+        while lo < hi:
+            if L.Q_Buffer_Count_K == 0 and hi - lo >= P:
+                pages = (hi - lo) // P
+                quantize_pack_k(src, lo, pages, L.PageTable_K, L.PageCount_K, L.KeyCache, L.KeyCache_metadata, P,
+                                L.D_BOOSTED, select=self.select)
+                L.PageCount_K += pages
+                lo += pages * P
+                continue
+            m = min(P - L.Q_Buffer_Count_K, hi - lo)
+            L.Q_Buffer_K[:B, :, L.Q_Buffer_Count_K:L.Q_Buffer_Count_K + m, :].copy_(src[:, :, lo:lo + m, :])
+            L.Q_Buffer_Count_K += m
+            lo += m
+            if L.Q_Buffer_Count_K == P:
+                quantize_pack_k(L.Q_Buffer_K, 0, 1, L.PageTable_K, L.PageCount_K, L.KeyCache, L.KeyCache_metadata,
+                                P, L.D_BOOSTED, select=self.select)
+                L.PageCount_K += 1
+                L.Q_Buffer_Count_K = 0
+
+    def _push_v(self, L: KVCache_Layer, src: torch.Tensor, lo: int, hi: int, B: int) -> None:
+        """The V side of ``_push_k``."""
+        P = L.PAGE_SIZE
+        while lo < hi:
+            if L.Q_Buffer_Count_V == 0 and hi - lo >= P:
+                pages = (hi - lo) // P
+                quantize_pack_v(src, lo, pages, L.PageTable_V, L.PageCount_V, L.ValueCache, L.ValueCache_metadata, P)
+                L.PageCount_V += pages
+                lo += pages * P
+                continue
+            m = min(P - L.Q_Buffer_Count_V, hi - lo)
+            L.Q_Buffer_V[:B, :, L.Q_Buffer_Count_V:L.Q_Buffer_Count_V + m, :].copy_(src[:, :, lo:lo + m, :])
+            L.Q_Buffer_Count_V += m
+            lo += m
+            if L.Q_Buffer_Count_V == P:
+                quantize_pack_v(L.Q_Buffer_V, 0, 1, L.PageTable_V, L.PageCount_V, L.ValueCache,
+                                L.ValueCache_metadata, P)
+                L.PageCount_V += 1
+                L.Q_Buffer_Count_V = 0
+
     def get_seq_length(self, layer_idx: int = 0) -> int:
         """Number of cached tokens of a layer."""
         return self.kv_cache[layer_idx].get_total_length()

@@ -344,6 +344,18 @@ class OracleLayer:
                 self.Write_Offset_Local_V = (w + 1) % self.PAGE_SIZE
         return False
 
+    def append(self, key_states: np.ndarray, value_states: np.ndarray) -> None:
+        """A chunk of T tokens, by definition T single-token steps of the reference's decode path
+        (update, then quantize_decode: modeling_qwen3.py:225-251); an empty layer takes the
+        reference's prefill path instead, as its update() would (kitty.py:91-95)."""
+        if self.get_total_length() == 0:
+            self.update(key_states, value_states)
+            self.quantize_prefill()
+            return
+        for t in range(key_states.shape[-2]):
+            self.update(key_states[:, :, t:t + 1], value_states[:, :, t:t + 1])
+            self.quantize_decode()
+
     # kitty.py:126-192
     def quantize_prefill(self) -> None:
         if self.key_states is None or self.value_states is None:

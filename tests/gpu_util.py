@@ -21,8 +21,10 @@ def to_dev(a):
     return torch.from_numpy(np.ascontiguousarray(a)).cuda()
 
 
-def layer_bytes_equal(layer, ol: O.OracleLayer):
-    """Bit-exact comparison of every tensor of a layer with the oracle's; returns list of mismatches."""
+def layer_bytes_equal(layer, ol: O.OracleLayer, live_q_rows_only: bool = False):
+    """Bit-exact comparison of every tensor of a layer with the oracle's; returns list of mismatches.
+    ``live_q_rows_only``: compare the Q-buffers up to their fill counts only (rows past the count are
+    stale, and a chunked append legitimately leaves other stale rows than single steps do)."""
     bad = []
 
     def cmp(name, t, a):
@@ -38,8 +40,10 @@ def layer_bytes_equal(layer, ol: O.OracleLayer):
     cmp("ValueCache_metadata", layer.ValueCache_metadata, ol.ValueCache_metadata)
     cmp("Sink_Buffer_K", layer.Sink_Buffer_K, ol.Sink_Buffer_K)
     cmp("Sink_Buffer_V", layer.Sink_Buffer_V, ol.Sink_Buffer_V)
-    cmp("Q_Buffer_K", layer.Q_Buffer_K, ol.Q_Buffer_K)
-    cmp("Q_Buffer_V", layer.Q_Buffer_V, ol.Q_Buffer_V)
+    nk = ol.Q_Buffer_Count_K if live_q_rows_only else ol.PAGE_SIZE
+    nv = ol.Q_Buffer_Count_V if live_q_rows_only else ol.PAGE_SIZE
+    cmp("Q_Buffer_K", layer.Q_Buffer_K[:, :, :nk], ol.Q_Buffer_K[:, :, :nk])
+    cmp("Q_Buffer_V", layer.Q_Buffer_V[:, :, :nv], ol.Q_Buffer_V[:, :, :nv])
     cmp("Local_Buffer_V", layer.Local_Buffer_V, ol.Local_Buffer_V)
     for f in ("Sink_Count", "PageCount_K", "PageCount_V", "Q_Buffer_Count_K", "Q_Buffer_Count_V",
               "Local_Count_V", "Write_Offset_Local_V"):

@@ -175,6 +175,106 @@ def test_config3_scaled_down_student_t(K):
     _run(K, cache, ol, H_KV, H_Q, B, Tq, seed=1003, student_t=True, what="config 3 scaled")
 
 
+@pytest.mark.parametrize("T0,steps,chunks", [(5, 0, [1, 30, 200]), (100, 0, [60, 300]), (32 + 128 * 2 + 96, 7, [25, 256, 131]),
+                                             (0, 0, [50, 500])])
+def test_append_on_device_equals_single_steps(K, T0, steps, chunks):
+    """KittyCache.append: same counters, same packed pages bit for bit, same fp16 rows in the same
+    slots as one update + quantize_decode per token (the oracle's definition)."""
+    B, H_KV, H_Q = 2, 2, 8
+    cache, ol = _state(K, B, H_KV, H_Q, T0, steps, 2048, seed=T0 + 11, student_t=True)
+    k, v = make_kv(B, H_KV, sum(chunks), seed=T0 + 12, student_t=True)
+    kd, vd = K.u.to_dev(k), K.u.to_dev(v)
+    t = 0
+    for c in chunks:
+        cache.append(kd[:, :, t:t + c], vd[:, :, t:t + c], 0)
+        ol.append(k[:, :, t:t + c], v[:, :, t:t + c])
+        t += c
+        assert K.u.layer_bytes_equal(cache.kv_cache[0], ol, live_q_rows_only=True) == []
+    assert cache.get_seq_length(0) == T0 + steps + t
+
+
+def test_chunk_then_append_then_decode(K):
+    """The chunked-prefill call order: attend the chunk over the cache, append it, decode."""
+    B, H_KV, H_Q, T0, Tq = 1, 2, 8, 32 + 128 * 3 + 96, 160
+    cache, ol = _state(K, B, H_KV, H_Q, T0, 0, 2048, seed=21)
+    got, q, kc, vc = _run(K, cache, ol, H_KV, H_Q, B, Tq, seed=21)
+    cache.append(K.u.to_dev(kc), K.u.to_dev(vc), 0)
+    ol.append(kc, vc)
+    assert K.u.layer_bytes_equal(cache.kv_cache[0], ol, live_q_rows_only=True) == []
+    q1 = _q(B, H_Q, 1, 22)
+    out, _ = K.attn(K.u.module(H_KV, H_Q), K.u.to_dev(q1), cache.kv_cache[0], SC, variant=1)
+    want = O.decode_attention(ol, q1, SC, reference_rounding=False, dequant="two")
+    assert np.abs(out.cpu().numpy().astype(np.float64) - want).max() <= ATOL
+
+
+def test_config3_full_size(K):
+    """BASELINE config 3 at its real shape: B=4, 32 Q / 8 KV heads, a 2048-token chunk over a
+    30720-token packed prefix (Student-t keys), then the append of the chunk.  The oracle cannot
+    attend 8192 x 32768 scores per head in seconds, so: (i) sampled query rows of two batch rows
+    are checked in float64 against the dequantized device cache, every cached and chunk token
+    included; (ii) after the append the counters have the closed form, and sampled new pages are
+    bit-exact against the oracle's quantizer."""
+    B, H_KV, H_Q, T0, Tq = 4, 8, 32, 30720, 2048
+    max_len = 32768 + 128
+    gen = torch.Generator(device="cuda").manual_seed(1003)
+    chi = torch.randn(B, H_KV, T0 + Tq, 128, 3, generator=gen, device="cuda").square_().sum(-1).div_(3).sqrt_()
+    k = torch.randn(B, H_KV, T0 + Tq, 128, generator=gen, device="cuda") / chi          # Student-t, nu = 3
+    del chi
+    for h in range(H_KV):
+        ch = torch.randperm(128, generator=torch.Generator().manual_seed(h))[:8]
+        k[:, h, :, ch] *= 10.0
+    k = k.clamp_(-6e4, 6e4).half()
+    v = torch.randn(B, H_KV, T0 + Tq, 128, generator=gen, device="cuda").half()
+    q = torch.randn(B, H_Q, Tq, 128, generator=gen, device="cuda").half()
+    cache = K.KittyCache(K.u.cfg(H_KV, H_Q), B, max_len)
+    cache.update(k[:, :, :T0], v[:, :, :T0], 0)
+    cache.quantize_prefill(0)
+    L = cache.kv_cache[0]
+    assert (L.PageCount_K, L.PageCount_V, L.Q_Buffer_Count_K, L.Q_Buffer_Count_V, L.Local_Count_V) == (239, 238, 96, 96, 128)
+    kc, vc = k[:, :, T0:], v[:, :, T0:]
+    out, _ = K.pre(K.u.module(H_KV, H_Q), q, kc, vc, L, SC)
+    torch.cuda.synchronize()
+    got = out.cpu().numpy().astype(np.float64)
+    assert np.isfinite(got).all()
+    ol = K.u.oracle_from_layer(L, max_len)
+    rows = np.array([0, 1, 63, 64, 127, 128, 1000, 1999, 2047])
+    G = H_Q // H_KV
+    for b in (0, 3):
+        Kd, Vd = O.gather_dense_kv(ol, b, dequant="two")                    # [H_KV, T0, D]
+        Kc = np.concatenate([Kd.astype(np.float64), kc[b].cpu().numpy().astype(np.float64)], axis=1)
+        Vc = np.concatenate([Vd.astype(np.float64), vc[b].cpu().numpy().astype(np.float64)], axis=1)
+        qb = q[b].cpu().numpy().astype(np.float64)
+        for hq in range(H_Q):
+            s = qb[hq, rows] @ Kc[hq // G].T * SC                           # [rows, T0 + Tq]
+            s = np.where(np.arange(T0 + Tq)[None, :] > (T0 + rows)[:, None], -np.inf, s)
+            e = np.exp(s - s.max(axis=1, keepdims=True))
+            want = (e / e.sum(axis=1, keepdims=True)) @ Vc[hq // G]
+            err = np.abs(got[b, rows, hq] - want).max()
+            assert err <= ATOL, f"b={b} hq={hq}: {err:.3e}"
+    # the append: 2048 tokens, 16 K pages and 16 V pages per (b, h), residuals unchanged
+    qk_before = L.Q_Buffer_K.cpu().numpy().copy()
+    cache.append(kc, vc, 0)
+    torch.cuda.synchronize()
+    assert (L.PageCount_K, L.PageCount_V, L.Q_Buffer_Count_K, L.Q_Buffer_Count_V, L.Local_Count_V) == (255, 254, 96, 96, 128)
+    assert cache.get_seq_length(0) == T0 + Tq
+    lay = O.Layout(H_KV=H_KV)
+    kcn = kc.cpu().numpy()
+    KC, KM = L.KeyCache.cpu().numpy(), L.KeyCache_metadata.cpu().numpy()
+    for b, h, page in ((0, 0, 239), (1, 3, 240), (3, 7, 254)):
+        if page == 239:      # the page completed from the 96 buffered rows and the first 32 chunk rows
+            x = np.concatenate([qk_before[b, h, :96], kcn[b, h, :32]], axis=0)
+        else:
+            lo = 32 + (page - 240) * 128
+            x = kcn[b, h, lo:lo + 128]
+        oc = np.zeros((1, lay.k_stride_h), np.uint8)
+        om = np.zeros((1, 1, 128, 2), np.float16)
+        O.quantize_pack_k(x[None, None], 0, 1, np.zeros((1, 1), np.int64), 0, oc, om, 128, 32)
+        pg = b * L.MAX_PAGE + page
+        assert np.array_equal(KC[pg, h * lay.k_stride_h:(h + 1) * lay.k_stride_h], oc[0]), (b, h, page)
+        assert np.array_equal(KM[pg, h].view(np.uint16), om[0, 0].view(np.uint16)), (b, h, page)
+    assert np.array_equal(L.Q_Buffer_K.cpu().numpy()[:, :, :96].view(np.uint16), kcn[:, :, -96:].view(np.uint16))
+
+
 def test_prefill_rejects_bad_arguments(K):
     cache = K.KittyCache(K.u.cfg(2, 8), 1, 512)
     L = cache.kv_cache[0]

@@ -211,3 +211,82 @@ def test_no_cpu_fallback():
     mod = types.SimpleNamespace(num_attention_heads=4, num_key_value_heads=1)
     with pytest.raises(RuntimeError, match="no CPU path"):
         kitty_attention_forward(mod, torch.zeros(1, 4, 1, 128, dtype=torch.float16), cache.kv_cache[0], 0.1)
+
+
+# ---------------------------------------------------------------------------------------------
+# multi-token append: the host logic against T single steps, quantizers played by the oracle
+# ---------------------------------------------------------------------------------------------
+@pytest.fixture()
+def cpu_cache_oracle_quant(monkeypatch):
+    import kitty_amd
+    from kitty_amd.kvcache import kitty as kmod
+
+    def qk(key_states, t_offset, pages, page_table, page_offset, cache, meta, page_size, d_boost, **kw):
+        O.quantize_pack_k(key_states.numpy(), t_offset, pages, page_table.numpy(), page_offset, cache.numpy(),
+                          meta.numpy(), page_size, d_boost)
+
+    def qv(value_states, t_offset, pages, page_table, page_offset, cache, meta, page_size):
+        O.quantize_pack_v(value_states.numpy(), t_offset, pages, page_table.numpy(), page_offset, cache.numpy(),
+                          meta.numpy(), page_size)
+
+    monkeypatch.setattr(kmod, "quantize_pack_k", qk)
+    monkeypatch.setattr(kmod, "quantize_pack_v", qv)
+    cfg = types.SimpleNamespace(num_hidden_layers=1, head_dim=128, num_key_value_heads=1, num_attention_heads=4,
+                                hidden_size=512)
+    return lambda max_len: kitty_amd.KittyCache(cfg, 1, max_len, device="cpu")
+
+
+def _same_state(L, ol):
+    fields = ("Sink_Count", "PageCount_K", "PageCount_V", "Q_Buffer_Count_K", "Q_Buffer_Count_V", "Local_Count_V",
+              "Write_Offset_Local_V")
+    assert [getattr(L, f) for f in fields] == [getattr(ol, f) for f in fields]
+    u16 = lambda a: a.view(np.uint16)
+    for name in ("KeyCache", "ValueCache"):
+        assert np.array_equal(getattr(L, name).numpy(), getattr(ol, name)), name
+    for name in ("KeyCache_metadata", "ValueCache_metadata", "Sink_Buffer_K", "Sink_Buffer_V", "Local_Buffer_V"):
+        assert np.array_equal(u16(getattr(L, name).numpy()), u16(getattr(ol, name))), name
+    # rows past the fill count of a Q-buffer are stale and may differ
+    for name, cnt in (("Q_Buffer_K", ol.Q_Buffer_Count_K), ("Q_Buffer_V", ol.Q_Buffer_Count_V)):
+        assert np.array_equal(u16(getattr(L, name).numpy()[:, :, :cnt]), u16(getattr(ol, name)[:, :, :cnt])), name
+
+
+@pytest.mark.parametrize("T0,chunks", [
+    (5, [1, 3, 30, 200]),                 # sink still filling, chunk straddles sink / ring / Q-buffers
+    (32, [128, 1, 127, 129]),             # exactly the sink
+    (100, [60, 60, 300]),                 # ring fills, then evicts
+    (300, [7, 512, 5]),                   # pages straight from the chunk
+    (32 + 128 * 2 + 96, [32, 256]),       # a flush exactly at the end of a chunk
+    (0, [50, 500]),                       # empty layer: the first chunk is a prefill
+    (417, [1] * 5 + [250]),
+])
+def test_append_equals_single_steps(cpu_cache_oracle_quant, T0, chunks):
+    max_len = 2048
+    cache = cpu_cache_oracle_quant(max_len)
+    ol = O.OracleLayer(1, max_len, 1)
+    k, v = make_kv(1, 1, T0 + sum(chunks), seed=T0 + len(chunks))
+    kt, vt = torch.from_numpy(k), torch.from_numpy(v)
+    if T0:
+        cache.update(kt[:, :, :T0], vt[:, :, :T0], 0)
+        cache.quantize_prefill(0)
+        ol.update(k[:, :, :T0], v[:, :, :T0])
+        ol.quantize_prefill()
+    t = T0
+    for c in chunks:
+        cache.append(kt[:, :, t:t + c], vt[:, :, t:t + c], 0)
+        ol.append(k[:, :, t:t + c], v[:, :, t:t + c])
+        t += c
+        assert cache.get_seq_length(0) == t
+        _same_state(cache.kv_cache[0], ol)
+
+
+def test_append_rejects_overflow_without_side_effects(cpu_cache_oracle_quant):
+    cache = cpu_cache_oracle_quant(512)
+    k, v = make_kv(1, 1, 1000, seed=2)
+    kt, vt = torch.from_numpy(k), torch.from_numpy(v)
+    cache.append(kt[:, :, :300], vt[:, :, :300], 0)
+    before = cache.get_seq_length(0)
+    with pytest.raises(ValueError):
+        cache.append(kt[:, :, 300:], vt[:, :, 300:], 0)
+    assert cache.get_seq_length(0) == before
+    with pytest.raises(ValueError):
+        cache.append(kt[:, :, :3], vt[:, :, :4], 0)
