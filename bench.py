@@ -8,6 +8,9 @@ independent copies of the cache so that every step streams from HBM rather than 
 Infinity Cache.  Prints ONE JSON line.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c1|c0|c4] [--copies N]
+
+``--workload c3`` measures the other kernel family instead (BASELINE.json configs[3]): a 2048-token
+chunk attending a 30720-token packed prefix, bound by the matrix cores, plus the append of the chunk.
 """
 import argparse
 import json
@@ -25,7 +28,11 @@ WORKLOADS = {
     "c1": (16, 32, 8, 32768, "Llama-3.1-8B-shaped decode B=16 32Q/8KV D=128 ctx=32768, 2-bit Kitty KV (configs[1])"),
     "c4": (1, 64, 8, 131072, "long-context decode B=1 64Q/8KV D=128 ctx=131072 (configs[4])"),
 }
+C3 = dict(B=4, H_Q=32, H_KV=8, T0=30720, Tq=2048,
+          desc="chunked prefill B=4 32Q/8KV D=128: 2048-token chunk over a 30720-token packed prefix, "
+               "Student-t(3) keys, then append of the chunk (configs[3])")
 HBM_PEAK_GBPS = 8000.0
+MFMA_F16_PEAK_TFLOPS = 2500.0
 TRAFFIC_FILE = os.path.join(ROOT, "profiles", "decode_split_pmc_traffic.txt")
 
 
@@ -43,7 +50,8 @@ def measured_traffic(workload, splits):
 
 
 def synth_kv(B, H, T, D, seed, device, student_t=False):
-    """K ~ N(0,1) with 8 fixed outlier channels per head scaled x10, V ~ N(0,1); fp16 [B,H,T,D]."""
+    """K ~ N(0,1) (or Student-t, nu=3) with 8 fixed outlier channels per head scaled x10, V ~ N(0,1);
+    fp16 [B,H,T,D]."""
     import torch
     g = torch.Generator(device=device).manual_seed(seed)
     K = torch.empty((B, H, T, D), dtype=torch.float16, device=device)
@@ -53,7 +61,11 @@ def synth_kv(B, H, T, D, seed, device, student_t=False):
     for h in range(H):
         mult[h, 0, torch.randperm(D, generator=pg)[:8].to(device)] = 10.0
     for b in range(B):
-        K[b] = (torch.randn((H, T, D), generator=g, device=device, dtype=torch.float32) * mult).half()
+        x = torch.randn((H, T, D), generator=g, device=device, dtype=torch.float32)
+        if student_t:   # Student-t with 3 degrees of freedom: normal / sqrt(chi2_3 / 3)
+            chi = torch.randn((H, T, D, 3), generator=g, device=device, dtype=torch.float32).square_().sum(-1)
+            x = x / (chi / 3).sqrt_()
+        K[b] = (x * mult).clamp_(-6e4, 6e4).half()
         V[b] = torch.randn((H, T, D), generator=g, device=device, dtype=torch.float32).half()
     return K, V
 
@@ -95,12 +107,90 @@ def cpu_baseline(K_row, V_row, q_row, H_Q, H_KV, B_full, budget_s=20.0):
     }
 
 
+def bench_chunked_prefill(args):
+    """configs[3]: a step = chunked-prefill attention of one layer; the append is timed beside it."""
+    import torch
+    import kitty_amd
+    from kitty_amd import _lib
+    from kitty_amd.kvcache.kernels import kitty_prefill_attention
+    _lib.lib()
+    dev = torch.device("cuda:0")
+    B, H_Q, H_KV, T0, Tq, D = C3["B"], C3["H_Q"], C3["H_KV"], C3["T0"], C3["Tq"], 128
+    cfg = types.SimpleNamespace(num_hidden_layers=1, head_dim=D, num_key_value_heads=H_KV,
+                                num_attention_heads=H_Q, hidden_size=H_Q * D)
+    mod = types.SimpleNamespace(num_attention_heads=H_Q, num_key_value_heads=H_KV)
+    K, V = synth_kv(B, H_KV, T0 + Tq, D, 1003, dev, student_t=True)
+    q = torch.randn((B, H_Q, Tq, D), generator=torch.Generator(device=dev).manual_seed(7), device=dev).half()
+    cache = kitty_amd.KittyCache(cfg, B, T0 + Tq + 256, device=dev)
+    cache.update(K[:, :, :T0], V[:, :, :T0], 0)
+    cache.quantize_prefill(0)
+    L = cache.kv_cache[0]
+    kc, vc = K[:, :, T0:], V[:, :, T0:]
+    scaling = D ** -0.5
+    for _ in range(args.warmup):
+        kitty_prefill_attention(mod, q, kc, vc, L, scaling)
+    torch.cuda.synchronize()
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+    t0 = time.perf_counter()
+    for a, b in ev:
+        a.record()
+        kitty_prefill_attention(mod, q, kc, vc, L, scaling)
+        b.record()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) / args.steps * 1e3
+    kern_ms = sum(a.elapsed_time(b) for a, b in ev) / len(ev)
+    flops = 4.0 * B * H_Q * Tq * (T0 + Tq / 2) * D
+    tflops = flops / (kern_ms * 1e-3) / 1e12
+    # the append: restore the counters after each one so that every repetition does the same work
+    fields = ("Sink_Count", "PageCount_K", "PageCount_V", "Q_Buffer_Count_K", "Q_Buffer_Count_V", "Local_Count_V",
+              "Write_Offset_Local_V")
+    saved = {f: getattr(L, f) for f in fields}
+    app_ms = []
+    for _ in range(5):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        cache.append(kc, vc, 0)
+        e1.record()
+        torch.cuda.synchronize()
+        app_ms.append(e0.elapsed_time(e1))
+        for f, x in saved.items():
+            setattr(L, f, x)
+    result = {
+        "metric": "chunked_prefill_attention_ms_per_step", "value": ms_per_step, "unit": "ms/step", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": False,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f16 operands (pages dequantized to f16), f32 accumulate",
+        "data": "synthetic (seeded Student-t(3) K with 8 outlier channels/head x10, N(0,1) V and Q)",
+        "config": {"workload": C3["desc"], "batch": B, "q_heads": H_Q, "kv_heads": H_KV, "head_dim": D,
+                   "prefix": T0, "chunk": Tq},
+        "roofline": {"bound": "mfma", "achieved": tflops, "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": tflops / MFMA_F16_PEAK_TFLOPS, "traffic": None, "kernel": "prefill_attn_kernel",
+                     "kernel_avg_us": kern_ms * 1e3, "algorithmic_flops_per_launch": flops},
+        "append": {"ms": min(app_ms), "input_bytes": 2 * B * H_KV * Tq * D * 2,
+                   "gbps_in": 2 * B * H_KV * Tq * D * 2 / (min(app_ms) * 1e-3) / 1e9,
+                   "what": "KittyCache.append of the 2048-token chunk (16 K + 16 V pages per head, host logic included)"},
+    }
+    if not args.no_cpu_baseline:
+        import torch.nn.functional as F
+        torch.set_num_threads(min(16, os.cpu_count() or 1))
+        kk, vv = K[:1, :1].float().cpu(), V[:1, :1].float().cpu()
+        G = H_Q // H_KV
+        qq = q[:1, :G].float().cpu()
+        mask = torch.ones(Tq, T0 + Tq, dtype=torch.bool).tril_(T0)
+        t1 = time.perf_counter()
+        F.scaled_dot_product_attention(qq, kk.expand(1, G, -1, -1), vv.expand(1, G, -1, -1), attn_mask=mask, scale=scaling)
+        dt = time.perf_counter() - t1
+        result["cpu_baseline"] = {"value": dt * B * H_KV * 1e3, "unit": "ms/step", "cores": torch.get_num_threads(),
+                                  "kind": "port", "sample": f"dense fp32 causal attention of 1 of {B * H_KV} "
+                                  f"(sequence, KV head) units, {dt:.2f} s, scaled x{B * H_KV}"}
+    print(json.dumps(result))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="c1", choices=sorted(WORKLOADS))
+    ap.add_argument("--workload", default="c1", choices=sorted(WORKLOADS) + ["c3"])
     ap.add_argument("--copies", type=int, default=0, help="independent cache copies to rotate over (0 = auto)")
     ap.add_argument("--splits", type=int, default=0)
     ap.add_argument("--variant", type=int, default=0)
@@ -114,6 +204,8 @@ def main():
               "(no collectives, sharding or multi-rank code exists in this path)", file=sys.stderr)
         sys.exit(2)
 
+    if args.workload == "c3":
+        return bench_chunked_prefill(args)
     import torch
     import kitty_amd
     from kitty_amd import _lib

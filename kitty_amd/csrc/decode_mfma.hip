@@ -16,18 +16,19 @@
 //
 // Codes as operands.  A 32-bit word of a packed plane holds 16 two-bit codes of ONE row (K: one
 // channel, 16 tokens; V: one token, 16 channels) but an MFMA register must hold two consecutive k
-// (K: two channels, V: two tokens) of one row of A.  Lanes n and n^1 each load one word of two
-// neighbouring plane rows, swap them with one DPP move and v_perm the matching 16-bit halves
-// together: X = [8 codes of row r | 8 codes of row r+1].  `X & (3 << 2u | 3 << 2u+16)` is then
+// (K: two channels, V: two tokens) of one row of A: X = [8 codes of row r | 8 codes of row r+1].
+// With the tile in LDS one transposing read (ds_read_b64_tr_b16: a 16-lane block reads 4 plane
+// rows, lane i receives 16-bit piece i of each) delivers two such registers; with the tile in
+// registers lanes n and n^1 each load one word of two neighbouring plane rows, swap them with one
+// DPP move and v_perm the matching 16-bit halves together.  `X & (3 << 2u | 3 << 2u+16)` is then
 // already a valid operand: fp16 SUBNORMALS code * 4^u * 2^-24 (the matrix cores do not flush
 // them), so unpacking costs one v_and_b32 per register and the factor is undone per tile after
 // the contraction.  Codes above bit 9 are reached through X >> 10.
 //
 // Index maps (all bijections chosen so that every load is 64 contiguous bytes per 16 lanes):
-//   K plane word of lane (kg, n) in 256-byte chunk c (= 8 plane rows):   row 2kg + (n&1), word n>>1
-//     -> channel 8c + 2kg + (n&1), tokens 16(n>>1) .. +15; lane n keeps tokens 8n .. 8n+7
-//     -> MFMA tile u (0..7) = tokens {8n + u}; k-slot (kg, 2pi + h) of chunk kc = channel
-//        32kc + 8pi + 2kg + h.
+//   K: lane n keeps tokens 8n .. 8n+7 of every plane row it touches; MFMA tile u (0..7) = tokens
+//     {8n + u}; k-slot (kg, 2pi + h) of the 32-channel chunk kc = channel 32kc + krow(pi, kg) + h
+//     with krow = 16 (pi>>1) + 4kg + 2 (pi&1): the four rows of a transposing read are consecutive.
 //   C[u][j] of lane (kg, n) = token 32kg + 8j + u, column n.
 //   V plane rows are tokens: lane group kg owns rows 32kg .. 32kg+31 (its own tokens), k-chunk j
 //   = rows 32kg + 8j .. +7, d-tile u = channels {8n + u}; O^T[u][j] = channel 32kg + 8j + u.
@@ -45,8 +46,7 @@ constexpr float kLog2e = 1.44269504088896340736f;
 constexpr int kQPad = 136;   // q_nat row length in halves: 128 channels + a zero entry at 128
 
 // A packed K page-head as it sits in LDS after the global->LDS loads: low plane, high plane, slot
-// map (128 bytes, loaded twice), (scale, zero) pairs.  A V page-head: codes (16-byte pieces
-// swizzled, see dma_v) and (scale, zero) pairs.
+// map (128 bytes, loaded twice), (scale, zero) pairs.  A V page-head: codes and (scale, zero) pairs.
 constexpr int kKOffHi = 4096, kKOffIdx = 5120, kKOffMeta = 5376, kKTile = 5888;
 constexpr int kVOffMeta = 4096, kVTile = 4608;
 
@@ -83,6 +83,19 @@ __device__ __forceinline__ uint32_t swap_pair(uint32_t v) {   // value of lane n
   return (uint32_t)__builtin_amdgcn_mov_dpp((int)v, 0xB1 /* quad_perm [1,0,3,2] */, 0xf, 0xf, true);
 }
 __device__ __forceinline__ float xor_lanes(float v, int mask) { return __shfl_xor(v, mask); }
+
+// first plane row (of a 32-row chunk) behind operand register pi of lane group kg
+__device__ __forceinline__ constexpr int krow(int pi, int kg) { return 16 * (pi >> 1) + 4 * kg + 2 * (pi & 1); }
+
+// Transposing LDS read: the 16 lanes of a block address 4 rows x 16 pieces of 16 bits (lane s:
+// row s/4, pieces 4(s%4) ..); lane i receives piece i of the 4 rows = two operand registers.
+typedef short short4v __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ void lds_tr2(const uint8_t* p, uint32_t& r0, uint32_t& r1) {
+  const short4v v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((short4v __attribute__((address_space(3)))*)p);
+  const uint2 u = __builtin_bit_cast(uint2, v);
+  r0 = u.x;
+  r1 = u.y;
+}
 
 // Mask of tile / d-tile u inside X (u < 5) or X >> 10 (u >= 5), and the factor that undoes the
 // subnormal encoding code * 4^u' * 2^-24.
@@ -135,11 +148,11 @@ struct Ctx {
   const kitty_kv_layer* L;
   SeqCounts c;
   int b, h, lane, kg, n;
-  uint32_t lane_off;    // byte offset of this lane's word inside a 256-byte plane chunk
+  uint32_t lane_off;    // register-fed tiles: byte offset of this lane's word relative to plane row krow(pi, 0)
   uint32_t sel;         // v_perm selector merging own / partner halves
   int g;                // query head of this column (n % G)
-  uint32_t kb0;         // LDS: byte offset of this lane's 16-bit piece in plane row 2kg (K tiles)
-  uint32_t vb[4];       // LDS: same for V rows 32kg + 2pi, swizzled (V tiles)
+  uint32_t ktr;         // LDS: this lane's corner of a transposing read of K plane rows 4kg .. 4kg+3
+  uint32_t vtr;         // LDS: same for V rows 32kg .. 32kg+3
   float sc2;            // scaling * log2(e)
   uint32_t qpair[16];   // q[col][32kc + 8pi + 2kg + {0,1}] as an fp16 pair, index 4kc + pi
 };
@@ -155,25 +168,27 @@ struct KRegs {
   uint32_t lo[16], hi[4];
   uint2 meta;
   uint32_t idx2;
-  __device__ __forceinline__ uint32_t x_lo(const Ctx& x, int c) const {
-    return __builtin_amdgcn_perm(swap_pair(lo[c]), lo[c], x.sel);
+  __device__ __forceinline__ void x4_lo(const Ctx& x, int kc, uint32_t (&X)[4]) const {
+#pragma unroll
+    for (int pi = 0; pi < 4; ++pi) X[pi] = __builtin_amdgcn_perm(swap_pair(lo[4 * kc + pi]), lo[4 * kc + pi], x.sel);
   }
-  __device__ __forceinline__ uint32_t x_hi(const Ctx& x, int c) const {
-    return __builtin_amdgcn_perm(swap_pair(hi[c]), hi[c], x.sel);
+  __device__ __forceinline__ void x4_hi(const Ctx& x, uint32_t (&X)[4]) const {
+#pragma unroll
+    for (int pi = 0; pi < 4; ++pi) X[pi] = __builtin_amdgcn_perm(swap_pair(hi[pi]), hi[pi], x.sel);
   }
   __device__ __forceinline__ uint2 meta2(const Ctx&) const { return meta; }
   __device__ __forceinline__ uint32_t idx(const Ctx&) const { return idx2; }
 };
-// KLds: the whole page-head in LDS; the two 16-bit pieces are read where they lie and merged.
+// KLds: the whole page-head in LDS; two transposing reads per 32-row chunk.
 struct KLds {
   const uint8_t* base;
-  __device__ __forceinline__ uint32_t x_lo(const Ctx& x, int c) const {
-    const uint16_t* p = (const uint16_t*)(base + c * 256 + x.kb0);
-    return __builtin_amdgcn_perm(p[16], p[0], 0x05040100u);     // [row 2kg piece | row 2kg+1 piece]
+  __device__ __forceinline__ void x4_lo(const Ctx& x, int kc, uint32_t (&X)[4]) const {
+    lds_tr2(base + kc * 1024 + x.ktr, X[0], X[1]);
+    lds_tr2(base + kc * 1024 + 512 + x.ktr, X[2], X[3]);
   }
-  __device__ __forceinline__ uint32_t x_hi(const Ctx& x, int c) const {
-    const uint16_t* p = (const uint16_t*)(base + kKOffHi + c * 256 + x.kb0);
-    return __builtin_amdgcn_perm(p[16], p[0], 0x05040100u);
+  __device__ __forceinline__ void x4_hi(const Ctx& x, uint32_t (&X)[4]) const {
+    lds_tr2(base + kKOffHi + x.ktr, X[0], X[1]);
+    lds_tr2(base + kKOffHi + 512 + x.ktr, X[2], X[3]);
   }
   __device__ __forceinline__ uint2 meta2(const Ctx& x) const { return *(const uint2*)(base + kKOffMeta + x.lane * 8); }
   __device__ __forceinline__ uint32_t idx(const Ctx& x) const { return *(const uint16_t*)(base + kKOffIdx + 2 * x.lane); }
@@ -186,10 +201,11 @@ __device__ __forceinline__ void k_load_regs(const Ctx& x, int page_index, KRegs&
   const uint8_t* page = L.key_cache + pg * L.key_cache_stride_page + (int64_t)x.h * k_head_bytes(BOOST ? 32 : 0);
   const uint8_t* meta = (const uint8_t*)L.key_meta + pg * L.key_meta_stride_page + (int64_t)x.h * kD * 4;
 #pragma unroll
-  for (int c = 0; c < 16; ++c) kb.lo[c] = *(const uint32_t*)(page + c * 256 + x.lane_off);
+  for (int c = 0; c < 16; ++c)   // register 4kc + pi: plane rows 32kc + krow(pi, kg) + (n&1)
+    kb.lo[c] = *(const uint32_t*)(page + ((c >> 2) * 32 + krow(c & 3, 0)) * kRowBytes + x.lane_off);
   if (BOOST) {
 #pragma unroll
-    for (int c = 0; c < 4; ++c) kb.hi[c] = *(const uint32_t*)(page + kLoBytes + c * 256 + x.lane_off);
+    for (int c = 0; c < 4; ++c) kb.hi[c] = *(const uint32_t*)(page + kLoBytes + krow(c, 0) * kRowBytes + x.lane_off);
     kb.idx2 = *(const uint16_t*)(page + kRowBytes * (kD + 32) + 2 * x.lane);
   }
   kb.meta = *(const uint2*)(meta + x.lane * 8);                          // [s0|z0], [s1|z1]
@@ -230,16 +246,16 @@ __device__ __forceinline__ void dma_k(const Ctx& x, int page_index, uint32_t lds
 }
 
 // Stage the page-head's (scale, zero) pairs and slot map in LDS in the order the operands need:
-// channel pair (2l, 2l+1) of lane l belongs to chunk kc = l/16, pair pi = (l/4)%4, lane group
-// l%4 and is stored at word 16kc + 4kg + pi, so that a lane reads the four pairs of a chunk with
-// one 128-bit LDS read.
+// channel pair (2l, 2l+1) of lane l belongs to chunk kc = l/16; within the chunk 2(l%16) =
+// krow(pi, kg) gives kg = (l/2)%4 and pi = 2((l/8)%2) + l%2.  It is stored at word
+// 16kc + 4kg + pi, so that a lane reads the four pairs of a chunk with one 128-bit LDS read.
 template <bool BOOST, class LDS, class KSRC>
 __device__ __forceinline__ void stage_k_meta(LDS& S, const Ctx& x, const KSRC& kb) {
   const int l = x.lane;
   const uint2 km = kb.meta2(x);
   const uint32_t ss = __builtin_amdgcn_perm(km.y, km.x, 0x05040100u);   // (s0, s1)
   const uint32_t zz = __builtin_amdgcn_perm(km.y, km.x, 0x07060302u);   // (z0, z1)
-  const int pos = (l >> 4) * 16 + (l & 3) * 4 + ((l >> 2) & 3);
+  const int pos = (l >> 4) * 16 + ((l >> 1) & 3) * 4 + 2 * ((l >> 3) & 1) + (l & 1);
   __syncthreads();
   S.ks_perm[pos] = ss;
   S.kz_perm[pos] = zz;
@@ -270,6 +286,7 @@ __device__ __forceinline__ void qk_packed(LDS& S, const Ctx& x, const KSRC& kb, 
     const uint4v sp = *(const uint4v*)&S.ks_perm[kc * 16 + x.kg * 4];
     const uint4v zp = *(const uint4v*)&S.kz_perm[kc * 16 + x.kg * 4];
     uint32_t bh[4], bl[4], bq[4], az[4], X[4], Y[4];
+    kb.x4_lo(x, kc, X);
 #pragma unroll
     for (int pi = 0; pi < 4; ++pi) {
       const half2v qq = as_h2(x.qpair[kc * 4 + pi]), s2 = as_h2(sp[pi]);
@@ -279,19 +296,19 @@ __device__ __forceinline__ void qk_packed(LDS& S, const Ctx& x, const KSRC& kb, 
       bl[pi] = as_u32(lo);
       bq[pi] = x.qpair[kc * 4 + pi];
       az[pi] = zp[pi];
-      X[pi] = kb.x_lo(x, kc * 4 + pi);
       Y[pi] = X[pi] >> 10;
     }
     Cz = mfma16(az, bq, Cz);
     unpack_mfma2(X, Y, bh, bl, C);
   }
   if (BOOST) {
-    // fifth chunk: the 32 high-plane slots; slot 8pi + 2kg + h carries bits 3:2 of the channel
+    // fifth chunk: the 32 high-plane slots; slot krow(pi, kg) + h carries bits 3:2 of the channel
     // inv[slot], weight 4 * scale
     uint32_t bh[4], bl[4], X[4], Y[4];
+    kb.x4_hi(x, X);
 #pragma unroll
     for (int pi = 0; pi < 4; ++pi) {
-      const uint32_t cc = *(const uint16_t*)&S.inv[8 * pi + 2 * x.kg];
+      const uint32_t cc = *(const uint16_t*)&S.inv[krow(pi, x.kg)];
       const uint32_t c0 = cc & 0xffu, c1 = cc >> 8;
       const half2v qq = {S.q_nat[x.g][c0], S.q_nat[x.g][c1]};
       const half2v s2 = {S.ks4_nat[c0], S.ks4_nat[c1]};
@@ -299,7 +316,6 @@ __device__ __forceinline__ void qk_packed(LDS& S, const Ctx& x, const KSRC& kb, 
       const half2v lo = __builtin_elementwise_fma(qq, s2, -hi);
       bh[pi] = as_u32(hi);
       bl[pi] = as_u32(lo);
-      X[pi] = kb.x_hi(x, pi);
       Y[pi] = X[pi] >> 10;
     }
     unpack_mfma2(X, Y, bh, bl, C);
@@ -313,13 +329,13 @@ __device__ __forceinline__ void qk_fp16(const Ctx& x, const uint8_t* rows, int n
   for (int u = 0; u < 8; ++u) {
     C[u] = float4v{0.f, 0.f, 0.f, 0.f};
     const int row = min(8 * x.n + u, nrows_alloc - 1);     // A row of this lane; clamped rows are masked later
-    const uint8_t* rp = rows + (int64_t)row * (kD * 2) + 4 * x.kg;
+    const uint8_t* rp = rows + (int64_t)row * (kD * 2);
 #pragma unroll
     for (int kc = 0; kc < 4; ++kc) {
       uint32_t a[4], bq[4];
 #pragma unroll
       for (int pi = 0; pi < 4; ++pi) {
-        a[pi] = *(const uint32_t*)(rp + (32 * kc + 8 * pi) * 2);   // channels 32kc + 8pi + 2kg + {0,1}
+        a[pi] = *(const uint32_t*)(rp + (32 * kc + krow(pi, x.kg)) * 2);   // channels 32kc + krow + {0,1}
         bq[pi] = x.qpair[kc * 4 + pi];
       }
       C[u] = mfma16(a, bq, C[u]);
@@ -375,16 +391,17 @@ __device__ __forceinline__ void softmax_tile(const Ctx& x, Acc& A, float4v (&C)[
 struct VRegs {
   uint32_t w[16];
   uint2 meta;
-  __device__ __forceinline__ uint32_t xv(const Ctx& x, int j, int pi) const {
-    return __builtin_amdgcn_perm(swap_pair(w[4 * j + pi]), w[4 * j + pi], x.sel);
+  __device__ __forceinline__ void x4(const Ctx& x, int j, uint32_t (&X)[4]) const {
+#pragma unroll
+    for (int pi = 0; pi < 4; ++pi) X[pi] = __builtin_amdgcn_perm(swap_pair(w[4 * j + pi]), w[4 * j + pi], x.sel);
   }
   __device__ __forceinline__ uint2 meta2(const Ctx&) const { return meta; }
 };
 struct VLds {
   const uint8_t* base;
-  __device__ __forceinline__ uint32_t xv(const Ctx& x, int j, int pi) const {
-    const uint16_t* p = (const uint16_t*)(base + j * 256 + x.vb[pi]);
-    return __builtin_amdgcn_perm(p[16], p[0], 0x05040100u);
+  __device__ __forceinline__ void x4(const Ctx& x, int j, uint32_t (&X)[4]) const {   // rows 32kg + 8j + 2pi + {0,1}
+    lds_tr2(base + j * 256 + x.vtr, X[0], X[1]);
+    lds_tr2(base + j * 256 + 128 + x.vtr, X[2], X[3]);
   }
   __device__ __forceinline__ uint2 meta2(const Ctx& x) const { return *(const uint2*)(base + kVOffMeta + x.lane * 8); }
 };
@@ -400,23 +417,20 @@ __device__ __forceinline__ void v_load_regs(const Ctx& x, int page_index, VRegs&
   vb.meta = *(const uint2*)(meta + x.lane * 8);                                        // tokens 2l, 2l+1
 }
 
-// Global -> LDS loads of one V page-head.  Lane group kg reads rows 32kg .. 32kg+31, i.e. the
-// four groups would hit the same LDS banks 1 KB apart; so instruction q (which fills LDS bytes
-// 1024q ..) fetches its 16-byte pieces in the order lane ^ 4q, which rotates the 64-byte windows
-// of the four groups apart (see Ctx::vb for the matching read offsets).
+// Global -> LDS loads of one V page-head, byte for byte.
 __device__ __forceinline__ void dma_v(const Ctx& x, int page_index, uint32_t lds) {
   const kitty_kv_layer& L = *x.L;
   const int64_t pg = L.page_table_v[(int64_t)x.b * L.page_table_v_stride_b + page_index];
   const uint8_t* page = L.value_cache + pg * L.value_cache_stride_page + (int64_t)x.h * kVBytes;
   const uint8_t* meta = (const uint8_t*)L.value_meta + pg * L.value_meta_stride_page + (int64_t)x.h * kPage * 4;
-  const uint32_t o0 = x.lane * 16, o1 = (x.lane ^ 4) * 16, o2 = (x.lane ^ 8) * 16, o3 = (x.lane ^ 12) * 16;
+  const uint32_t off16 = x.lane * 16;
   asm volatile(
-      "s_mov_b32 m0, %5\n\t"
-      "global_load_lds_dwordx4 %0, %4\n\t"
-      "global_load_lds_dwordx4 %1, %4 offset:1024\n\t"
-      "global_load_lds_dwordx4 %2, %4 offset:2048\n\t"
-      "global_load_lds_dwordx4 %3, %4 offset:3072"
-      :: "v"(o0), "v"(o1), "v"(o2), "v"(o3), "s"(page), "s"(lds) : "memory", "m0");
+      "s_mov_b32 m0, %2\n\t"
+      "global_load_lds_dwordx4 %0, %1\n\t"
+      "global_load_lds_dwordx4 %0, %1 offset:1024\n\t"
+      "global_load_lds_dwordx4 %0, %1 offset:2048\n\t"
+      "global_load_lds_dwordx4 %0, %1 offset:3072"
+      :: "v"(off16), "s"(page), "s"(lds) : "memory", "m0");
   const uint32_t off4 = x.lane * 4;
   asm volatile(
       "s_mov_b32 m0, %2\n\t"
@@ -441,13 +455,13 @@ __device__ __forceinline__ void pv_packed(LDS& S, const Ctx& x, float4v (&out)[8
     const uint4v sp = *(const uint4v*)&S.vs_nat[16 * x.kg + 4 * j];
     const uint4v zr = *(const uint4v*)&lz_rows[16 * x.kg + 4 * j];
     uint32_t bp[4], p16[4], alz[4], X[4], Y[4];
+    vb.x4(x, j, X);
 #pragma unroll
     for (int pi = 0; pi < 4; ++pi) {
       const half2v p2 = {(_Float16)P[2 * pi][j], (_Float16)P[2 * pi + 1][j]};   // tokens 32kg + 8j + 2pi + {0,1}
       p16[pi] = as_u32(p2);
       alz[pi] = zr[pi];
       bp[pi] = as_u32(p2 * as_h2(sp[pi]));
-      X[pi] = vb.xv(x, j, pi);
       Y[pi] = X[pi] >> 10;
     }
     lz = mfma16(alz, p16, lz);
@@ -523,21 +537,20 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(kitty_kv_layer L, co
   x.kg = x.lane >> 4;
   x.n = x.lane & 15;
   x.c = load_counts(L, x.b);
-  x.lane_off = (2 * x.kg + (x.n & 1)) * kRowBytes + (x.n >> 1) * 4;
+  x.lane_off = (4 * x.kg + (x.n & 1)) * kRowBytes + (x.n >> 1) * 4;
   x.sel = (x.n & 1) ? 0x03020706u : 0x05040100u;
   x.sc2 = scaling * kLog2e;
   const int G = H_Q / L.H_KV;
   x.g = x.n % G;
-  x.kb0 = x.kg * 64 + 2 * x.n;
-#pragma unroll
-  for (int pi = 0; pi < 4; ++pi) x.vb[pi] = x.kg * 1024 + ((pi ^ x.kg) * 64) + 2 * x.n;
+  x.ktr = (4 * x.kg + (x.n >> 2)) * kRowBytes + (x.n & 3) * 8;
+  x.vtr = (32 * x.kg + (x.n >> 2)) * kRowBytes + (x.n & 3) * 8;
 
   // q of this column: operand-order pairs in registers, natural order in LDS for the slot gather
   const __half* qrow = q + ((int64_t)x.b * H_Q + (int64_t)x.h * G + x.g) * kD;
 #pragma unroll
   for (int kc = 0; kc < 4; ++kc)
 #pragma unroll
-    for (int pi = 0; pi < 4; ++pi) x.qpair[kc * 4 + pi] = *(const uint32_t*)(qrow + 32 * kc + 8 * pi + 2 * x.kg);
+    for (int pi = 0; pi < 4; ++pi) x.qpair[kc * 4 + pi] = *(const uint32_t*)(qrow + 32 * kc + krow(pi, x.kg));
   if (x.n < G) {   // one copy per head
     const uint4* src = (const uint4*)(qrow + 32 * x.kg);
     uint4* dst = (uint4*)&S.q_nat[x.g][32 * x.kg];
