@@ -34,6 +34,11 @@
 //   = rows 32kg + 8j .. +7, d-tile u = channels {8n + u}; O^T[u][j] = channel 32kg + 8j + u.
 #include "decode_common.h"
 
+// Wave priority while a phase is dominated by matrix instructions / by vector instructions: the
+// wave that feeds the matrix pipe wins arbitration, the other one fills the gaps (worth ~2 %).
+#define KITTY_PRIO_MFMA 2
+#define KITTY_PRIO_VALU 0
+
 namespace kitty {
 namespace {
 
@@ -83,6 +88,10 @@ __device__ __forceinline__ uint32_t swap_pair(uint32_t v) {   // value of lane n
   return (uint32_t)__builtin_amdgcn_mov_dpp((int)v, 0xB1 /* quad_perm [1,0,3,2] */, 0xf, 0xf, true);
 }
 __device__ __forceinline__ float xor_lanes(float v, int mask) { return __shfl_xor(v, mask); }
+
+// The workgroup is one wavefront, and the LDS unit executes a wavefront's instructions in order:
+// a write followed by a read needs no hardware wait, only the compiler must keep the order.
+__device__ __forceinline__ void wave_lds_fence() { asm volatile("" ::: "memory"); }
 
 // first plane row (of a 32-row chunk) behind operand register pi of lane group kg
 __device__ __forceinline__ constexpr int krow(int pi, int kg) { return 16 * (pi >> 1) + 4 * kg + 2 * (pi & 1); }
@@ -256,20 +265,20 @@ __device__ __forceinline__ void stage_k_meta(LDS& S, const Ctx& x, const KSRC& k
   const uint32_t ss = __builtin_amdgcn_perm(km.y, km.x, 0x05040100u);   // (s0, s1)
   const uint32_t zz = __builtin_amdgcn_perm(km.y, km.x, 0x07060302u);   // (z0, z1)
   const int pos = (l >> 4) * 16 + ((l >> 1) & 3) * 4 + 2 * ((l >> 3) & 1) + (l & 1);
-  __syncthreads();
+  wave_lds_fence();
   S.ks_perm[pos] = ss;
   S.kz_perm[pos] = zz;
   if (BOOST) {
     const half2v four = {(_Float16)4.0f, (_Float16)4.0f};
     ((uint32_t*)S.ks4_nat)[l] = as_u32(as_h2(ss) * four);
     if (l < 8) ((uint32_t*)S.inv)[l] = 0x80808080u;
-    __syncthreads();
+    wave_lds_fence();
     const uint32_t ib = kb.idx(x);
     const uint32_t i0 = ib & 0xffu, i1 = ib >> 8;
     if (i0 < 32) S.inv[i0] = (uint8_t)(2 * l);
     if (i1 < 32) S.inv[i1] = (uint8_t)(2 * l + 1);
   }
-  __syncthreads();
+  wave_lds_fence();
 }
 
 // logits of one packed K page: C[u][j] = sum_ch code * q * scale, still in subnormal units
@@ -443,10 +452,10 @@ template <class LDS, class VSRC>
 __device__ __forceinline__ void pv_packed(LDS& S, const Ctx& x, float4v (&out)[8], float4v& lz, const VSRC& vb,
                                           const float4v (&P)[8]) {
   const uint2 vm = vb.meta2(x);
-  __syncthreads();
+  wave_lds_fence();
   S.vs_nat[x.lane] = __builtin_amdgcn_perm(vm.y, vm.x, 0x05040100u);
   S.vz_nat[x.lane] = __builtin_amdgcn_perm(vm.y, vm.x, 0x07060302u);
-  __syncthreads();
+  wave_lds_fence();
   // sum p and sum p*zero_v ride along as one more A tile: even rows are ones, odd rows the zero
   // points, so row 0 of the product is the column's sum of p and row 1 its sum of p * zero_v
   const uint32_t* lz_rows = (x.n & 1) ? S.vz_nat : S.ones;
@@ -560,7 +569,7 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(kitty_kv_layer L, co
   }
   if (x.lane == 0) S.ks4_nat[128] = (_Float16)0.0f;
   S.ones[x.lane] = 0x3C003C00u;
-  __syncthreads();
+  wave_lds_fence();
 
   Acc A;
 #pragma unroll
@@ -605,11 +614,14 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(kitty_kv_layer L, co
         float cz;
         const int buf = (i - t0) & 1;
         if (i == t0) wait_vmcnt<nK + kDmaV>(); else wait_vmcnt<nK + 2 * kDmaV>();
+        __builtin_amdgcn_s_setprio(KITTY_PRIO_MFMA);
         qk_packed<BOOST>(S, x, KLds{S.kbuf[buf]}, C, cz);
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
         dma_k<BOOST>(x, min(i + 2, t1 - 1), buf ? lk1 : lk0);
+        __builtin_amdgcn_s_setprio(KITTY_PRIO_VALU);
         softmax_tile<true>(x, A, C, cz, kPage);
         wait_vmcnt<nK>();
+        __builtin_amdgcn_s_setprio(KITTY_PRIO_MFMA);
         pv_packed(S, x, A.out, A.lz, VLds{S.vbuf}, C);
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
         dma_v(x, min(i + 1, t1 - 1), lv);
