@@ -15,12 +15,6 @@ using namespace kitty;
 
 namespace {
 
-// |x| * 2^24 of an fp16 bit pattern as an exact integer (fits 41 bits for finite x).
-__device__ inline uint64_t abs_fixed(uint16_t bits) {
-  uint32_t e = (bits >> 10) & 31u, m = bits & 1023u;
-  return e == 0 ? (uint64_t)m : ((uint64_t)(1024u + m) << (e - 1));
-}
-
 // fp16 bit pattern of (S * 2^-31) rounded to nearest even, S = sum over 128 tokens of |x| * 2^24,
 // i.e. the mean of |x| rounded once.  Positive fp16 patterns order like their values.
 __device__ inline uint16_t mean_abs_fp16_bits(uint64_t S) {
@@ -48,6 +42,43 @@ __device__ inline uint16_t mean_abs_fp16_bits(uint64_t S) {
 
 __device__ inline float h2f(uint16_t bits) { return __half2float(__ushort_as_half(bits)); }
 
+// IEEE fp32 division by a divisor that is shared by a whole group.  This is the correctly rounded
+// sequence the compiler emits for `/` (reciprocal, one Newton step, quotient, two residual
+// corrections) without its range scaling and special-case fix-up, which cannot trigger here: the
+// divisor is a scale in [1e-6, 4.4e4], the dividend x - min is 0 or in [2^-24, 1.4e5].  The
+// reciprocal part depends on the divisor only and is computed once per group.  Bit-identical to
+// `/` on that domain except that -0 / d gives +0, which the + 0.5 that follows erases.
+struct Divisor {
+  float d, r;
+};
+__device__ __forceinline__ Divisor make_divisor(float d) {
+  float r = __builtin_amdgcn_rcpf(d);
+  const float e = __builtin_fmaf(-d, r, 1.0f);
+  r = __builtin_fmaf(e, r, r);
+  return {d, r};
+}
+__device__ __forceinline__ float div_by(float n, Divisor k) {
+  float q = n * k.r;
+  float rem = __builtin_fmaf(-k.d, q, n);
+  q = __builtin_fmaf(rem, k.r, q);
+  rem = __builtin_fmaf(-k.d, q, n);
+  return __builtin_fmaf(rem, k.r, q);
+}
+// floor(min(x / scale + 0.5, qmax + 0.5)) as a float: the code.  x >= 0, so the lower clamp of
+// the reference never acts, and clamping before the floor gives the same integer.
+__device__ __forceinline__ float code_of(float x_minus_min, Divisor k, float qlim) {
+  return __builtin_floorf(fminf(div_by(x_minus_min, k) + 0.5f, qlim));
+}
+// Bits {1,0} (SHIFT = 0) or {3,2} (SHIFT = 2) of the 8 nibbles of n, packed into 16 bits.
+template <int SHIFT>
+__device__ __forceinline__ uint32_t gather_fields(uint32_t n) {
+  uint32_t x = SHIFT ? (n >> SHIFT) : n;
+  x = ((x >> 2) & 0x0C0C0C0Cu) | (x & ~0x0C0C0C0Cu);   // nibble pairs -> low nibble of each byte
+  x = ((x >> 4) & 0x00F000F0u) | (x & ~0x00F000F0u);   // byte pairs -> low byte of each half
+  x = ((x >> 8) & 0x0000FF00u) | (x & ~0x0000FF00u);   // halves -> low half
+  return x & 0xffffu;
+}
+
 // MODE 0: slot map given.  MODE 1: selection fused, then quantize.  MODE 2: selection only.
 template <int MODE>
 __global__ __launch_bounds__(256) void quant_pack_k_kernel(
@@ -64,8 +95,8 @@ __global__ __launch_bounds__(256) void quant_pack_k_kernel(
 
   __shared__ float s_pmin[16][kD];
   __shared__ float s_pmax[16][kD];
-  __shared__ uint64_t s_psum[MODE == 0 ? 1 : 16][kD];
-  __shared__ float s_scale[kD], s_min[kD], s_qmax[kD];
+  __shared__ double s_psum[MODE == 0 ? 1 : 16][kD];
+  __shared__ float4 s_q[kD];   // per channel: min, scale, refined reciprocal of the scale, qmax + 0.5
   __shared__ uint16_t s_score[kD];
   __shared__ __attribute__((aligned(16))) uint8_t s_idx[kD];
   __shared__ __attribute__((aligned(16))) uint16_t s_lo[kD * 16];
@@ -76,19 +107,23 @@ __global__ __launch_bounds__(256) void quant_pack_k_kernel(
 #pragma unroll
   for (int r = 0; r < 8; ++r) rows[r] = *(const uint4*)(src + (int64_t)r * stride_t);
 
-  // per-channel partial min / max (/ sum of |x|) over this thread's 8 tokens
+  // this thread's 8 tokens x 8 channels as floats, and per channel the partial min / max (/ sum
+  // of |x|: exact in fp64, every term is a multiple of 2^-24 below 2^16)
+  float xs[8][8];   // [channel j][token r]
 #pragma unroll
   for (int j = 0; j < 8; ++j) {
-    float mn = INFINITY, mx = -INFINITY;
-    uint64_t sum = 0;
 #pragma unroll
     for (int r = 0; r < 8; ++r) {
       const uint32_t w = ((const uint32_t*)&rows[r])[j >> 1];
-      const uint16_t bits = (j & 1) ? (uint16_t)(w >> 16) : (uint16_t)(w & 0xffffu);
-      const float x = h2f(bits);
-      mn = fminf(mn, x);
-      mx = fmaxf(mx, x);
-      if (MODE != 0) sum += abs_fixed(bits);
+      xs[j][r] = h2f((j & 1) ? (uint16_t)(w >> 16) : (uint16_t)(w & 0xffffu));
+    }
+    float mn = xs[j][0], mx = xs[j][0];
+    double sum = 0.0;
+#pragma unroll
+    for (int r = 0; r < 8; ++r) {
+      mn = fminf(mn, xs[j][r]);
+      mx = fmaxf(mx, xs[j][r]);
+      if (MODE != 0) sum += (double)fabsf(xs[j][r]);
     }
     s_pmin[tg][c8 * 8 + j] = mn;
     s_pmax[tg][c8 * 8 + j] = mx;
@@ -103,10 +138,11 @@ __global__ __launch_bounds__(256) void quant_pack_k_kernel(
     for (int i = 1; i < 16; ++i) { mn = fminf(mn, s_pmin[i][tid]); mx = fmaxf(mx, s_pmax[i][tid]); }
     ch_min = mn; ch_max = mx;
     if (MODE != 0) {
-      uint64_t sum = 0;
+      double sum = 0.0;
 #pragma unroll
       for (int i = 0; i < 16; ++i) sum += s_psum[i][tid];
-      s_score[tid] = mean_abs_fp16_bits(sum);
+      // an integer below 2^47 (or inf / nan for non-finite inputs, which saturate)
+      s_score[tid] = mean_abs_fp16_bits(sum < 1.8e19 ? (uint64_t)(sum * 16777216.0) : ~0ull);
     } else {
       s_idx[tid] = slot_map_in[(((int64_t)b * H + h) * pages + p) * kD + tid];
     }
@@ -138,9 +174,8 @@ __global__ __launch_bounds__(256) void quant_pack_k_kernel(
     const float qmax = boosted ? 15.0f : 3.0f;
     float scale = (ch_max - ch_min) / qmax;
     scale = scale < 1e-6f ? 1e-6f : scale;
-    s_scale[tid] = scale;
-    s_min[tid] = ch_min;
-    s_qmax[tid] = qmax;
+    const Divisor k = make_divisor(scale);
+    s_q[tid] = float4{ch_min, k.d, k.r, qmax + 0.5f};
     __half2 m2 = __halves2half2(__float2half_rn(scale), __float2half_rn(ch_min));
     *(__half2*)(meta + pg * meta_stride_page + ((int64_t)h * kD + tid) * 4) = m2;
   }
@@ -149,21 +184,18 @@ __global__ __launch_bounds__(256) void quant_pack_k_kernel(
 #pragma unroll
   for (int j = 0; j < 8; ++j) {
     const int d = c8 * 8 + j;
-    const float scale = s_scale[d], mn = s_min[d], qmax = s_qmax[d];
-    uint32_t lo = 0, hi = 0;
+    const float4 qp = s_q[d];
+    const Divisor k = {qp.y, qp.z};
+    // the 8 codes (0..15) as one word of nibbles, built in floating point (exact: 16 bits per half)
+    float c[8];
 #pragma unroll
-    for (int r = 0; r < 8; ++r) {
-      const uint32_t w = ((const uint32_t*)&rows[r])[j >> 1];
-      const uint16_t bits = (j & 1) ? (uint16_t)(w >> 16) : (uint16_t)(w & 0xffffu);
-      const float xf = (h2f(bits) - mn) / scale;
-      const float q = fminf(fmaxf(floorf(xf + 0.5f), 0.0f), qmax);
-      const uint32_t code = (uint32_t)q;
-      lo |= (code & 3u) << (2 * r);
-      hi |= (code >> 2) << (2 * r);
-    }
-    s_lo[d * 16 + tg] = (uint16_t)lo;
+    for (int r = 0; r < 8; ++r) c[r] = code_of(xs[j][r] - qp.x, k, qp.w);
+    const float h0 = __builtin_fmaf(__builtin_fmaf(__builtin_fmaf(c[3], 16.f, c[2]), 16.f, c[1]), 16.f, c[0]);
+    const float h1 = __builtin_fmaf(__builtin_fmaf(__builtin_fmaf(c[7], 16.f, c[6]), 16.f, c[5]), 16.f, c[4]);
+    const uint32_t nib = (uint32_t)h0 | ((uint32_t)h1 << 16);
+    s_lo[d * 16 + tg] = (uint16_t)gather_fields<0>(nib);
     const uint8_t slot = s_idx[d];
-    if (slot < d_boost) *(uint16_t*)(dst + kLoBytes + slot * kRowBytes + tg * 2) = (uint16_t)hi;
+    if (slot < d_boost) *(uint16_t*)(dst + kLoBytes + slot * kRowBytes + tg * 2) = (uint16_t)gather_fields<2>(nib);
   }
   __syncthreads();
   ((uint4*)dst)[tid] = ((const uint4*)s_lo)[tid];
@@ -208,12 +240,15 @@ __global__ __launch_bounds__(256) void quant_pack_v_kernel(
     }
     float scale = (mx - mn) / 3.0f;
     scale = scale < 1e-6f ? 1e-6f : scale;
-    uint32_t packed = 0;
+    const Divisor kd = make_divisor(scale);
+    // 16 codes (0..3), 2 bits each, built in floating point in two exact 16-bit halves
+    float h0 = 0.f, h1 = 0.f;
 #pragma unroll
-    for (int k = 0; k < 16; ++k) {
-      const float q = fminf(fmaxf(floorf((x[k] - mn) / scale + 0.5f), 0.0f), 3.0f);
-      packed |= (uint32_t)q << (2 * k);
+    for (int k = 7; k >= 0; --k) {
+      h0 = __builtin_fmaf(h0, 4.f, code_of(x[k] - mn, kd, 3.5f));
+      h1 = __builtin_fmaf(h1, 4.f, code_of(x[8 + k] - mn, kd, 3.5f));
     }
+    const uint32_t packed = (uint32_t)h0 | ((uint32_t)h1 << 16);
     *(uint32_t*)(dst + t * kRowBytes + cg * 4) = packed;
     if (cg == 0) *(__half2*)(mdst + t * 4) = __halves2half2(__float2half_rn(scale), __float2half_rn(mn));
   }
