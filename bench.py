@@ -7,7 +7,7 @@ heads, head_dim 128, batch 16, 32k context (BASELINE.json configs[1]).  Steps ro
 independent copies of the cache so that every step streams from HBM rather than from the 256 MB
 Infinity Cache.  Prints ONE JSON line.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c1|c0|c4] [--copies N]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c1|c0|c2|c4] [--copies N]
 
 ``--workload c3`` measures the other kernel family instead (BASELINE.json configs[3]): a 2048-token
 chunk attending a 30720-token packed prefix, bound by the matrix cores, plus the append of the chunk.
@@ -27,6 +27,8 @@ WORKLOADS = {
     "c0": (1, 32, 8, 4096, "decode B=1 32Q/8KV D=128 ctx=4096 (configs[0])"),
     "c1": (16, 32, 8, 32768, "Llama-3.1-8B-shaped decode B=16 32Q/8KV D=128 ctx=32768, 2-bit Kitty KV (configs[1])"),
     "c4": (1, 64, 8, 131072, "long-context decode B=1 64Q/8KV D=128 ctx=131072 (configs[4])"),
+    # per-sequence contexts uniform in [1k, 16k] and residual fill uniform in [0, 128): T below is the allocation
+    "c2": (64, 32, 8, 16543, "Qwen3-8B-shaped ragged decode B=64 32Q/8KV D=128 ctx~U[1k,16k] (configs[2])"),
 }
 C3 = dict(B=4, H_Q=32, H_KV=8, T0=30720, Tq=2048,
           desc="chunked prefill B=4 32Q/8KV D=128: 2048-token chunk over a 30720-token packed prefix, "
@@ -223,7 +225,21 @@ def main():
     probe = kitty_amd.KittyCache(cfg, B, max_len, device=dev)
     probe.update(K, V, 0)
     probe.quantize_prefill(0)
-    total_bytes, packed_bytes = algorithmic_bytes(B, H_Q, H_KV, probe.kv_cache[0])
+    seq_counts = None
+    if args.workload == "c2":
+        import numpy as np
+        rng = np.random.default_rng(1002)
+        rows = []
+        for _ in range(B):
+            Ti, Ri = int(rng.integers(1024, 16385)), int(rng.integers(0, 128))
+            pk = (Ti - 32 - Ri) // 128
+            rows.append([32, pk, Ri, pk - 1, Ri, 128, int(rng.integers(0, 128)), 0])
+        seq_counts = torch.tensor(rows, dtype=torch.int32, device=dev)
+        total_bytes = sum(H_KV * (5760 * r[1] + 4608 * r[3] + 256 * (2 * r[0] + r[2] + r[4] + r[5])) + 2 * H_Q * 128 * 2
+                          for r in rows)
+        packed_bytes = sum(H_KV * (5760 * r[1] + 4608 * r[3]) for r in rows)
+    else:
+        total_bytes, packed_bytes = algorithmic_bytes(B, H_Q, H_KV, probe.kv_cache[0])
     copies = args.copies or max(2, -(-3 * 256 * 2 ** 20 // total_bytes))      # > 3x the Infinity Cache
     caches = [probe]
     quant_ms = []
@@ -246,10 +262,13 @@ def main():
     q = torch.randn((B, H_Q, 1, D), generator=torch.Generator(device=dev).manual_seed(7), device=dev,
                     dtype=torch.float32).half()
     out = torch.empty((B, 1, H_Q, D), dtype=torch.float16, device=dev)
-    max_tiles = 1 + (T - L0.Sink_Count + 127) // 128
+    max_tiles = (2 + L0.MAX_PAGE) if seq_counts is not None else 1 + (T - L0.Sink_Count + 127) // 128
     splits = args.splits or lib.kitty_decode_attn_default_splits(B, H_KV, max_tiles)
     ws_bytes = lib.kitty_decode_attn_workspace_bytes(B, H_Q, D, splits)
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    if seq_counts is not None:
+        for c in caches:
+            c.kv_cache[0].seq_counts = seq_counts
     descs = [c.kv_cache[0].descriptor() for c in caches]
     stream = torch.cuda.current_stream(dev).cuda_stream
     scaling = D ** -0.5

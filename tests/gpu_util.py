@@ -65,3 +65,26 @@ def oracle_from_layer(layer, max_len) -> O.OracleLayer:
               "Local_Count_V", "Write_Offset_Local_V"):
         setattr(ol, f, getattr(layer, f))
     return ol
+
+
+def oracle_head_view(layer, b: int, h: int, max_len: int, counts=None) -> O.OracleLayer:
+    """OracleLayer (batch 1, one KV head) holding a copy of row ``b``, head ``h`` of a device layer
+    whose page table is the identity; ``counts`` = (sink, pk, rk, pv, rv, lv, off) overrides the
+    layer's counters (per-sequence occupancy)."""
+    ol = O.OracleLayer(1, max_len, 1)
+    lay = O.Layout(H_KV=layer.H_KV)
+    mp = layer.MAX_PAGE
+    assert ol.MAX_PAGE == mp
+    rows = slice(b * mp, (b + 1) * mp)
+    ol.KeyCache = layer.KeyCache[rows, h * lay.k_stride_h:(h + 1) * lay.k_stride_h].cpu().numpy().copy()
+    ol.ValueCache = layer.ValueCache[rows, h * lay.v_stride_h:(h + 1) * lay.v_stride_h].cpu().numpy().copy()
+    ol.KeyCache_metadata = layer.KeyCache_metadata[rows, h:h + 1].cpu().numpy().copy()
+    ol.ValueCache_metadata = layer.ValueCache_metadata[rows, h:h + 1].cpu().numpy().copy()
+    for name in ("Sink_Buffer_K", "Sink_Buffer_V", "Q_Buffer_K", "Q_Buffer_V", "Local_Buffer_V"):
+        setattr(ol, name, getattr(layer, name)[b:b + 1, h:h + 1].cpu().numpy().copy())
+    fields = ("Sink_Count", "PageCount_K", "Q_Buffer_Count_K", "PageCount_V", "Q_Buffer_Count_V", "Local_Count_V",
+              "Write_Offset_Local_V")
+    vals = counts if counts is not None else [getattr(layer, f) for f in fields]
+    for f, v in zip(fields, vals):
+        setattr(ol, f, int(v))
+    return ol
