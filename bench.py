@@ -264,6 +264,8 @@ def main():
     out = torch.empty((B, 1, H_Q, D), dtype=torch.float16, device=dev)
     max_tiles = (2 + L0.MAX_PAGE) if seq_counts is not None else 1 + (T - L0.Sink_Count + 127) // 128
     splits = args.splits or lib.kitty_decode_attn_default_splits(B, H_KV, max_tiles)
+    if not args.splits and seq_counts is not None and splits < 12:
+        splits = 12          # the library's rule for batches with per-sequence lengths
     ws_bytes = lib.kitty_decode_attn_workspace_bytes(B, H_Q, D, splits)
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
     if seq_counts is not None:

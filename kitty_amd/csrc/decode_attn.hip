@@ -23,13 +23,15 @@ extern "C" size_t kitty_decode_attn_workspace_bytes(int B, int H_Q, int D, int n
   return ws_total_bytes(B, H_Q, num_splits);
 }
 
-// Enough workgroups to cover every SIMD of the 256 CUs a few times over, never more splits than
-// there are tiles.
+// Enough workgroups to cover every SIMD of the 256 CUs twice over, but no body split with fewer
+// than 4 tiles (a wave's fixed cost is about one tile's worth); three more for the sink and the
+// tiles with fp16 rows when the body splits are short.
 extern "C" int kitty_decode_attn_default_splits(int B, int H_KV, int max_tiles) {
   if (B <= 0 || H_KV <= 0 || max_tiles <= 0) return 1;
   const int units = B * H_KV;
   int s = (2048 + units - 1) / units;
-  if (s > max_tiles) s = max_tiles;
+  const int by_tiles = (max_tiles + 3) / 4 + 3;
+  if (s > by_tiles) s = by_tiles;
   if (s > 512) s = 512;
   return s < 1 ? 1 : s;
 }
@@ -130,7 +132,11 @@ extern "C" int kitty_decode_attn(const kitty_kv_layer* layer, const void* q, int
                                  void* stream) {
   int max_tiles = 0;
   if (int rc = check_layer(layer, q, B, H_Q, &max_tiles)) return rc;
-  if (num_splits <= 0) num_splits = kitty_decode_attn_default_splits(B, layer->H_KV, max_tiles);
+  if (num_splits <= 0) {
+    num_splits = kitty_decode_attn_default_splits(B, layer->H_KV, max_tiles);
+    // sequences of different lengths: more, shorter splits even out the load
+    if (layer->seq_counts && num_splits < 12 && max_tiles >= 48) num_splits = 12;
+  }
   if (int rc = kitty_decode_attn_split(layer, q, B, H_Q, scaling, workspace, workspace_bytes, num_splits, variant,
                                        stream))
     return rc;

@@ -579,20 +579,30 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(kitty_kv_layer L, co
   A.first = true;
   A.true_units = false;
 
-  // Tiles with both sides packed are shared by all splits but the last, which takes the rest
-  // (tiles with fp16 rows on either side, and the sink); a single split takes everything.
+  // Work of one (batch row, kv head): the tiles with both sides packed ("body"), and the slow rest
+  // ("tail": the sink, and the one or two tiles with fp16 rows on either side).  The tail takes the
+  // FIRST splits, so that its long-latency waves start with the launch and run beside the body: one
+  // split when a body split is long enough to hide it (12 tiles or more), else three (sink / first
+  // tail tile / the others).  The remaining splits share the body evenly.  1 split: everything.
   const int nbt = c_div_up(x.c.nbody, kPage);
   const int npp = min(min(x.c.pv, x.c.pk), nbt);
-  int t0, t1;
-  bool tail;
+  const int n_tail = num_splits >= 4 && npp < 12 * (num_splits - 3) ? 3 : (num_splits >= 2 ? 1 : 0);
+  int t0 = 0, t1 = 0;          // body tiles of this split
+  int u0 = nbt, u1 = nbt;      // tail tiles of this split
+  bool do_sink = false;
   if (num_splits == 1) {
-    t0 = 0; t1 = npp; tail = true;
-  } else if (split < num_splits - 1) {
-    const int per = (npp + num_splits - 2) / (num_splits - 1);
-    t0 = min(npp, split * per); t1 = min(npp, t0 + per); tail = false;
+    t1 = npp; u0 = npp; do_sink = true;
+  } else if (split < n_tail) {
+    if (n_tail == 1) { u0 = npp; do_sink = true; }
+    else if (split == 0) do_sink = true;
+    else if (split == 1) { u0 = npp; u1 = min(nbt, npp + 1); }
+    else u0 = min(nbt, npp + 1);
   } else {
-    t0 = t1 = 0; tail = true;
+    const int n_body = num_splits - n_tail;
+    const int per = (npp + n_body - 1) / n_body;
+    t0 = min(npp, (split - n_tail) * per); t1 = min(npp, t0 + per);
   }
+  const bool tail = do_sink || u0 < u1;
   const uint8_t* qbuf_k = (const uint8_t*)L.qbuf_k + (int64_t)x.b * L.win_stride_b + (int64_t)x.h * L.win_stride_h;
 
   float4v C[8];
@@ -651,7 +661,7 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(kitty_kv_layer L, co
     KRegs kb;
     VRegs vb;
 #pragma unroll 1
-    for (int i = npp; i < nbt; ++i) {
+    for (int i = u0; i < u1; ++i) {
       float cz = 0.f;
       const int ntok = min(kPage, x.c.nbody - i * kPage);
       if (i < x.c.pk) {
@@ -676,7 +686,7 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(kitty_kv_layer L, co
         pv_fp16<false>(x, A, (i - x.c.pv) * kPage, ntok, C);
       }
     }
-    if (x.c.sink > 0) {
+    if (do_sink && x.c.sink > 0) {
       const uint8_t* sink_k = (const uint8_t*)L.sink_k + (int64_t)x.b * L.sink_stride_b + (int64_t)x.h * L.sink_stride_h;
       qk_fp16(x, sink_k, L.S, C);
       softmax_tile<false>(x, A, C, 0.f, x.c.sink);

@@ -172,22 +172,38 @@ __global__ __launch_bounds__(256) void decode_plain_kernel(kitty_kv_layer L, con
 }
 
 // out[b, 0, hq, :] = sum_s acc_s * 2^(m_s - m) / sum_s l_s * 2^(m_s - m); the running maxima of
-// the partials are in log2 units.
-__global__ __launch_bounds__(128) void decode_merge_kernel(const float* __restrict__ ws_ml,
-                                                           const float* __restrict__ ws_acc,
-                                                           __half* __restrict__ out, int num_splits) {
-  const int64_t row0 = ((int64_t)blockIdx.y * gridDim.x + blockIdx.x) * num_splits;
-  const int d = threadIdx.x;
+// the partials are in log2 units.  One block per (32 channels, query head, batch row): 8 groups
+// of 32 lanes stride over the splits, then combine through LDS in a fixed order.
+constexpr int kMergeGroups = 8, kMergeChannels = 32;
+__global__ __launch_bounds__(kMergeGroups * kMergeChannels) void decode_merge_kernel(
+    const float* __restrict__ ws_ml, const float* __restrict__ ws_acc, __half* __restrict__ out, int num_splits) {
+  __shared__ float s_m[kMergeGroups], s_l[kMergeGroups], s_o[kMergeGroups][kMergeChannels];
+  const int64_t head = (int64_t)blockIdx.z * gridDim.y + blockIdx.y;
+  const int64_t row0 = head * num_splits;
+  const int lane = threadIdx.x & (kMergeChannels - 1), grp = threadIdx.x / kMergeChannels;
+  const int d = blockIdx.x * kMergeChannels + lane;
   float m = -INFINITY;
-  for (int s = 0; s < num_splits; ++s) m = fmaxf(m, ws_ml[(row0 + s) * 2]);
+  for (int s = grp; s < num_splits; s += kMergeGroups) m = fmaxf(m, ws_ml[(row0 + s) * 2]);
+  if (lane == 0) s_m[grp] = m;
+  __syncthreads();
+#pragma unroll
+  for (int g = 0; g < kMergeGroups; ++g) m = fmaxf(m, s_m[g]);
   float l = 0.f, o = 0.f;
-  for (int s = 0; s < num_splits; ++s) {
+  for (int s = grp; s < num_splits; s += kMergeGroups) {
     const float ms = ws_ml[(row0 + s) * 2];
     const float w = (ms == -INFINITY) ? 0.f : exp2f(ms - m);
     l += ws_ml[(row0 + s) * 2 + 1] * w;
     o += ws_acc[(row0 + s) * kD + d] * w;
   }
-  out[((int64_t)blockIdx.y * gridDim.x + blockIdx.x) * kD + d] = __float2half_rn(l > 0.f ? o / l : 0.f);
+  if (lane == 0) s_l[grp] = l;
+  s_o[grp][lane] = o;
+  __syncthreads();
+  if (grp == 0) {
+    l = 0.f, o = 0.f;
+#pragma unroll
+    for (int g = 0; g < kMergeGroups; ++g) { l += s_l[g]; o += s_o[g][lane]; }
+    out[head * kD + d] = __float2half_rn(l > 0.f ? o / l : 0.f);
+  }
 }
 
 void launch_decode_plain(const kitty_kv_layer& L, const void* q, int B, int H_Q, float scaling, float* ws_ml,
@@ -198,8 +214,8 @@ void launch_decode_plain(const kitty_kv_layer& L, const void* q, int B, int H_Q,
 
 void launch_decode_merge(const float* ws_ml, const float* ws_acc, void* out, int B, int H_Q, int num_splits,
                          hipStream_t stream) {
-  hipLaunchKernelGGL(decode_merge_kernel, dim3(H_Q, B), dim3(kD), 0, stream, ws_ml, ws_acc, (__half*)out,
-                     num_splits);
+  hipLaunchKernelGGL(decode_merge_kernel, dim3(kD / kMergeChannels, H_Q, B), dim3(kMergeGroups * kMergeChannels), 0,
+                     stream, ws_ml, ws_acc, (__half*)out, num_splits);
 }
 
 }  // namespace kitty
