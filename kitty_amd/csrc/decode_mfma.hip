@@ -75,6 +75,7 @@ struct WaveLds<true> : Tables {
 template <>
 struct WaveLds<false> : Tables {
   __attribute__((aligned(16))) _Float16 q_nat[16][kQPad];
+  __attribute__((aligned(16))) uint8_t kbuf[1][10240];     // staging of fp16 V rows (pv_fp16)
 };
 
 __device__ __forceinline__ float4v mfma16(const uint32_t (&a)[4], const uint32_t (&b)[4], float4v c) {
@@ -478,44 +479,72 @@ __device__ __forceinline__ void pv_packed(LDS& S, const Ctx& x, float4v (&out)[8
   }
 }
 
-// fp16 V rows (sink, V Q-buffer, local ring): A gathered column-wise, accumulators in true units
+// fp16 V rows (sink, V Q-buffer, local ring), accumulators in true units.  The matrix core wants
+// A[row = channel][k = token], i.e. the rows transposed: 32 tokens at a time (the tokens of one
+// lane group) are copied into LDS as [channel][token] with 16-bit stores, after which the eight
+// k-slots of a lane are one 128-bit read.  The other three lane groups multiply by zero meanwhile.
+constexpr int kVtPitch = 80;                 // bytes per channel row: 32 tokens + padding
+constexpr int kVtBytes = kD * kVtPitch;      // 10240
+static_assert(kVtBytes <= 2 * kKTile && kVtBytes <= 10240, "the staging area reuses the K tile buffers");
 template <bool SINK>
-__device__ __forceinline__ void pv_fp16(const Ctx& x, Acc& A, int tail_first_row, int ntok, const float4v (&P)[8]) {
+__device__ __forceinline__ void pv_fp16(uint8_t* vt, const Ctx& x, Acc& A, int tail_first_row, int ntok,
+                                        const float4v (&P)[8]) {
   const kitty_kv_layer& L = *x.L;
   const uint32_t one_or_zero = (x.n & 1) ? 0u : 0x3C003C00u;    // even rows sum p, odd rows stay 0
-#pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    uint32_t bp[4], alz[4];
-    const __half* rp[8];
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      // rows past the tile's end carry p = 0; read a valid row instead so that 0 * value stays 0
-      const int t = min(32 * x.kg + 8 * j + i, ntok - 1);
+  const int tt = x.lane >> 1, c0 = (x.lane & 1) * 8;            // staging: token of the quarter, first piece
+  // the rows of quarter qt + 1 are fetched while quarter qt is multiplied
+  auto fetch = [&](int qt, uint4 (&piece)[8]) {
+    const int t = 32 * qt + tt;
+    const bool ok = t < ntok;   // rows past the tile's end carry p = 0; zeros keep 0 * value at 0
+    const __half* row = nullptr;
+    if (ok) {
       if (SINK)
-        rp[i] = (const __half*)((const uint8_t*)L.sink_v + (int64_t)x.b * L.sink_stride_b +
-                                (int64_t)x.h * L.sink_stride_h) + (int64_t)t * kD;
+        row = (const __half*)((const uint8_t*)L.sink_v + (int64_t)x.b * L.sink_stride_b +
+                              (int64_t)x.h * L.sink_stride_h) + (int64_t)t * kD;
       else
-        rp[i] = v_tail_row(L, x.c, x.b, x.h, tail_first_row + t);
+        row = v_tail_row(L, x.c, x.b, x.h, tail_first_row + t);
     }
 #pragma unroll
-    for (int pi = 0; pi < 4; ++pi) {
-      const half2v p2 = {(_Float16)P[2 * pi][j], (_Float16)P[2 * pi + 1][j]};
-      bp[pi] = as_u32(p2);
-      alz[pi] = one_or_zero;
-    }
-    A.lz = mfma16(alz, bp, A.lz);
+    for (int k = 0; k < 8; ++k) piece[k] = ok ? ((const uint4*)row)[c0 + k] : uint4{0u, 0u, 0u, 0u};
+  };
+  uint4 piece[8];
+  fetch(0, piece);
+#pragma unroll 1
+  for (int qt = 0; qt < 4; ++qt) {
+    if (32 * qt >= ntok) break;
+    wave_lds_fence();
 #pragma unroll
-    for (int u = 0; u < 8; ++u) {
-      uint32_t a[4];
+    for (int k = 0; k < 8; ++k) {
+      const uint32_t w4[4] = {piece[k].x, piece[k].y, piece[k].z, piece[k].w};
+      uint8_t* dst = vt + (8 * (c0 + k)) * kVtPitch + 2 * tt;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        *(uint16_t*)(dst + (2 * i) * kVtPitch) = (uint16_t)(w4[i] & 0xffffu);
+        *(uint16_t*)(dst + (2 * i + 1) * kVtPitch) = (uint16_t)(w4[i] >> 16);
+      }
+    }
+    if (32 * (qt + 1) < ntok) fetch(qt + 1, piece);
+    wave_lds_fence();
+    const bool mine = x.kg == qt;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      uint32_t bp[4], alz[4];
 #pragma unroll
       for (int pi = 0; pi < 4; ++pi) {
-        const uint32_t lo = __half_as_ushort(rp[2 * pi][8 * x.n + u]);
-        const uint32_t hi = __half_as_ushort(rp[2 * pi + 1][8 * x.n + u]);
-        a[pi] = lo | (hi << 16);
+        const half2v p2 = {(_Float16)P[2 * pi][j], (_Float16)P[2 * pi + 1][j]};   // tokens 32kg + 8j + 2pi + {0,1}
+        bp[pi] = mine ? as_u32(p2) : 0u;
+        alz[pi] = one_or_zero;
       }
-      A.out[u] = mfma16(a, bp, A.out[u]);
+      A.lz = mfma16(alz, bp, A.lz);
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const uint4v a4 = *(const uint4v*)(vt + (8 * x.n + u) * kVtPitch + 16 * j);   // tokens 8j .. 8j+7 of the quarter
+        const uint32_t a[4] = {a4[0], a4[1], a4[2], a4[3]};
+        A.out[u] = mfma16(a, bp, A.out[u]);
+      }
     }
   }
+  wave_lds_fence();
 }
 
 __device__ __forceinline__ void to_true_units(Acc& A) {
@@ -683,14 +712,14 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(kitty_kv_layer L, co
 #pragma unroll
         for (int u = 0; u < 8; ++u) A.out[u] += tmp[u] * code_unscale(u);
       } else {
-        pv_fp16<false>(x, A, (i - x.c.pv) * kPage, ntok, C);
+        pv_fp16<false>(&S.kbuf[0][0], x, A, (i - x.c.pv) * kPage, ntok, C);
       }
     }
     if (do_sink && x.c.sink > 0) {
       const uint8_t* sink_k = (const uint8_t*)L.sink_k + (int64_t)x.b * L.sink_stride_b + (int64_t)x.h * L.sink_stride_h;
       qk_fp16(x, sink_k, L.S, C);
       softmax_tile<false>(x, A, C, 0.f, x.c.sink);
-      pv_fp16<true>(x, A, 0, x.c.sink, C);
+      pv_fp16<true>(&S.kbuf[0][0], x, A, 0, x.c.sink, C);
     }
   }
   to_true_units(A);
