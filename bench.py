@@ -9,6 +9,7 @@ Infinity Cache.  Prints ONE JSON line.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c1|c0|c2|c4] [--copies N]
 
+``--workload e2e`` times a whole 32-layer decoder step around the cache (tokens/s).
 ``--workload c3`` measures the other kernel family instead (BASELINE.json configs[3]): a 2048-token
 chunk attending a 30720-token packed prefix, bound by the matrix cores, plus the append of the chunk.
 """
@@ -187,12 +188,94 @@ def bench_chunked_prefill(args):
     print(json.dumps(result))
 
 
+def bench_end_to_end(args):
+    """The side number of configs[4]: decode tokens/s of a full 32-layer Llama-3.1-8B-shaped model
+    with random weights, every layer's KV in the packed cache.  The dense parts (projections, MLP,
+    norms, RoPE, LM head) are plain torch; attention and the cache are this library, driven in the
+    reference's call order (update -> attend -> quantize_decode, modeling_qwen3.py:225-251)."""
+    import torch
+    import torch.nn.functional as F
+    import kitty_amd
+    from kitty_amd import _lib
+    from kitty_amd.kvcache.kernels import kitty_attention_forward
+    _lib.lib()
+    dev = torch.device("cuda:0")
+    B, T0 = args.e2e_batch, args.e2e_context
+    LAYERS, HID, H_Q, H_KV, D, FF, VOCAB = 32, 4096, 32, 8, 128, 14336, 128256
+    cfg = types.SimpleNamespace(num_hidden_layers=LAYERS, head_dim=D, num_key_value_heads=H_KV,
+                                num_attention_heads=H_Q, hidden_size=HID)
+    mod = types.SimpleNamespace(num_attention_heads=H_Q, num_key_value_heads=H_KV)
+    g = torch.Generator(device=dev).manual_seed(8)
+    rnd = lambda *shape, std=0.02: (torch.randn(*shape, generator=g, device=dev, dtype=torch.float32) * std).half()
+    layers = [dict(wqkv=rnd((H_Q + 2 * H_KV) * D, HID), wo=rnd(HID, HID), wgu=rnd(2 * FF, HID), wd=rnd(HID, FF),
+                   n1=torch.ones(HID, device=dev, dtype=torch.float16),
+                   n2=torch.ones(HID, device=dev, dtype=torch.float16)) for _ in range(LAYERS)]
+    emb, head = rnd(VOCAB, HID), rnd(VOCAB, HID)
+    nf = torch.ones(HID, device=dev, dtype=torch.float16)
+    steps = args.warmup + args.steps
+    cache = kitty_amd.KittyCache(cfg, B, T0 + steps + 256, device=dev)
+    K, V = synth_kv(B, H_KV, T0, D, 1004, dev)
+    for li in range(LAYERS):              # a context of T0 tokens in every layer (same synthetic K/V)
+        cache.update(K, V, li)
+        cache.quantize_prefill(li)
+    del K, V
+    inv_freq = 1.0 / (500000.0 ** (torch.arange(0, D, 2, device=dev, dtype=torch.float32) / D))
+
+    def rope(x, pos):                     # x [B, H, 1, D], rotate-half convention
+        ang = pos * inv_freq
+        cos, sin = torch.cat([ang.cos(), ang.cos()]).half(), torch.cat([ang.sin(), ang.sin()]).half()
+        x1, x2 = x[..., : D // 2], x[..., D // 2:]
+        return x * cos + torch.cat([-x2, x1], dim=-1) * sin
+
+    def rms(x, w):
+        xf = x.float()
+        return (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + 1e-5)).half() * w
+
+    @torch.no_grad()
+    def step(tok, pos):
+        x = emb[tok]                      # [B, HID]: 2-D activations keep the GEMM launches cheap
+        for li, w in enumerate(layers):
+            h = rms(x, w["n1"])
+            qkv = F.linear(h, w["wqkv"]).view(B, 1, H_Q + 2 * H_KV, D).transpose(1, 2)
+            q, k, v = qkv[:, :H_Q], qkv[:, H_Q:H_Q + H_KV], qkv[:, H_Q + H_KV:]
+            q, k = rope(q, pos).contiguous(), rope(k, pos)
+            cache.update(k, v, li)
+            a, _ = kitty_attention_forward(mod, q, cache.kv_cache[li], D ** -0.5)
+            cache.quantize_decode(li)
+            x = x + F.linear(a.view(B, HID), w["wo"])
+            h = rms(x, w["n2"])
+            gu = F.linear(h, w["wgu"])
+            x = x + F.linear(F.silu(gu[..., :FF]) * gu[..., FF:], w["wd"])
+        return F.linear(rms(x, nf), head).argmax(-1).view(B)
+
+    tok = torch.zeros(B, dtype=torch.long, device=dev)
+    for i in range(args.warmup):
+        tok = step(tok, T0 + i)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        tok = step(tok, T0 + args.warmup + i)
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / args.steps
+    print(json.dumps({
+        "metric": "end_to_end_decode_tokens_per_s", "value": B / dt, "unit": "tokens/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": dt * 1e3, "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f16 model, 2/4-bit packed KV",
+        "data": "synthetic (random-init Llama-3.1-8B shapes, synthetic KV context in every layer)",
+        "config": {"workload": f"32-layer Llama-3.1-8B-shaped decode, batch {B}, context {T0}, greedy (configs[4] side number)",
+                   "batch": B, "context": T0, "layers": LAYERS},
+        "note": "dense layers are torch (hipBLASLt); one Python-driven launch sequence per layer, not graph-captured",
+    }))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="c1", choices=sorted(WORKLOADS) + ["c3"])
+    ap.add_argument("--workload", default="c1", choices=sorted(WORKLOADS) + ["c3", "e2e"])
+    ap.add_argument("--e2e-batch", type=int, default=16)
+    ap.add_argument("--e2e-context", type=int, default=32768)
     ap.add_argument("--copies", type=int, default=0, help="independent cache copies to rotate over (0 = auto)")
     ap.add_argument("--splits", type=int, default=0)
     ap.add_argument("--variant", type=int, default=0)
@@ -208,6 +291,8 @@ def main():
 
     if args.workload == "c3":
         return bench_chunked_prefill(args)
+    if args.workload == "e2e":
+        return bench_end_to_end(args)
     import torch
     import kitty_amd
     from kitty_amd import _lib
