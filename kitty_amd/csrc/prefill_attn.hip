@@ -19,7 +19,7 @@
 //   S^T[pos][row]  = sum_ch  K[pos][ch]  * Q[row][ch]      A = keys,   B = queries (registers)
 //   O^T[cp][row]   = sum_pos V[pos][cp]  * P^T[pos][row]   A = values, B = probabilities
 // The accumulator of the first product is, lane for lane, the B operand of the second: k-slot j
-// of lane group kg stands for position 32 m2 + 16 (j / 4) + 4 kg + j % 4.
+// of lane group kg stands for position 16 (j / 4) + 4 kg + j % 4 of a 32-position sub-tile.
 //
 // LDS layouts, chosen so that dequantization writes 128-bit rows and the matrix-core operands
 // come out of `ds_read_b64_tr_b16` (a 16-lane block reads 4 rows x 16 columns and lane i
@@ -262,39 +262,46 @@ struct WaveAcc {
   bool first;
 };
 
-// 64 positions [64 sub, 64 sub + 64) of the tile in (kt, vt) against this wavefront's rows.
+// 32 positions [32 sub, 32 sub + 32) of the tile in (kt, vt) against this wavefront's rows (a
+// sub-tile this small keeps the logits in 32 registers; the 128 accumulator registers and the 64
+// query registers leave room for little more).
 // limit[nt]: tokens of the tile with index < limit are visible to the row of column tile nt.
 __device__ __forceinline__ void attend_sub(const uint8_t* kt, const uint8_t* vt, int sub, const half8 (&q)[4][4],
                                            WaveAcc& A, float sc2, bool masked, const int (&limit)[4], int kg,
                                            int n) {
-  float4v S[4][4];
+  float4v S[2][4];
 #pragma unroll
-  for (int mt = 0; mt < 4; ++mt)
+  for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
     for (int nt = 0; nt < 4; ++nt) S[mt][nt] = float4v{0.f, 0.f, 0.f, 0.f};
   // lane's corner inside a 16-lane transposing read: row n / 4 of 4, columns 4 (n % 4) ..
   const int lane_off = (4 * kg + (n >> 2)) * kPitch + (n & 3) * 8;
-  const uint8_t* kbase = kt + lane_off + sub * 128;
+  const uint8_t* kbase = kt + lane_off + sub * 64;
   // channel chunk c+1 is fetched while chunk c is multiplied; the fences keep the scheduler from
-  // hoisting every operand load to the top (which costs more registers than the wave has)
-  half8 a_cur[4], a_nxt[4];
+  // hoisting every operand load to the top
+  half8 a_cur[2], a_nxt[2];
 #pragma unroll
-  for (int mt = 0; mt < 4; ++mt) a_cur[mt] = load_a(kbase + mt * 32);
+  for (int mt = 0; mt < 2; ++mt) a_cur[mt] = load_a(kbase + mt * 32);
 #pragma unroll
   for (int c = 0; c < 4; ++c) {
     if (c < 3) {
 #pragma unroll
-      for (int mt = 0; mt < 4; ++mt) a_nxt[mt] = load_a(kbase + (32 * (c + 1)) * kPitch + mt * 32);
+      for (int mt = 0; mt < 2; ++mt) a_nxt[mt] = load_a(kbase + (32 * (c + 1)) * kPitch + mt * 32);
     }
 #pragma unroll
-    for (int mt = 0; mt < 4; ++mt)
+    for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
       for (int nt = 0; nt < 4; ++nt)
         S[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a_cur[mt], q[c][nt], S[mt][nt], 0, 0, 0);
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-    for (int mt = 0; mt < 4; ++mt) a_cur[mt] = a_nxt[mt];
+    for (int mt = 0; mt < 2; ++mt) a_cur[mt] = a_nxt[mt];
   }
+  // the first value operands travel while the softmax runs
+  const uint8_t* vbase = vt + lane_off + (32 * sub) * kPitch;
+  half8 v_cur[2], v_nxt[2];
+  v_cur[0] = load_a(vbase);
+  v_cur[1] = load_a(vbase + 32);
 
   // online softmax, column by column (a column = one query row, spread over the 4 lane groups)
   float mt_[4];
@@ -303,12 +310,12 @@ __device__ __forceinline__ void attend_sub(const uint8_t* kt, const uint8_t* vt,
     const float cst = -A.m[nt];
     float mx = -INFINITY;
 #pragma unroll
-    for (int mt = 0; mt < 4; ++mt)
+    for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         float v = S[mt][nt][i] * sc2 + cst;
         if (masked) {
-          const int tok = 64 * sub + 16 * mt + 2 * kg + (i >> 1) + 8 * (i & 1);
+          const int tok = 32 * sub + 16 * mt + 2 * kg + (i >> 1) + 8 * (i & 1);
           if (tok >= limit[nt]) v = -INFINITY;
         }
         S[mt][nt][i] = v;
@@ -324,7 +331,7 @@ __device__ __forceinline__ void attend_sub(const uint8_t* kt, const uint8_t* vt,
     for (int nt = 0; nt < 4; ++nt) {
       const float dm = A.first ? mt_[nt] : fmaxf(mt_[nt], 0.f);
 #pragma unroll
-      for (int mt = 0; mt < 4; ++mt)
+      for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
         for (int i = 0; i < 4; ++i) S[mt][nt][i] -= dm;
       if (!A.first) {
@@ -337,12 +344,12 @@ __device__ __forceinline__ void attend_sub(const uint8_t* kt, const uint8_t* vt,
     }
     A.first = false;
   }
-  half8 p[2][4];
+  half8 p[4];
 #pragma unroll
   for (int nt = 0; nt < 4; ++nt) {
     float sum = 0.f;
 #pragma unroll
-    for (int mt = 0; mt < 4; ++mt)
+    for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const float e = __builtin_amdgcn_exp2f(S[mt][nt][i]);
@@ -350,31 +357,23 @@ __device__ __forceinline__ void attend_sub(const uint8_t* kt, const uint8_t* vt,
         sum += e;
       }
     A.l[nt] += sum;
-#pragma unroll
-    for (int m2 = 0; m2 < 2; ++m2) {
-      const float4v x0 = S[2 * m2][nt], x1 = S[2 * m2 + 1][nt];
-      p[m2][nt] = half8{(_Float16)x0[0], (_Float16)x0[1], (_Float16)x0[2], (_Float16)x0[3],
-                        (_Float16)x1[0], (_Float16)x1[1], (_Float16)x1[2], (_Float16)x1[3]};
-    }
+    const float4v x0 = S[0][nt], x1 = S[1][nt];
+    p[nt] = half8{(_Float16)x0[0], (_Float16)x0[1], (_Float16)x0[2], (_Float16)x0[3],
+                  (_Float16)x1[0], (_Float16)x1[1], (_Float16)x1[2], (_Float16)x1[3]};
   }
-  const uint8_t* vbase = vt + lane_off + (64 * sub) * kPitch;
-  // 8 groups of (m2, two channel-slot tiles); group i+1 is fetched while group i is multiplied
-  half8 v_cur[2], v_nxt[2];
-  v_cur[0] = load_a(vbase);
-  v_cur[1] = load_a(vbase + 32);
+  // 4 groups of two channel-slot tiles; group i+1 is fetched while group i is multiplied
 #pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    const int m2 = i >> 2, ct = 2 * (i & 3);
-    if (i < 7) {
-      const int m2n = (i + 1) >> 2, ctn = 2 * ((i + 1) & 3);
-      v_nxt[0] = load_a(vbase + (32 * m2n) * kPitch + ctn * 32);
-      v_nxt[1] = load_a(vbase + (32 * m2n) * kPitch + (ctn + 1) * 32);
+  for (int i = 0; i < 4; ++i) {
+    const int ct = 2 * i;
+    if (i < 3) {
+      v_nxt[0] = load_a(vbase + (ct + 2) * 32);
+      v_nxt[1] = load_a(vbase + (ct + 3) * 32);
     }
 #pragma unroll
     for (int j = 0; j < 2; ++j)
 #pragma unroll
       for (int nt = 0; nt < 4; ++nt)
-        A.o[ct + j][nt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(v_cur[j], p[m2][nt], A.o[ct + j][nt], 0, 0, 0);
+        A.o[ct + j][nt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(v_cur[j], p[nt], A.o[ct + j][nt], 0, 0, 0);
     __builtin_amdgcn_sched_barrier(0);
     v_cur[0] = v_nxt[0];
     v_cur[1] = v_nxt[1];
@@ -457,8 +456,9 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
     for (int nt = 0; nt < 4; ++nt)
       limit[nt] = cur.chunk_t0 >= 0 ? min(cur.ntok, qpos[nt] - cur.chunk_t0 + 1) : cur.ntok;
     const bool masked = cur.chunk_t0 >= 0 || cur.ntok < kPage;
-    attend_sub(kt, vt, 0, qreg, A, sc2, masked, limit, kg, n);
-    if (cur.ntok > 64) attend_sub(kt, vt, 1, qreg, A, sc2, masked, limit, kg, n);
+#pragma unroll 1
+    for (int sub = 0; sub < 4; ++sub)
+      if (32 * sub < cur.ntok) attend_sub(kt, vt, sub, qreg, A, sc2, masked, limit, kg, n);
     if (more) P.finish(nxt, g, lds + (buf ^ 1) * kTile, lds + (2 + (buf ^ 1)) * kTile);
     cur = nxt;
     __syncthreads();
