@@ -304,23 +304,27 @@ __device__ __forceinline__ void attend_sub(const uint8_t* kt, const uint8_t* vt,
   v_cur[1] = load_a(vbase + 32);
 
   // online softmax, column by column (a column = one query row, spread over the 4 lane groups)
+#pragma unroll
+  for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+    for (int mt = 0; mt < 2; ++mt) S[mt][nt] = S[mt][nt] * sc2 - A.m[nt];
+  if (masked) {   // one wave-uniform branch: partial tiles and the chunk's own tiles only
+#pragma unroll
+    for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+      for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int tok = 32 * sub + 16 * mt + 2 * kg + (i >> 1) + 8 * (i & 1);
+          if (tok >= limit[nt]) S[mt][nt][i] = -INFINITY;
+        }
+    asm volatile("" ::: "memory");   // keep this a branch, not 32 selects on every tile
+  }
   float mt_[4];
 #pragma unroll
   for (int nt = 0; nt < 4; ++nt) {
-    const float cst = -A.m[nt];
-    float mx = -INFINITY;
-#pragma unroll
-    for (int mt = 0; mt < 2; ++mt)
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        float v = S[mt][nt][i] * sc2 + cst;
-        if (masked) {
-          const int tok = 32 * sub + 16 * mt + 2 * kg + (i >> 1) + 8 * (i & 1);
-          if (tok >= limit[nt]) v = -INFINITY;
-        }
-        S[mt][nt][i] = v;
-        mx = fmaxf(mx, v);
-      }
+    float mx = fmaxf(fmaxf(S[0][nt][0], S[0][nt][1]), fmaxf(S[0][nt][2], S[0][nt][3]));
+    mx = fmaxf(mx, fmaxf(fmaxf(S[1][nt][0], S[1][nt][1]), fmaxf(S[1][nt][2], S[1][nt][3])));
     mx = fmaxf(mx, xor_lanes(mx, 16));
     mx = fmaxf(mx, xor_lanes(mx, 32));
     mt_[nt] = mx;
