@@ -43,7 +43,12 @@ constexpr int kPitch = 288;                   // bytes per LDS row: 128 fp16 + 3
 constexpr int kTile = kPage * kPitch;         // 36864 bytes, one K or V tile
 constexpr int kLdsBytes = 4 * kTile;          // K and V, two buffers each
 constexpr int kRows = 256;                    // query rows per workgroup
-constexpr int kThreads = 256;
+constexpr int kWaves = 8;                     // two per SIMD: one does vector work while the other feeds the matrix pipe
+constexpr int kThreads = 64 * kWaves;
+constexpr int kNT = kRows / (16 * kWaves);    // 16-row column tiles per wave
+constexpr int kParts = kThreads / 128;        // threads that share one row of a tile while staging it
+constexpr int kW = 8 / kParts;                // 16-code words of a packed row per thread
+constexpr int kPartBytes = 256 / kParts;      // bytes of an fp16 row per thread
 constexpr float kLog2e = 1.4426950408889634f;
 
 enum SrcKind : int { SRC_PACKED = 0, SRC_ROWS = 1, SRC_VTAIL = 2 };
@@ -63,7 +68,7 @@ struct TileSrc {
 
 // what issue() leaves in flight for a packed tile (fp16 rows are few and are copied by finish())
 struct Stage {
-  uint4 klo, khi, v;
+  uint32_t klo[kW], khi[kW], v[kW];
   uint32_t kmeta, vmeta;
 };
 
@@ -162,50 +167,57 @@ struct Prefill {
 
   // ---- stage 1: global loads of a packed tile into registers ----------------------------------
   __device__ __forceinline__ void issue(const TileSrc& s, Stage& g) const {
-    const int e = tid >> 1, half = tid & 1;   // element (channel or token) and 64-wide half
+    const int e = tid / kParts, part = tid % kParts;   // element (channel or token) and its part of the row
     if (s.k_kind == SRC_PACKED) {
-      g.klo = *(const uint4*)(s.k_ptr + e * kRowBytes + half * 16);
+      const uint32_t* lo = (const uint32_t*)(s.k_ptr + e * kRowBytes + part * (4 * kW));
+#pragma unroll
+      for (int w = 0; w < kW; ++w) g.klo[w] = lo[w];
       g.kmeta = *(const uint32_t*)(s.k_meta + e * 4);
-      g.khi = uint4{0u, 0u, 0u, 0u};
+#pragma unroll
+      for (int w = 0; w < kW; ++w) g.khi[w] = 0u;
       if (BOOST) {
         const int slot = s.k_ptr[kLoBytes + L.D_BOOSTED * kRowBytes + e];
-        if (slot < L.D_BOOSTED) g.khi = *(const uint4*)(s.k_ptr + kLoBytes + slot * kRowBytes + half * 16);
+        if (slot < L.D_BOOSTED) {
+          const uint32_t* hi = (const uint32_t*)(s.k_ptr + kLoBytes + slot * kRowBytes + part * (4 * kW));
+#pragma unroll
+          for (int w = 0; w < kW; ++w) g.khi[w] = hi[w];
+        }
       }
     }
     if (s.v_kind == SRC_PACKED) {
-      g.v = *(const uint4*)(s.v_ptr + e * kRowBytes + half * 16);
+      const uint32_t* vv = (const uint32_t*)(s.v_ptr + e * kRowBytes + part * (4 * kW));
+#pragma unroll
+      for (int w = 0; w < kW; ++w) g.v[w] = vv[w];
       g.vmeta = *(const uint32_t*)(s.v_meta + e * 4);
     }
   }
 
   // ---- stage 2: registers -> fp16 tile in LDS -----------------------------------------------
   __device__ __forceinline__ void finish(const TileSrc& s, const Stage& g, uint8_t* kt, uint8_t* vt) const {
-    const int e = tid >> 1, half = tid & 1;
+    const int e = tid / kParts, part = tid % kParts;
     if (s.k_kind == SRC_PACKED) {
-      // thread = one channel, 64 tokens: four plane words of 16 tokens each
+      // thread = one channel, 16 kW tokens: plane words of 16 tokens each
       const half2v m2 = __builtin_bit_cast(half2v, g.kmeta);
       const half2v scale = {m2[0], m2[0]}, zero = {m2[1], m2[1]};
-      const uint32_t lo[4] = {g.klo.x, g.klo.y, g.klo.z, g.klo.w};
-      const uint32_t hi[4] = {g.khi.x, g.khi.y, g.khi.z, g.khi.w};
-      uint8_t* row = kt + e * kPitch + half * 128;
+      uint8_t* row = kt + e * kPitch + part * kPartBytes;
 #pragma unroll
-      for (int w = 0; w < 4; ++w) {
+      for (int w = 0; w < kW; ++w) {
         uint32_t o[8];
 #pragma unroll
         for (int u = 0; u < 8; ++u) {
-          uint32_t code = (lo[w] >> (2 * u)) & 0x00030003u;
-          if (BOOST) code |= ((hi[w] >> (2 * u)) & 0x00030003u) << 2;
+          uint32_t code = (g.klo[w] >> (2 * u)) & 0x00030003u;
+          if (BOOST) code |= ((g.khi[w] >> (2 * u)) & 0x00030003u) << 2;
           o[u] = dequant_pair(code, scale, zero);
         }
         *(uint4*)(row + w * 32) = uint4{o[0], o[1], o[2], o[3]};
         *(uint4*)(row + w * 32 + 16) = uint4{o[4], o[5], o[6], o[7]};
       }
     } else if (e < s.ntok) {
-      // thread = one token, 64 channels: transpose into [channel][slot] with 16-bit stores
-      uint8_t* col = kt + (half * 64) * kPitch + slot_of(e) * 2;
-      const uint4* src = (const uint4*)(s.k_ptr + (int64_t)e * s.k_stride + half * 128);
+      // thread = one token, 16 kW channels: transpose into [channel][slot] with 16-bit stores
+      uint8_t* col = kt + (part * 16 * kW) * kPitch + slot_of(e) * 2;
+      const uint4* src = (const uint4*)(s.k_ptr + (int64_t)e * s.k_stride + part * kPartBytes);
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
+      for (int i = 0; i < 2 * kW; ++i) {
         const uint4 x = src[i];
         const uint32_t w4[4] = {x.x, x.y, x.z, x.w};
 #pragma unroll
@@ -215,17 +227,16 @@ struct Prefill {
         }
       }
     }
-    uint8_t* vrow = vt + slot_of(e) * kPitch + half * 128;
+    uint8_t* vrow = vt + slot_of(e) * kPitch + part * kPartBytes;
     if (s.v_kind == SRC_PACKED) {
-      // thread = one token, 64 channels: four words of 16 channels each
+      // thread = one token, 16 kW channels: words of 16 channels each
       const half2v m2 = __builtin_bit_cast(half2v, g.vmeta);
       const half2v scale = {m2[0], m2[0]}, zero = {m2[1], m2[1]};
-      const uint32_t wv[4] = {g.v.x, g.v.y, g.v.z, g.v.w};
 #pragma unroll
-      for (int w = 0; w < 4; ++w) {
+      for (int w = 0; w < kW; ++w) {
         uint32_t o[8];
 #pragma unroll
-        for (int u = 0; u < 8; ++u) o[u] = dequant_pair((wv[w] >> (2 * u)) & 0x00030003u, scale, zero);
+        for (int u = 0; u < 8; ++u) o[u] = dequant_pair((g.v[w] >> (2 * u)) & 0x00030003u, scale, zero);
         *(uint4*)(vrow + w * 32) = uint4{o[0], o[1], o[2], o[3]};
         *(uint4*)(vrow + w * 32 + 16) = uint4{o[4], o[5], o[6], o[7]};
       }
@@ -235,11 +246,11 @@ struct Prefill {
       const uint4* src = nullptr;
       if (ok)
         src = s.v_kind == SRC_VTAIL
-                  ? (const uint4*)((const uint8_t*)v_tail_row(L, c, b, h, s.v_u0 + e) + half * 128)
-                  : (const uint4*)(s.v_ptr + (int64_t)e * s.v_stride + half * 128);
+                  ? (const uint4*)((const uint8_t*)v_tail_row(L, c, b, h, s.v_u0 + e) + part * kPartBytes)
+                  : (const uint4*)(s.v_ptr + (int64_t)e * s.v_stride + part * kPartBytes);
       const uint4 zero4 = uint4{0u, 0u, 0u, 0u};
 #pragma unroll
-      for (int w = 0; w < 4; ++w) {
+      for (int w = 0; w < kW; ++w) {
         const uint4 a = ok ? src[2 * w] : zero4, bb = ok ? src[2 * w + 1] : zero4;   // channels 0..7, 8..15
         const uint32_t a4[4] = {a.x, a.y, a.z, a.w}, b4[4] = {bb.x, bb.y, bb.z, bb.w};
         uint32_t o[8];
@@ -255,10 +266,10 @@ struct Prefill {
   }
 };
 
-// One wavefront's state: 64 query rows (4 column tiles of 16) against the tiles in LDS.
+// One wavefront's state: 16 kNT query rows (kNT column tiles of 16) against the tiles in LDS.
 struct WaveAcc {
-  float4v o[8][4];    // O^T: [channel-slot tile][row tile]
-  float m[4], l[4];   // running max (log2 units) per row tile column, per-lane partial sums
+  float4v o[8][kNT];    // O^T: [channel-slot tile][row tile]
+  float m[kNT], l[kNT];   // running max (log2 units) per row tile column, per-lane partial sums
   bool first;
 };
 
@@ -266,14 +277,14 @@ struct WaveAcc {
 // sub-tile this small keeps the logits in 32 registers; the 128 accumulator registers and the 64
 // query registers leave room for little more).
 // limit[nt]: tokens of the tile with index < limit are visible to the row of column tile nt.
-__device__ __forceinline__ void attend_sub(const uint8_t* kt, const uint8_t* vt, int sub, const half8 (&q)[4][4],
-                                           WaveAcc& A, float sc2, bool masked, const int (&limit)[4], int kg,
+__device__ __forceinline__ void attend_sub(const uint8_t* kt, const uint8_t* vt, int sub, const half8 (&q)[4][kNT],
+                                           WaveAcc& A, float sc2, bool masked, const int (&limit)[kNT], int kg,
                                            int n) {
-  float4v S[2][4];
+  float4v S[2][kNT];
 #pragma unroll
   for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
-    for (int nt = 0; nt < 4; ++nt) S[mt][nt] = float4v{0.f, 0.f, 0.f, 0.f};
+    for (int nt = 0; nt < kNT; ++nt) S[mt][nt] = float4v{0.f, 0.f, 0.f, 0.f};
   // lane's corner inside a 16-lane transposing read: row n / 4 of 4, columns 4 (n % 4) ..
   const int lane_off = (4 * kg + (n >> 2)) * kPitch + (n & 3) * 8;
   const uint8_t* kbase = kt + lane_off + sub * 64;
@@ -291,7 +302,7 @@ __device__ __forceinline__ void attend_sub(const uint8_t* kt, const uint8_t* vt,
 #pragma unroll
     for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
-      for (int nt = 0; nt < 4; ++nt)
+      for (int nt = 0; nt < kNT; ++nt)
         S[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a_cur[mt], q[c][nt], S[mt][nt], 0, 0, 0);
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -305,12 +316,12 @@ __device__ __forceinline__ void attend_sub(const uint8_t* kt, const uint8_t* vt,
 
   // online softmax, column by column (a column = one query row, spread over the 4 lane groups)
 #pragma unroll
-  for (int nt = 0; nt < 4; ++nt)
+  for (int nt = 0; nt < kNT; ++nt)
 #pragma unroll
     for (int mt = 0; mt < 2; ++mt) S[mt][nt] = S[mt][nt] * sc2 - A.m[nt];
   if (masked) {   // one wave-uniform branch: partial tiles and the chunk's own tiles only
 #pragma unroll
-    for (int nt = 0; nt < 4; ++nt)
+    for (int nt = 0; nt < kNT; ++nt)
 #pragma unroll
       for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
@@ -320,19 +331,21 @@ __device__ __forceinline__ void attend_sub(const uint8_t* kt, const uint8_t* vt,
         }
     asm volatile("" ::: "memory");   // keep this a branch, not 32 selects on every tile
   }
-  float mt_[4];
+  float mt_[kNT];
 #pragma unroll
-  for (int nt = 0; nt < 4; ++nt) {
+  for (int nt = 0; nt < kNT; ++nt) {
     float mx = fmaxf(fmaxf(S[0][nt][0], S[0][nt][1]), fmaxf(S[0][nt][2], S[0][nt][3]));
     mx = fmaxf(mx, fmaxf(fmaxf(S[1][nt][0], S[1][nt][1]), fmaxf(S[1][nt][2], S[1][nt][3])));
     mx = fmaxf(mx, xor_lanes(mx, 16));
     mx = fmaxf(mx, xor_lanes(mx, 32));
     mt_[nt] = mx;
   }
-  const bool move = A.first || mt_[0] > 0.f || mt_[1] > 0.f || mt_[2] > 0.f || mt_[3] > 0.f;
+  bool move = A.first;
+#pragma unroll
+  for (int nt = 0; nt < kNT; ++nt) move = move || mt_[nt] > 0.f;
   if (__any(move)) {
 #pragma unroll
-    for (int nt = 0; nt < 4; ++nt) {
+    for (int nt = 0; nt < kNT; ++nt) {
       const float dm = A.first ? mt_[nt] : fmaxf(mt_[nt], 0.f);
 #pragma unroll
       for (int mt = 0; mt < 2; ++mt)
@@ -348,9 +361,9 @@ __device__ __forceinline__ void attend_sub(const uint8_t* kt, const uint8_t* vt,
     }
     A.first = false;
   }
-  half8 p[4];
+  half8 p[kNT];
 #pragma unroll
-  for (int nt = 0; nt < 4; ++nt) {
+  for (int nt = 0; nt < kNT; ++nt) {
     float sum = 0.f;
 #pragma unroll
     for (int mt = 0; mt < 2; ++mt)
@@ -376,7 +389,7 @@ __device__ __forceinline__ void attend_sub(const uint8_t* kt, const uint8_t* vt,
 #pragma unroll
     for (int j = 0; j < 2; ++j)
 #pragma unroll
-      for (int nt = 0; nt < 4; ++nt)
+      for (int nt = 0; nt < kNT; ++nt)
         A.o[ct + j][nt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(v_cur[j], p[nt], A.o[ct + j][nt], 0, 0, 0);
     __builtin_amdgcn_sched_barrier(0);
     v_cur[0] = v_nxt[0];
@@ -385,7 +398,7 @@ __device__ __forceinline__ void attend_sub(const uint8_t* kt, const uint8_t* vt,
 }
 
 template <bool BOOST>
-__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))) void prefill_attn_kernel(
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(kWaves / 4, kWaves / 4))) void prefill_attn_kernel(
     kitty_kv_layer L, const uint8_t* __restrict__ q, int64_t q_stride_b, int64_t q_stride_h, int64_t q_stride_t,
     const uint8_t* __restrict__ k_new, const uint8_t* __restrict__ v_new, int64_t new_stride_b,
     int64_t new_stride_h, int64_t new_stride_t, int H_Q, int Tq, float scaling, __half* __restrict__ out) {
@@ -407,12 +420,12 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
   P.first_chunk = P.first_body + P.n_body;
   P.n_tiles = P.first_chunk + c_div_up(P.kv_chunk, kPage);
 
-  // this lane's query rows: column n of row tile nt is row 64 w + 16 nt + n
-  half8 qreg[4][4];
-  int qpos[4];
+  // this lane's query rows: column n of row tile nt is row 16 kNT w + 16 nt + n
+  half8 qreg[4][kNT];
+  int qpos[kNT];
 #pragma unroll
-  for (int nt = 0; nt < 4; ++nt) {
-    const int r = 64 * w + 16 * nt + n;
+  for (int nt = 0; nt < kNT; ++nt) {
+    const int r = 16 * kNT * w + 16 * nt + n;
     const int g = r / PB, pos = p0 + r % PB;
     const bool ok = g < G && pos < Tq;
     qpos[nt] = ok ? pos : -1;
@@ -433,9 +446,9 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
 #pragma unroll
   for (int ct = 0; ct < 8; ++ct)
 #pragma unroll
-    for (int nt = 0; nt < 4; ++nt) A.o[ct][nt] = float4v{0.f, 0.f, 0.f, 0.f};
+    for (int nt = 0; nt < kNT; ++nt) A.o[ct][nt] = float4v{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-  for (int nt = 0; nt < 4; ++nt) A.m[nt] = 0.f, A.l[nt] = 0.f;
+  for (int nt = 0; nt < kNT; ++nt) A.m[nt] = 0.f, A.l[nt] = 0.f;
   A.first = true;
   const float sc2 = scaling * kLog2e;
 
@@ -455,9 +468,9 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
     }
     const uint8_t* kt = lds + buf * kTile;
     const uint8_t* vt = lds + (2 + buf) * kTile;
-    int limit[4];
+    int limit[kNT];
 #pragma unroll
-    for (int nt = 0; nt < 4; ++nt)
+    for (int nt = 0; nt < kNT; ++nt)
       limit[nt] = cur.chunk_t0 >= 0 ? min(cur.ntok, qpos[nt] - cur.chunk_t0 + 1) : cur.ntok;
     const bool masked = cur.chunk_t0 >= 0 || cur.ntok < kPage;
 #pragma unroll 1
@@ -468,15 +481,15 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
     __syncthreads();
   }
 
-  // normalise and store: O^T[ct][nt][i] is channel slot 16 ct + 4 kg + i of row 64 w + 16 nt + n
+  // normalise and store: O^T[ct][nt][i] is channel slot 16 ct + 4 kg + i of row 16 kNT w + 16 nt + n
 #pragma unroll
-  for (int nt = 0; nt < 4; ++nt) {
+  for (int nt = 0; nt < kNT; ++nt) {
     float l = A.l[nt];
     l += xor_lanes(l, 16);
     l += xor_lanes(l, 32);
     if (qpos[nt] < 0) continue;
     const float inv = 1.f / l;
-    const int r = 64 * w + 16 * nt + n;
+    const int r = 16 * kNT * w + 16 * nt + n;
     const int g_ = r / PB;
     __half* orow = out + (((int64_t)b * Tq + qpos[nt]) * H_Q + (h * G + g_)) * kD;
 #pragma unroll
