@@ -11,8 +11,8 @@
 // group; wavefront w owns rows 64w .. 64w+63.  The workgroup walks the sequence in 128-token
 // tiles.  Each tile is brought into LDS once, as fp16, by all 256 threads: packed pages are
 // dequantized on the way (exactly the reference's two fp16 roundings), fp16 rows are copied.
-// Two tile buffers alternate: the global loads of tile t+1 are issued before the arithmetic on
-// tile t and its dequantization follows it, one barrier per tile.
+// Two tile buffers alternate: while tile t is multiplied, tile t+1 is converted into the other
+// buffer and the packed bytes of tile t+2 are in flight; one barrier per tile.
 //
 // Matrix-core formulation (v_mfma_f32_16x16x32_f16; lane = 16 kg + n holds A[n][8 k-slots],
 // B[8 k-slots][n], C[4kg .. 4kg+3][n]):
@@ -452,20 +452,33 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(kWaves
   A.first = true;
   const float sc2 = scaling * kLog2e;
 
-  Stage g;
-  TileSrc cur = P.tile(0);
-  P.issue(cur, g);
-  P.finish(cur, g, lds, lds + 2 * kTile);
+  // Software pipeline over tiles: tile t is multiplied from LDS buffer t & 1 while tile t+1 is
+  // turned into fp16 in the other buffer from registers loaded one iteration earlier, and the
+  // packed bytes of tile t+2 are on their way.  The waves of a SIMD take the two jobs in opposite
+  // order (waves 0..3 convert first, waves 4..7 multiply first), so that one does vector work
+  // while the other keeps the matrix pipe busy.  One barrier per tile.
+  const int nt_ = P.n_tiles;
+  const bool convert_first = w < kWaves / 2;
+  Stage ga, gb;                       // tile t+1, tile t+2
+  TileSrc cur = P.tile(0), nxt = cur, nn = cur;
+  P.issue(cur, ga);
+  P.finish(cur, ga, lds, lds + 2 * kTile);
+  if (nt_ > 1) {
+    nxt = P.tile(1);
+    P.issue(nxt, ga);
+  }
   __syncthreads();
 #pragma unroll 1
-  for (int t = 0; t < P.n_tiles; ++t) {
+  for (int t = 0; t < nt_; ++t) {
     const int buf = t & 1;
-    const bool more = t + 1 < P.n_tiles;
-    TileSrc nxt = cur;
-    if (more) {
-      nxt = P.tile(t + 1);
-      P.issue(nxt, g);
+    const bool more = t + 1 < nt_;
+    if (t + 2 < nt_) {
+      nn = P.tile(t + 2);
+      P.issue(nn, gb);
     }
+    uint8_t* kn = lds + (buf ^ 1) * kTile;
+    uint8_t* vn = lds + (2 + (buf ^ 1)) * kTile;
+    if (more && convert_first) P.finish(nxt, ga, kn, vn);
     const uint8_t* kt = lds + buf * kTile;
     const uint8_t* vt = lds + (2 + buf) * kTile;
     int limit[kNT];
@@ -476,8 +489,10 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(kWaves
 #pragma unroll 1
     for (int sub = 0; sub < 4; ++sub)
       if (32 * sub < cur.ntok) attend_sub(kt, vt, sub, qreg, A, sc2, masked, limit, kg, n);
-    if (more) P.finish(nxt, g, lds + (buf ^ 1) * kTile, lds + (2 + (buf ^ 1)) * kTile);
+    if (more && !convert_first) P.finish(nxt, ga, kn, vn);
     cur = nxt;
+    nxt = nn;
+    ga = gb;
     __syncthreads();
   }
 
