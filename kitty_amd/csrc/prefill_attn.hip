@@ -273,129 +273,144 @@ struct WaveAcc {
   bool first;
 };
 
-// 32 positions [32 sub, 32 sub + 32) of the tile in (kt, vt) against this wavefront's rows (a
-// sub-tile this small keeps the logits in 32 registers; the 128 accumulator registers and the 64
-// query registers leave room for little more).
+// One 128-token tile in (kt, vt) against this wavefront's rows, in sub-tiles of 32 positions (the
+// logits of a sub-tile fit 16 registers).  Software-pipelined: the QK^T MFMAs of sub-tile s+1 are
+// issued between the exponentials of sub-tile s, so that a wave's instruction stream mixes matrix
+// and vector work instead of alternating long runs of each.
 // limit[nt]: tokens of the tile with index < limit are visible to the row of column tile nt.
-__device__ __forceinline__ void attend_sub(const uint8_t* kt, const uint8_t* vt, int sub, const half8 (&q)[4][kNT],
-                                           WaveAcc& A, float sc2, bool masked, const int (&limit)[kNT], int kg,
-                                           int n) {
-  float4v S[2][kNT];
-#pragma unroll
-  for (int mt = 0; mt < 2; ++mt)
-#pragma unroll
-    for (int nt = 0; nt < kNT; ++nt) S[mt][nt] = float4v{0.f, 0.f, 0.f, 0.f};
-  // lane's corner inside a 16-lane transposing read: row n / 4 of 4, columns 4 (n % 4) ..
-  const int lane_off = (4 * kg + (n >> 2)) * kPitch + (n & 3) * 8;
-  const uint8_t* kbase = kt + lane_off + sub * 64;
-  // channel chunk c+1 is fetched while chunk c is multiplied; the fences keep the scheduler from
-  // hoisting every operand load to the top
-  half8 a_cur[2], a_nxt[2];
-#pragma unroll
-  for (int mt = 0; mt < 2; ++mt) a_cur[mt] = load_a(kbase + mt * 32);
-#pragma unroll
-  for (int c = 0; c < 4; ++c) {
-    if (c < 3) {
-#pragma unroll
-      for (int mt = 0; mt < 2; ++mt) a_nxt[mt] = load_a(kbase + (32 * (c + 1)) * kPitch + mt * 32);
-    }
+struct TileAttend {
+  const uint8_t* kb;   // K tile + this lane's corner of a transposing read
+  const uint8_t* vb;   // V tile + the same corner
+  const half8 (&q)[4][kNT];
+  WaveAcc& A;
+  const float sc2;
+  const bool masked;
+  const int (&limit)[kNT];
+  const int kg;
+
+  __device__ __forceinline__ void qk_issue(int sub, float4v (&S)[2][kNT]) const {
 #pragma unroll
     for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
-      for (int nt = 0; nt < kNT; ++nt)
-        S[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a_cur[mt], q[c][nt], S[mt][nt], 0, 0, 0);
-    __builtin_amdgcn_sched_barrier(0);
+      for (int nt = 0; nt < kNT; ++nt) S[mt][nt] = float4v{0.f, 0.f, 0.f, 0.f};
+    const uint8_t* kbase = kb + sub * 64;
 #pragma unroll
-    for (int mt = 0; mt < 2; ++mt) a_cur[mt] = a_nxt[mt];
+    for (int c = 0; c < 4; ++c)
+#pragma unroll
+      for (int mt = 0; mt < 2; ++mt) {
+        const half8 a = load_a(kbase + (32 * c) * kPitch + mt * 32);
+#pragma unroll
+        for (int nt = 0; nt < kNT; ++nt) S[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, q[c][nt], S[mt][nt], 0, 0, 0);
+      }
   }
-  // the first value operands travel while the softmax runs
-  const uint8_t* vbase = vt + lane_off + (32 * sub) * kPitch;
-  half8 v_cur[2], v_nxt[2];
-  v_cur[0] = load_a(vbase);
-  v_cur[1] = load_a(vbase + 32);
 
-  // online softmax, column by column (a column = one query row, spread over the 4 lane groups)
-#pragma unroll
-  for (int nt = 0; nt < kNT; ++nt)
-#pragma unroll
-    for (int mt = 0; mt < 2; ++mt) S[mt][nt] = S[mt][nt] * sc2 - A.m[nt];
-  if (masked) {   // one wave-uniform branch: partial tiles and the chunk's own tiles only
+  // scale, mask, column maxima, and the (rare, wave-uniform) move of the running maxima
+  __device__ __forceinline__ void softmax_head(int sub, float4v (&S)[2][kNT]) const {
 #pragma unroll
     for (int nt = 0; nt < kNT; ++nt)
+#pragma unroll
+      for (int mt = 0; mt < 2; ++mt) S[mt][nt] = S[mt][nt] * sc2 - A.m[nt];
+    if (masked) {   // one wave-uniform branch: partial tiles and the chunk's own tiles only
+#pragma unroll
+      for (int nt = 0; nt < kNT; ++nt)
+#pragma unroll
+        for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const int tok = 32 * sub + 16 * mt + 2 * kg + (i >> 1) + 8 * (i & 1);
+            if (tok >= limit[nt]) S[mt][nt][i] = -INFINITY;
+          }
+      asm volatile("" ::: "memory");   // keep this a branch, not selects on every tile
+    }
+    float mt_[kNT];
+#pragma unroll
+    for (int nt = 0; nt < kNT; ++nt) {
+      float mx = fmaxf(fmaxf(S[0][nt][0], S[0][nt][1]), fmaxf(S[0][nt][2], S[0][nt][3]));
+      mx = fmaxf(mx, fmaxf(fmaxf(S[1][nt][0], S[1][nt][1]), fmaxf(S[1][nt][2], S[1][nt][3])));
+      mx = fmaxf(mx, xor_lanes(mx, 16));
+      mx = fmaxf(mx, xor_lanes(mx, 32));
+      mt_[nt] = mx;
+    }
+    bool move = A.first;
+#pragma unroll
+    for (int nt = 0; nt < kNT; ++nt) move = move || mt_[nt] > 0.f;
+    if (__any(move)) {
+#pragma unroll
+      for (int nt = 0; nt < kNT; ++nt) {
+        const float dm = A.first ? mt_[nt] : fmaxf(mt_[nt], 0.f);
+#pragma unroll
+        for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) S[mt][nt][i] -= dm;
+        if (!A.first) {
+          const float alpha = __builtin_amdgcn_exp2f(-dm);
+          A.l[nt] *= alpha;
+#pragma unroll
+          for (int ct = 0; ct < 8; ++ct) A.o[ct][nt] *= alpha;
+        }
+        A.m[nt] += dm;
+      }
+      A.first = false;
+    }
+  }
+
+  // exponentials, row sums, fp16 probabilities
+  __device__ __forceinline__ void softmax_tail(float4v (&S)[2][kNT], half8 (&p)[kNT]) const {
+#pragma unroll
+    for (int nt = 0; nt < kNT; ++nt) {
+      float sum = 0.f;
 #pragma unroll
       for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          const int tok = 32 * sub + 16 * mt + 2 * kg + (i >> 1) + 8 * (i & 1);
-          if (tok >= limit[nt]) S[mt][nt][i] = -INFINITY;
+          const float e = __builtin_amdgcn_exp2f(S[mt][nt][i]);
+          S[mt][nt][i] = e;
+          sum += e;
         }
-    asm volatile("" ::: "memory");   // keep this a branch, not 32 selects on every tile
+      A.l[nt] += sum;
+      const float4v x0 = S[0][nt], x1 = S[1][nt];
+      p[nt] = half8{(_Float16)x0[0], (_Float16)x0[1], (_Float16)x0[2], (_Float16)x0[3],
+                    (_Float16)x1[0], (_Float16)x1[1], (_Float16)x1[2], (_Float16)x1[3]};
+    }
   }
-  float mt_[kNT];
+
+  __device__ __forceinline__ void pv(int sub, const half8 (&p)[kNT]) const {
+    const uint8_t* vbase = vb + (32 * sub) * kPitch;
 #pragma unroll
-  for (int nt = 0; nt < kNT; ++nt) {
-    float mx = fmaxf(fmaxf(S[0][nt][0], S[0][nt][1]), fmaxf(S[0][nt][2], S[0][nt][3]));
-    mx = fmaxf(mx, fmaxf(fmaxf(S[1][nt][0], S[1][nt][1]), fmaxf(S[1][nt][2], S[1][nt][3])));
-    mx = fmaxf(mx, xor_lanes(mx, 16));
-    mx = fmaxf(mx, xor_lanes(mx, 32));
-    mt_[nt] = mx;
+    for (int ct = 0; ct < 8; ++ct) {
+      const half8 a = load_a(vbase + ct * 32);
+#pragma unroll
+      for (int nt = 0; nt < kNT; ++nt) A.o[ct][nt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, p[nt], A.o[ct][nt], 0, 0, 0);
+    }
   }
-  bool move = A.first;
+
+  __device__ __forceinline__ void run(int nsub) const {
+    float4v Sc[2][kNT], Sn[2][kNT];
+    half8 p[kNT];
+    qk_issue(0, Sc);
+#pragma unroll 1
+    for (int sub = 0; sub + 1 < nsub; ++sub) {
+      softmax_head(sub, Sc);
+      // one basic block: 16 operand reads + 16 kNT MFMAs of the next sub-tile between the vector work
+      softmax_tail(Sc, p);
+      qk_issue(sub + 1, Sn);
 #pragma unroll
-  for (int nt = 0; nt < kNT; ++nt) move = move || mt_[nt] > 0.f;
-  if (__any(move)) {
-#pragma unroll
-    for (int nt = 0; nt < kNT; ++nt) {
-      const float dm = A.first ? mt_[nt] : fmaxf(mt_[nt], 0.f);
+      for (int k = 0; k < 16; ++k) {
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);     // one LDS read
+        __builtin_amdgcn_sched_group_barrier(0x008, kNT, 0);   // its MFMAs
+        __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);     // a few vector instructions
+      }
+      pv(sub, p);
 #pragma unroll
       for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) S[mt][nt][i] -= dm;
-      if (!A.first) {
-        const float alpha = __builtin_amdgcn_exp2f(-dm);
-        A.l[nt] *= alpha;
-#pragma unroll
-        for (int ct = 0; ct < 8; ++ct) A.o[ct][nt] *= alpha;
-      }
-      A.m[nt] += dm;
+        for (int nt = 0; nt < kNT; ++nt) Sc[mt][nt] = Sn[mt][nt];
     }
-    A.first = false;
+    softmax_head(nsub - 1, Sc);
+    softmax_tail(Sc, p);
+    pv(nsub - 1, p);
   }
-  half8 p[kNT];
-#pragma unroll
-  for (int nt = 0; nt < kNT; ++nt) {
-    float sum = 0.f;
-#pragma unroll
-    for (int mt = 0; mt < 2; ++mt)
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const float e = __builtin_amdgcn_exp2f(S[mt][nt][i]);
-        S[mt][nt][i] = e;
-        sum += e;
-      }
-    A.l[nt] += sum;
-    const float4v x0 = S[0][nt], x1 = S[1][nt];
-    p[nt] = half8{(_Float16)x0[0], (_Float16)x0[1], (_Float16)x0[2], (_Float16)x0[3],
-                  (_Float16)x1[0], (_Float16)x1[1], (_Float16)x1[2], (_Float16)x1[3]};
-  }
-  // 4 groups of two channel-slot tiles; group i+1 is fetched while group i is multiplied
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int ct = 2 * i;
-    if (i < 3) {
-      v_nxt[0] = load_a(vbase + (ct + 2) * 32);
-      v_nxt[1] = load_a(vbase + (ct + 3) * 32);
-    }
-#pragma unroll
-    for (int j = 0; j < 2; ++j)
-#pragma unroll
-      for (int nt = 0; nt < kNT; ++nt)
-        A.o[ct + j][nt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(v_cur[j], p[nt], A.o[ct + j][nt], 0, 0, 0);
-    __builtin_amdgcn_sched_barrier(0);
-    v_cur[0] = v_nxt[0];
-    v_cur[1] = v_nxt[1];
-  }
-}
+};
 
 template <bool BOOST>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(kWaves / 4, kWaves / 4))) void prefill_attn_kernel(
@@ -479,16 +494,20 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(kWaves
     uint8_t* kn = lds + (buf ^ 1) * kTile;
     uint8_t* vn = lds + (2 + (buf ^ 1)) * kTile;
     if (more && convert_first) P.finish(nxt, ga, kn, vn);
-    const uint8_t* kt = lds + buf * kTile;
-    const uint8_t* vt = lds + (2 + buf) * kTile;
     int limit[kNT];
 #pragma unroll
     for (int nt = 0; nt < kNT; ++nt)
       limit[nt] = cur.chunk_t0 >= 0 ? min(cur.ntok, qpos[nt] - cur.chunk_t0 + 1) : cur.ntok;
     const bool masked = cur.chunk_t0 >= 0 || cur.ntok < kPage;
-#pragma unroll 1
-    for (int sub = 0; sub < 4; ++sub)
-      if (32 * sub < cur.ntok) attend_sub(kt, vt, sub, qreg, A, sc2, masked, limit, kg, n);
+    {
+      // the lane's corner inside a 16-lane transposing read: row n / 4 of 4, columns 4 (n % 4) ..;
+      // made opaque so that every read's offset stays a small immediate on these two bases
+      uint32_t ok_ = buf * kTile + (4 * kg + (n >> 2)) * kPitch + (n & 3) * 8;
+      uint32_t ov_ = ok_ + 2 * kTile;
+      asm volatile("" : "+v"(ok_), "+v"(ov_));
+      const TileAttend T{lds + ok_, lds + ov_, qreg, A, sc2, masked, limit, kg};
+      T.run((cur.ntok + 31) >> 5);
+    }
     if (more && !convert_first) P.finish(nxt, ga, kn, vn);
     cur = nxt;
     nxt = nn;
