@@ -30,6 +30,9 @@
 // the same token permutation, the output undoes the channel permutation.
 #include "decode_common.h"
 
+// wave priority while a wave issues the PV MFMAs (the other wave of the SIMD fills the gaps)
+#define KITTY_PV_PRIO 2
+
 namespace kitty {
 namespace {
 
@@ -400,7 +403,9 @@ struct TileAttend {
         __builtin_amdgcn_sched_group_barrier(0x008, kNT, 0);   // its MFMAs
         __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);     // a few vector instructions
       }
+      __builtin_amdgcn_s_setprio(KITTY_PV_PRIO);
       pv(sub, p);
+      __builtin_amdgcn_s_setprio(0);
 #pragma unroll
       for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
