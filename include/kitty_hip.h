@@ -34,7 +34,8 @@ enum {
 
 /*
  * One layer's storage, field for field the tensors of the reference's KVCache_Layer
- * (utils_kv_per_layer.py:12-95).  Strides are in bytes.  fp16 windows are [MAX_BS, H_KV, rows, D]
+ * (utils_kv_per_layer.py:12-95).  Strides are in bytes, except the page-table row strides, which
+ * count int64 entries.  fp16 windows are [MAX_BS, H_KV, rows, D]
  * with D contiguous; *_stride_b / *_stride_h give their batch and head strides.
  *
  * Occupancy is given either by the scalar counters (the reference: host ints shared by the whole
@@ -62,8 +63,8 @@ typedef struct kitty_kv_layer {
   const void*    key_meta;     int64_t key_meta_stride_page;      /* KeyCache_metadata   */
   const uint8_t* value_cache;  int64_t value_cache_stride_page;   /* ValueCache          */
   const void*    value_meta;   int64_t value_meta_stride_page;    /* ValueCache_metadata */
-  const int64_t* page_table_k; int64_t page_table_k_stride_b;     /* PageTable_K         */
-  const int64_t* page_table_v; int64_t page_table_v_stride_b;     /* PageTable_V         */
+  const int64_t* page_table_k; int64_t page_table_k_stride_b;     /* PageTable_K, stride in entries */
+  const int64_t* page_table_v; int64_t page_table_v_stride_b;     /* PageTable_V, stride in entries */
 
   const void* sink_k;  const void* sink_v;      /* Sink_Buffer_K/V  [MAX_BS,H_KV,S,D]         */
   int64_t sink_stride_b, sink_stride_h;
@@ -92,7 +93,8 @@ int kitty_select_boost_k(const void* key, int64_t stride_b, int64_t stride_h, in
  * Quantizes `pages` pages of every (b,h) into cache pages page_table[b][page_offset + p].
  * slot_map NULL: the selection above is fused into the same kernel (one pass over K).
  * slot_map given: uint8 [B,H,pages,D], consumed exactly like the reference kernel consumes
- * dense_sparse_idx.  meta is fp16 [pages_total,H,D,2] (scale, zero).
+ * dense_sparse_idx.  meta is fp16 [pages_total,H,D,2] (scale, zero).  page_table_stride_b counts
+ * int64 entries; every other stride is in bytes.
  */
 int kitty_quant_pack_k(const void* key, int64_t stride_b, int64_t stride_h, int64_t stride_t,
                        int B, int H, int T, int D, int t_offset, int pages, int page_size, int d_boost,
