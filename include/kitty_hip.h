@@ -57,7 +57,8 @@ enum {
 typedef struct kitty_kv_layer {
   int32_t H_KV, D, D_BOOSTED, PAGE_SIZE, S, MAX_PAGE;
   int32_t counts[KITTY_SEQ_COUNT_FIELDS];       /* used when seq_counts == NULL */
-  const int32_t* seq_counts;                    /* optional, device, [B][8] */
+  const int32_t* seq_counts;                    /* optional, device, [B][8]; the two append
+                                                   entry points below write it */
 
   const uint8_t* key_cache;    int64_t key_cache_stride_page;     /* KeyCache            */
   const void*    key_meta;     int64_t key_meta_stride_page;      /* KeyCache_metadata   */
@@ -161,6 +162,29 @@ int kitty_prefill_attn(const kitty_kv_layer* layer,
                        const void* k_new, const void* v_new,
                        int64_t new_stride_b, int64_t new_stride_h, int64_t new_stride_t,
                        int B, int H_Q, int T_q, float scaling, void* out, void* stream);
+
+/*
+ * Decode-time bookkeeping with per-sequence counters kept on the device (layer->seq_counts must be
+ * set; it is read AND written).  The reference keeps one set of host ints for the whole batch and
+ * drives slice copies from them (KittyCache.update, kitty.py:97-123; quantize_decode,
+ * kitty.py:194-236); these two calls run the same state machine per sequence, with no host
+ * round trip, so that sequences of different lengths decode in one batch and the launch sequence
+ * of a decode step never changes (a captured graph can replay it).  Call order per step, as in
+ * modeling_qwen3.py:225-251: kitty_append_token, kitty_decode_attn, kitty_flush_full.
+ *
+ * kitty_append_token: one token per sequence.  k_new / v_new: fp16 [B,H_KV,1,D], D contiguous, byte
+ * strides.  Per sequence: sink not full -> the sink row; else K -> Q_Buffer_K[Q_Buffer_Count_K],
+ * V -> the local ring (a full ring first moves its oldest row to Q_Buffer_V).  A sequence whose
+ * Q-buffer is full (a skipped kitty_flush_full) is left unchanged and the token dropped.
+ *
+ * kitty_flush_full: every sequence whose K (V) Q-buffer holds PAGE_SIZE rows gets it quantized,
+ * with channel selection, into page page_table[b][PageCount] and its counters advanced; the
+ * arithmetic is that of kitty_quant_pack_k / _v.  A sequence already at MAX_PAGE pages, or whose
+ * page id is outside [0, cache_pages), is left as it is.
+ */
+int kitty_append_token(const kitty_kv_layer* layer, const void* k_new, const void* v_new,
+                       int64_t stride_b, int64_t stride_h, int B, void* stream);
+int kitty_flush_full(const kitty_kv_layer* layer, int B, int64_t cache_pages, void* stream);
 
 #ifdef __cplusplus
 }

@@ -56,6 +56,8 @@ _SIGNATURES = {
                                   c_size_t, c_int, c_int, c_void_p]),
     "kitty_prefill_attn": (c_int, [POINTER(KittyKVLayer), c_void_p, c_int64, c_int64, c_int64, c_void_p, c_void_p,
                                    c_int64, c_int64, c_int64, c_int, c_int, c_int, c_float, c_void_p, c_void_p]),
+    "kitty_append_token": (c_int, [POINTER(KittyKVLayer), c_void_p, c_void_p, c_int64, c_int64, c_int, c_void_p]),
+    "kitty_flush_full": (c_int, [POINTER(KittyKVLayer), c_int, c_int64, c_void_p]),
 }
 
 EXPORTS = tuple(_SIGNATURES)

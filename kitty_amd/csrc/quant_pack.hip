@@ -79,16 +79,14 @@ __device__ __forceinline__ uint32_t gather_fields(uint32_t n) {
   return x & 0xffffu;
 }
 
-// MODE 0: slot map given.  MODE 1: selection fused, then quantize.  MODE 2: selection only.
+// One K page of one head.  MODE 0: slot map given.  MODE 1: selection fused, then quantize.
+// MODE 2: selection only.  src: the page's first token row of this head; slot_in / slot_out: 128
+// bytes (or NULL); dst: the page-head in the cache, meta_dst: its 128 (scale, zero) pairs.
+// Called by all 256 threads of a workgroup.
 template <int MODE>
-__global__ __launch_bounds__(256) void quant_pack_k_kernel(
-    const uint8_t* __restrict__ key, int64_t stride_b, int64_t stride_h, int64_t stride_t,
-    int t_offset, int d_boost,
-    const uint8_t* __restrict__ slot_map_in, uint8_t* __restrict__ slot_map_out, int pages,
-    const int64_t* __restrict__ page_table, int64_t pt_stride_b, int page_offset,
-    uint8_t* __restrict__ cache, int64_t cache_stride_page,
-    uint8_t* __restrict__ meta, int64_t meta_stride_page, int64_t cache_pages) {
-  const int p = blockIdx.x, h = blockIdx.y, b = blockIdx.z, H = gridDim.y;
+__device__ __forceinline__ void quant_k_page(const uint8_t* __restrict__ src_page, int64_t stride_t, int d_boost,
+                                             const uint8_t* __restrict__ slot_in, uint8_t* __restrict__ slot_out,
+                                             uint8_t* __restrict__ dst, uint8_t* __restrict__ meta_dst) {
   const int tid = threadIdx.x;
   const int tg = tid >> 4;   // tokens tg*8 .. tg*8+7
   const int c8 = tid & 15;   // channels c8*8 .. c8*8+7
@@ -101,8 +99,7 @@ __global__ __launch_bounds__(256) void quant_pack_k_kernel(
   __shared__ __attribute__((aligned(16))) uint8_t s_idx[kD];
   __shared__ __attribute__((aligned(16))) uint16_t s_lo[kD * 16];
 
-  const uint8_t* src = key + (int64_t)b * stride_b + (int64_t)h * stride_h +
-                       (int64_t)(t_offset + p * kPage + tg * 8) * stride_t + c8 * 16;
+  const uint8_t* src = src_page + (int64_t)(tg * 8) * stride_t + c8 * 16;
   uint4 rows[8];
 #pragma unroll
   for (int r = 0; r < 8; ++r) rows[r] = *(const uint4*)(src + (int64_t)r * stride_t);
@@ -144,7 +141,7 @@ __global__ __launch_bounds__(256) void quant_pack_k_kernel(
       // an integer below 2^47 (or inf / nan for non-finite inputs, which saturate)
       s_score[tid] = mean_abs_fp16_bits(sum < 1.8e19 ? (uint64_t)(sum * 16777216.0) : ~0ull);
     } else {
-      s_idx[tid] = slot_map_in[(((int64_t)b * H + h) * pages + p) * kD + tid];
+      s_idx[tid] = slot_in[tid];
     }
   }
   if (MODE != 0) {
@@ -160,14 +157,10 @@ __global__ __launch_bounds__(256) void quant_pack_k_kernel(
       }
       const uint8_t slot = (uint8_t)(rank < d_boost ? rank : d_boost);
       s_idx[tid] = slot;
-      if (slot_map_out) slot_map_out[(((int64_t)b * H + h) * pages + p) * kD + tid] = slot;
+      if (slot_out) slot_out[tid] = slot;
     }
     if (MODE == 2) return;
   }
-
-  const int64_t pg = page_table[(int64_t)b * pt_stride_b + page_offset + p];
-  if (pg < 0 || pg >= cache_pages) return;   // never write outside the cache
-  uint8_t* dst = cache + pg * cache_stride_page + (int64_t)h * k_head_bytes(d_boost);
 
   if (tid < kD) {
     const bool boosted = s_idx[tid] < d_boost;
@@ -177,7 +170,7 @@ __global__ __launch_bounds__(256) void quant_pack_k_kernel(
     const Divisor k = make_divisor(scale);
     s_q[tid] = float4{ch_min, k.d, k.r, qmax + 0.5f};
     __half2 m2 = __halves2half2(__float2half_rn(scale), __float2half_rn(ch_min));
-    *(__half2*)(meta + pg * meta_stride_page + ((int64_t)h * kD + tid) * 4) = m2;
+    *(__half2*)(meta_dst + tid * 4) = m2;
   }
   __syncthreads();
 
@@ -202,22 +195,36 @@ __global__ __launch_bounds__(256) void quant_pack_k_kernel(
   if (tid < kD / 4) ((uint32_t*)(dst + kRowBytes * (kD + d_boost)))[tid] = ((const uint32_t*)s_idx)[tid];
 }
 
-// 256 threads: 8 consecutive lanes share a token (16 channels each), 4 tokens per thread.
-__global__ __launch_bounds__(256) void quant_pack_v_kernel(
-    const uint8_t* __restrict__ value, int64_t stride_b, int64_t stride_h, int64_t stride_t,
-    int t_offset,
+template <int MODE>
+__global__ __launch_bounds__(256) void quant_pack_k_kernel(
+    const uint8_t* __restrict__ key, int64_t stride_b, int64_t stride_h, int64_t stride_t,
+    int t_offset, int d_boost,
+    const uint8_t* __restrict__ slot_map_in, uint8_t* __restrict__ slot_map_out, int pages,
     const int64_t* __restrict__ page_table, int64_t pt_stride_b, int page_offset,
     uint8_t* __restrict__ cache, int64_t cache_stride_page,
     uint8_t* __restrict__ meta, int64_t meta_stride_page, int64_t cache_pages) {
-  const int p = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+  const int p = blockIdx.x, h = blockIdx.y, b = blockIdx.z, H = gridDim.y;
+  const uint8_t* src = key + (int64_t)b * stride_b + (int64_t)h * stride_h + (int64_t)(t_offset + p * kPage) * stride_t;
+  const int64_t slot_off = (((int64_t)b * H + h) * pages + p) * kD;
+  uint8_t* dst = nullptr;
+  uint8_t* mdst = nullptr;
+  if (MODE != 2) {
+    const int64_t pg = page_table[(int64_t)b * pt_stride_b + page_offset + p];
+    if (pg < 0 || pg >= cache_pages) return;   // never write outside the cache
+    dst = cache + pg * cache_stride_page + (int64_t)h * k_head_bytes(d_boost);
+    mdst = meta + pg * meta_stride_page + (int64_t)h * kD * 4;
+  }
+  quant_k_page<MODE>(src, stride_t, d_boost, slot_map_in ? slot_map_in + slot_off : nullptr,
+                     slot_map_out ? slot_map_out + slot_off : nullptr, dst, mdst);
+}
+
+// One V page of one head: 256 threads, 8 consecutive lanes share a token (16 channels each), 4
+// tokens per thread.  src: the page's first token row of this head.
+__device__ __forceinline__ void quant_v_page(const uint8_t* __restrict__ src_page, int64_t stride_t,
+                                             uint8_t* __restrict__ dst, uint8_t* __restrict__ mdst) {
   const int tid = threadIdx.x;
   const int cg = tid & 7;
-  const int64_t pg = page_table[(int64_t)b * pt_stride_b + page_offset + p];
-  if (pg < 0 || pg >= cache_pages) return;
-  uint8_t* dst = cache + pg * cache_stride_page + (int64_t)h * kVBytes;
-  uint8_t* mdst = meta + pg * meta_stride_page + (int64_t)h * kPage * 4;
-  const uint8_t* src = value + (int64_t)b * stride_b + (int64_t)h * stride_h +
-                       (int64_t)(t_offset + p * kPage) * stride_t + cg * 32;
+  const uint8_t* src = src_page + cg * 32;
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int t = (tid >> 3) + 32 * i;
@@ -251,6 +258,112 @@ __global__ __launch_bounds__(256) void quant_pack_v_kernel(
     const uint32_t packed = (uint32_t)h0 | ((uint32_t)h1 << 16);
     *(uint32_t*)(dst + t * kRowBytes + cg * 4) = packed;
     if (cg == 0) *(__half2*)(mdst + t * 4) = __halves2half2(__float2half_rn(scale), __float2half_rn(mn));
+  }
+}
+
+__global__ __launch_bounds__(256) void quant_pack_v_kernel(
+    const uint8_t* __restrict__ value, int64_t stride_b, int64_t stride_h, int64_t stride_t,
+    int t_offset,
+    const int64_t* __restrict__ page_table, int64_t pt_stride_b, int page_offset,
+    uint8_t* __restrict__ cache, int64_t cache_stride_page,
+    uint8_t* __restrict__ meta, int64_t meta_stride_page, int64_t cache_pages) {
+  const int p = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+  const int64_t pg = page_table[(int64_t)b * pt_stride_b + page_offset + p];
+  if (pg < 0 || pg >= cache_pages) return;
+  quant_v_page(value + (int64_t)b * stride_b + (int64_t)h * stride_h + (int64_t)(t_offset + p * kPage) * stride_t,
+               stride_t, cache + pg * cache_stride_page + (int64_t)h * kVBytes,
+               meta + pg * meta_stride_page + (int64_t)h * kPage * 4);
+}
+
+// ---------------------------------------------------------------------------------------------
+// Decode-time append and flush with per-sequence counters on the device (int32 [B][8], the
+// KITTY_CNT_* fields).  The state machine is KittyCache.update's decode branch (kitty.py:97-123)
+// and quantize_decode (kitty.py:194-236), per sequence instead of per batch.
+// ---------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void append_token_kernel(kitty_kv_layer L, const uint8_t* __restrict__ k_new,
+                                                           const uint8_t* __restrict__ v_new, int64_t stride_b,
+                                                           int64_t stride_h) {
+  const int b = blockIdx.x;
+  int32_t* cnt = const_cast<int32_t*>(L.seq_counts) + b * KITTY_SEQ_COUNT_FIELDS;
+  const int sink = cnt[KITTY_CNT_SINK], rk = cnt[KITTY_CNT_QBUF_K], rv = cnt[KITTY_CNT_QBUF_V];
+  const int lv = cnt[KITTY_CNT_LOCAL_V], off = cnt[KITTY_CNT_LOCAL_OFF] & (kPage - 1);
+  const bool to_sink = sink < L.S;
+  // a full Q-buffer means the caller skipped a flush: drop the token rather than write out of bounds
+  const bool ok = to_sink || (rk < kPage && (lv < kPage || rv < kPage));
+  __syncthreads();   // every thread has read the counters before thread 0 rewrites them
+  if (ok) {
+    for (int i = threadIdx.x; i < L.H_KV * 32; i += blockDim.x) {
+      const int h = i >> 5, part = (i & 31) * 8;   // 8 bytes = 4 channels
+      const uint2 kk = *(const uint2*)(k_new + (int64_t)b * stride_b + (int64_t)h * stride_h + part);
+      const uint2 vv = *(const uint2*)(v_new + (int64_t)b * stride_b + (int64_t)h * stride_h + part);
+      if (to_sink) {
+        const int64_t o = (int64_t)b * L.sink_stride_b + (int64_t)h * L.sink_stride_h + (int64_t)sink * (kD * 2) + part;
+        *(uint2*)((uint8_t*)L.sink_k + o) = kk;
+        *(uint2*)((uint8_t*)L.sink_v + o) = vv;
+      } else {
+        const int64_t w = (int64_t)b * L.win_stride_b + (int64_t)h * L.win_stride_h + part;
+        *(uint2*)((uint8_t*)L.qbuf_k + w + (int64_t)rk * (kD * 2)) = kk;
+        if (lv < kPage) {
+          *(uint2*)((uint8_t*)L.local_v + w + (int64_t)lv * (kD * 2)) = vv;
+        } else {   // ring full: its oldest row moves to the V Q-buffer, the new one takes the slot
+          uint2* slot = (uint2*)((uint8_t*)L.local_v + w + (int64_t)off * (kD * 2));
+          *(uint2*)((uint8_t*)L.qbuf_v + w + (int64_t)rv * (kD * 2)) = *slot;
+          *slot = vv;
+        }
+      }
+    }
+    if (threadIdx.x == 0) {
+      if (to_sink) {
+        cnt[KITTY_CNT_SINK] = sink + 1;
+      } else {
+        cnt[KITTY_CNT_QBUF_K] = rk + 1;
+        if (lv < kPage) {
+          cnt[KITTY_CNT_LOCAL_V] = lv + 1;
+        } else {
+          cnt[KITTY_CNT_QBUF_V] = rv + 1;
+          cnt[KITTY_CNT_LOCAL_OFF] = (off + 1) & (kPage - 1);
+        }
+      }
+    }
+  }
+}
+
+// blockIdx.z = 0: the K Q-buffer of (b, h) if it is full; 1: the V Q-buffer.
+__global__ __launch_bounds__(256) void flush_full_kernel(kitty_kv_layer L, int64_t cache_pages) {
+  const int h = blockIdx.x, b = blockIdx.y;
+  const int32_t* cnt = L.seq_counts + b * KITTY_SEQ_COUNT_FIELDS;
+  const int64_t w = (int64_t)b * L.win_stride_b + (int64_t)h * L.win_stride_h;
+  if (blockIdx.z == 0) {
+    const int pk = cnt[KITTY_CNT_PAGES_K];
+    if (cnt[KITTY_CNT_QBUF_K] != kPage || pk < 0 || pk >= L.MAX_PAGE) return;
+    const int64_t pg = L.page_table_k[(int64_t)b * L.page_table_k_stride_b + pk];
+    if (pg < 0 || pg >= cache_pages) return;
+    quant_k_page<1>((const uint8_t*)L.qbuf_k + w, kD * 2, L.D_BOOSTED, nullptr, nullptr,
+                    const_cast<uint8_t*>(L.key_cache) + pg * L.key_cache_stride_page + (int64_t)h * k_head_bytes(L.D_BOOSTED),
+                    (uint8_t*)L.key_meta + pg * L.key_meta_stride_page + (int64_t)h * kD * 4);
+  } else {
+    const int pv = cnt[KITTY_CNT_PAGES_V];
+    if (cnt[KITTY_CNT_QBUF_V] != kPage || pv < 0 || pv >= L.MAX_PAGE) return;
+    const int64_t pg = L.page_table_v[(int64_t)b * L.page_table_v_stride_b + pv];
+    if (pg < 0 || pg >= cache_pages) return;
+    quant_v_page((const uint8_t*)L.qbuf_v + w, kD * 2,
+                 const_cast<uint8_t*>(L.value_cache) + pg * L.value_cache_stride_page + (int64_t)h * kVBytes,
+                 (uint8_t*)L.value_meta + pg * L.value_meta_stride_page + (int64_t)h * kPage * 4);
+  }
+}
+
+// after flush_full_kernel: the flushed Q-buffers are empty, their pages count
+__global__ void advance_counts_kernel(kitty_kv_layer L, int B) {
+  const int b = blockIdx.x * blockDim.x + threadIdx.x;
+  if (b >= B) return;
+  int32_t* cnt = const_cast<int32_t*>(L.seq_counts) + b * KITTY_SEQ_COUNT_FIELDS;
+  if (cnt[KITTY_CNT_QBUF_K] == kPage && cnt[KITTY_CNT_PAGES_K] >= 0 && cnt[KITTY_CNT_PAGES_K] < L.MAX_PAGE) {
+    cnt[KITTY_CNT_PAGES_K] += 1;
+    cnt[KITTY_CNT_QBUF_K] = 0;
+  }
+  if (cnt[KITTY_CNT_QBUF_V] == kPage && cnt[KITTY_CNT_PAGES_V] >= 0 && cnt[KITTY_CNT_PAGES_V] < L.MAX_PAGE) {
+    cnt[KITTY_CNT_PAGES_V] += 1;
+    cnt[KITTY_CNT_QBUF_V] = 0;
   }
 }
 
@@ -343,4 +456,55 @@ extern "C" int kitty_quant_pack_v(const void* value, int64_t stride_b, int64_t s
                      page_table_stride_b, page_offset, cache, cache_stride_page, (uint8_t*)meta, meta_stride_page,
                      cache_pages);
   return check_launch("kitty_quant_pack_v");
+}
+
+namespace {
+int check_append_layer(const kitty_kv_layer* layer, int B) {
+  KITTY_REQUIRE(layer != nullptr, KITTY_E_NULL, "layer is NULL");
+  const kitty_kv_layer& L = *layer;
+  KITTY_REQUIRE(L.seq_counts != nullptr, KITTY_E_NULL, "this entry point needs per-sequence counters (seq_counts)");
+  KITTY_REQUIRE(L.D == kD && L.PAGE_SIZE == kPage, KITTY_E_SHAPE,
+                "kernels are built for head_dim 128 and page_size 128, got D=%d page_size=%d", L.D, L.PAGE_SIZE);
+  KITTY_REQUIRE(L.H_KV >= 1 && L.H_KV <= 65535 && B >= 1 && B <= 65535, KITTY_E_RANGE, "bad H_KV=%d or B=%d", L.H_KV, B);
+  KITTY_REQUIRE(L.S >= 0 && L.S <= kPage && L.MAX_PAGE >= 0 && L.D_BOOSTED >= 0 && L.D_BOOSTED <= kD &&
+                    k_head_bytes(L.D_BOOSTED) % 16 == 0,
+                KITTY_E_SHAPE, "bad S=%d, MAX_PAGE=%d or D_BOOSTED=%d", L.S, L.MAX_PAGE, L.D_BOOSTED);
+  KITTY_REQUIRE(L.key_cache && L.key_meta && L.value_cache && L.value_meta && L.page_table_k && L.page_table_v &&
+                    L.sink_k && L.sink_v && L.qbuf_k && L.qbuf_v && L.local_v,
+                KITTY_E_NULL, "a cache tensor pointer is NULL");
+  KITTY_REQUIRE(((uintptr_t)L.key_cache % 16) == 0 && L.key_cache_stride_page % 16 == 0 &&
+                    ((uintptr_t)L.value_cache % 16) == 0 && L.value_cache_stride_page % 16 == 0 &&
+                    ((uintptr_t)L.key_meta % 4) == 0 && L.key_meta_stride_page % 4 == 0 &&
+                    ((uintptr_t)L.value_meta % 4) == 0 && L.value_meta_stride_page % 4 == 0 &&
+                    ((uintptr_t)L.sink_k % 16) == 0 && ((uintptr_t)L.sink_v % 16) == 0 &&
+                    ((uintptr_t)L.qbuf_k % 16) == 0 && ((uintptr_t)L.qbuf_v % 16) == 0 &&
+                    ((uintptr_t)L.local_v % 16) == 0 && L.sink_stride_b % 16 == 0 && L.sink_stride_h % 16 == 0 &&
+                    L.win_stride_b % 16 == 0 && L.win_stride_h % 16 == 0 && ((uintptr_t)L.seq_counts % 4) == 0,
+                KITTY_E_ALIGN, "cache tensors need 16-byte alignment");
+  KITTY_REQUIRE(L.key_cache_stride_page >= (int64_t)L.H_KV * k_head_bytes(L.D_BOOSTED) &&
+                    L.value_cache_stride_page >= (int64_t)L.H_KV * kVBytes &&
+                    L.key_meta_stride_page >= (int64_t)L.H_KV * kD * 4 &&
+                    L.value_meta_stride_page >= (int64_t)L.H_KV * kPage * 4,
+                KITTY_E_RANGE, "a page stride is smaller than one page");
+  return 0;
+}
+}  // namespace
+
+extern "C" int kitty_append_token(const kitty_kv_layer* layer, const void* k_new, const void* v_new,
+                                  int64_t stride_b, int64_t stride_h, int B, void* stream) {
+  if (int rc = check_append_layer(layer, B)) return rc;
+  KITTY_REQUIRE(k_new && v_new, KITTY_E_NULL, "k_new / v_new is NULL");
+  KITTY_REQUIRE(((uintptr_t)k_new % 8) == 0 && ((uintptr_t)v_new % 8) == 0 && stride_b % 8 == 0 && stride_h % 8 == 0,
+                KITTY_E_ALIGN, "k_new / v_new need 8-byte aligned bases and strides");
+  hipLaunchKernelGGL(append_token_kernel, dim3(B), dim3(256), 0, (hipStream_t)stream, *layer, (const uint8_t*)k_new,
+                     (const uint8_t*)v_new, stride_b, stride_h);
+  return check_launch("kitty_append_token");
+}
+
+extern "C" int kitty_flush_full(const kitty_kv_layer* layer, int B, int64_t cache_pages, void* stream) {
+  if (int rc = check_append_layer(layer, B)) return rc;
+  KITTY_REQUIRE(cache_pages >= 0, KITTY_E_RANGE, "bad cache_pages");
+  hipLaunchKernelGGL(flush_full_kernel, dim3(layer->H_KV, B, 2), dim3(256), 0, (hipStream_t)stream, *layer, cache_pages);
+  hipLaunchKernelGGL(advance_counts_kernel, dim3((B + 63) / 64), dim3(64), 0, (hipStream_t)stream, *layer, B);
+  return check_launch("kitty_flush_full");
 }

@@ -14,6 +14,7 @@ try:  # the plugin subclasses HF's Cache when transformers is importable
 except Exception:  # pragma: no cover - transformers is optional for the kernels themselves
     _HFCache = object
 
+from .. import _lib
 from .kernels.kitty_quant_pack import quantize_pack_k, quantize_pack_v
 from .utils_kv_per_layer import KVCache_Layer
 
@@ -59,6 +60,9 @@ class KittyCache(_HFCache):
         assert key_states.shape[-2] == 1 and value_states.shape[-2] == 1, \
             "Decode: key_states and value_states should have sequence length of 1."
         B = key_states.shape[0]
+        if kvcache.device_counters:
+            self._append_token_device(kvcache, key_states, value_states)
+            return False
         with torch.no_grad():
             if kvcache.Sink_Count < kvcache.S:
                 idx = kvcache.Sink_Count
@@ -130,6 +134,9 @@ class KittyCache(_HFCache):
         """Flush a full Q-buffer into the next packed page; K and V fill up independently
         (kitty.py:194-236)."""
         kvcache = self.kv_cache[layer_idx]
+        if kvcache.device_counters:
+            self._flush_full_device(kvcache)
+            return
         if kvcache.Q_Buffer_Count_K == kvcache.PAGE_SIZE:
             if kvcache.PageCount_K >= kvcache.MAX_PAGE:
                 raise ValueError(f"key cache is full (max_length={kvcache.MAX_LEN})")
@@ -145,6 +152,53 @@ class KittyCache(_HFCache):
             kvcache.PageCount_V += 1
             kvcache.Q_Buffer_Count_V = 0
 
+    # ---- per-sequence counters on the device ---------------------------------------------------
+    def enable_device_counters(self, seq_counts: Optional[torch.Tensor] = None) -> None:
+        """Switch every layer to device-side per-sequence counters (after the prefill): decode
+        steps then cost one append launch and one flush launch per layer, never read the device,
+        and serve sequences of different lengths.  ``seq_counts [MAX_BS, 8]`` sets a ragged
+        starting state for all layers; default: every sequence at the layer's current state."""
+        if self.select != "hip":
+            raise ValueError("device counters use the fused channel selection (select='hip')")
+        for L in self.kv_cache:
+            L.enable_device_counters(seq_counts)
+
+    def _append_token_device(self, L: KVCache_Layer, key_states: torch.Tensor, value_states: torch.Tensor) -> None:
+        B = key_states.shape[0]
+        for name, t in (("key_states", key_states), ("value_states", value_states)):
+            _lib.require_hip(t, name)
+            if t.dtype != torch.float16:
+                raise ValueError(f"{name} must be float16, got {t.dtype}")
+        if key_states.shape != (B, L.H_KV, 1, L.D) or value_states.shape != key_states.shape or B > L.MAX_BS:
+            raise ValueError(f"key_states / value_states must be [B <= {L.MAX_BS}, {L.H_KV}, 1, {L.D}]")
+        if key_states.stride(-1) != 1:
+            key_states = key_states.contiguous()
+        if value_states.stride() != key_states.stride():
+            key_states, value_states = key_states.contiguous(), value_states.contiguous()
+        if L.Sink_Count >= L.S and L.Q_Buffer_Count_K >= L.PAGE_SIZE:
+            raise ValueError("Q-buffer is full: call quantize_decode() after every decode step")
+        rc = _lib.lib().kitty_append_token(L.descriptor(), key_states.data_ptr(), value_states.data_ptr(),
+                                           key_states.stride(0) * 2, key_states.stride(1) * 2, B,
+                                           _lib.current_stream_ptr(key_states.device))
+        _lib.check(rc, "KittyCache.update")
+        L.active_batch = B
+        L.step_host_counters()
+
+    def _flush_full_device(self, L: KVCache_Layer) -> None:
+        P = L.PAGE_SIZE
+        if (L.Q_Buffer_Count_K == P and L.PageCount_K >= L.MAX_PAGE) or \
+                (L.Q_Buffer_Count_V == P and L.PageCount_V >= L.MAX_PAGE):
+            raise ValueError(f"cache is full (max_length={L.MAX_LEN})")
+        rc = _lib.lib().kitty_flush_full(L.descriptor(), L.active_batch, L.KeyCache.size(0),
+                                         _lib.current_stream_ptr(L.device))
+        _lib.check(rc, "KittyCache.quantize_decode")
+        if L.Q_Buffer_Count_K == P:
+            L.PageCount_K += 1
+            L.Q_Buffer_Count_K = 0
+        if L.Q_Buffer_Count_V == P:
+            L.PageCount_V += 1
+            L.Q_Buffer_Count_V = 0
+
     def append(self, key_states: torch.Tensor, value_states: torch.Tensor, layer_idx: int = 0) -> None:
         """Append a chunk of T >= 1 tokens ``[B, H_KV, T, D]`` to a layer in one go.
 
@@ -157,6 +211,9 @@ class KittyCache(_HFCache):
         ``update`` + ``quantize_prefill``.
         """
         L = self.kv_cache[layer_idx]
+        if L.device_counters:
+            raise NotImplementedError("chunk append works on the shared host counters; with device "
+                                      "counters append token by token (update + quantize_decode)")
         if key_states.shape != value_states.shape or key_states.dim() != 4:
             raise ValueError("key_states and value_states must both be [B, H_KV, T, D]")
         if L.get_total_length() == 0:

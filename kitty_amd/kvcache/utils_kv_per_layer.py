@@ -9,7 +9,9 @@ against the reference keeps working.  Differences, all additive:
   (:56-59);
 * ``seq_counts`` - an optional int32 ``[MAX_BS, 8]`` device tensor with per-sequence occupancy for
   ragged batches (the reference keeps one set of host ints for the whole batch, :53-54,65,71-72,
-  79-80).  When it is ``None`` the shared counters are used, exactly like the reference.
+  79-80).  When it is ``None`` the shared counters are used, exactly like the reference;
+* ``enable_device_counters()`` - from then on decode steps advance ``seq_counts`` on the device
+  (one fused append kernel, one flush launch) and the host ints only shadow the longest sequence.
 """
 import math
 from typing import Optional
@@ -70,6 +72,8 @@ class KVCache_Layer:
         self.value_states: Optional[torch.Tensor] = None
         # extensions
         self.seq_counts: Optional[torch.Tensor] = None
+        self.device_counters = False
+        self.active_batch = MAX_BS
         self._workspace: Optional[torch.Tensor] = None
         self._desc: Optional[_lib.KittyKVLayer] = None
 
@@ -80,6 +84,52 @@ class KVCache_Layer:
                     + self.Local_Count_V)
         assert total_length == seqlen_V, f"seqlen_K: {total_length}, seqlen_V: {seqlen_V}"
         return total_length
+
+    COUNT_FIELDS = ("Sink_Count", "PageCount_K", "Q_Buffer_Count_K", "PageCount_V", "Q_Buffer_Count_V",
+                    "Local_Count_V", "Write_Offset_Local_V")
+
+    def enable_device_counters(self, seq_counts: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """Keep the occupancy counters on the device, one int32 row of 8 per sequence, and let
+        ``KittyCache.update`` / ``quantize_decode`` advance them there.
+
+        ``seq_counts`` (``[MAX_BS, 8]``, field order of ``counts()``) gives every sequence its own
+        state; without it every row starts from the host counters.  The host ints stay in use as
+        a shadow of the longest sequence: they advance by the same rules on every step, without
+        reading the device, and answer ``get_total_length()`` and the capacity checks.
+        """
+        if seq_counts is None:
+            seq_counts = torch.tensor([self.counts()] * self.MAX_BS, dtype=torch.int32)
+        if tuple(seq_counts.shape) != (self.MAX_BS, _lib.SEQ_COUNT_FIELDS):
+            raise ValueError(f"seq_counts must be [{self.MAX_BS}, {_lib.SEQ_COUNT_FIELDS}], got {tuple(seq_counts.shape)}")
+        host = seq_counts.detach().to("cpu", torch.int64)
+        P = self.PAGE_SIZE
+        if bool((host < 0).any()) or bool((host[:, [0]] > self.S).any()) or bool((host[:, [2, 4, 5]] > P).any()) \
+                or bool((host[:, 6] >= P).any()) or bool((host[:, [1, 3]] > self.MAX_PAGE).any()):
+            raise ValueError("seq_counts holds a counter outside its range")
+        len_k = host[:, 0] + host[:, 1] * P + host[:, 2]
+        len_v = host[:, 0] + host[:, 3] * P + host[:, 4] + host[:, 5]
+        if not bool((len_k == len_v).all()):
+            raise ValueError("seq_counts: a sequence holds different numbers of keys and values")
+        longest = host[int(torch.argmax(len_k))].tolist()
+        for f, v in zip(self.COUNT_FIELDS, longest):
+            setattr(self, f, int(v))
+        self.seq_counts = seq_counts.detach().to(self.device, torch.int32).contiguous().clone()
+        self.device_counters = True
+        return self.seq_counts
+
+    def step_host_counters(self) -> None:
+        """One decode token in the host counters (the reference's rules, kitty.py:104-123)."""
+        if self.Sink_Count < self.S:
+            self.Sink_Count += 1
+            return
+        assert self.Q_Buffer_Count_K < self.PAGE_SIZE
+        self.Q_Buffer_Count_K += 1
+        if self.Local_Count_V < self.PAGE_SIZE:
+            self.Local_Count_V += 1
+        else:
+            assert self.Q_Buffer_Count_V < self.PAGE_SIZE
+            self.Q_Buffer_Count_V += 1
+            self.Write_Offset_Local_V = (self.Write_Offset_Local_V + 1) % self.PAGE_SIZE
 
     # ---- C-ABI view -------------------------------------------------------------------------
     def counts(self):

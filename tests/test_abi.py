@@ -88,6 +88,17 @@ def test_host_side_rejection_without_gpu(lib):
     L.counts[2] = 0
     L.D = 64
     assert lib.kitty_decode_attn(*args(4, fake, 1 << 20, 4)) == E_SHAPE
+    L.D = 128
+    assert lib.kitty_append_token(ctypes.byref(L), fake, fake, 256, 256, 1, None) == E_NULL    # no seq_counts
+    assert b"seq_counts" in lib.kitty_last_error()
+    assert lib.kitty_flush_full(ctypes.byref(L), 1, 4, None) == E_NULL
+    L.seq_counts = 4096
+    assert lib.kitty_append_token(ctypes.byref(L), None, fake, 256, 256, 1, None) == E_NULL
+    assert lib.kitty_append_token(ctypes.byref(L), fake, fake, 250, 256, 1, None) == E_ALIGN
+    assert lib.kitty_append_token(ctypes.byref(L), fake, fake, 256, 256, 0, None) == E_RANGE
+    assert lib.kitty_flush_full(ctypes.byref(L), 1, -1, None) == E_RANGE
+    L.PAGE_SIZE = 256
+    assert lib.kitty_flush_full(ctypes.byref(L), 1, 4, None) == E_SHAPE
     assert lib.kitty_decode_attn_workspace_bytes(16, 32, 128, 16) == 16 * 32 * 16 * 2 * 4 + 16 * 32 * 16 * 128 * 4
     assert lib.kitty_decode_attn_workspace_bytes(16, 32, 64, 16) == 0
     assert 1 <= lib.kitty_decode_attn_default_splits(16, 8, 257) <= 257

@@ -290,3 +290,50 @@ def test_append_rejects_overflow_without_side_effects(cpu_cache_oracle_quant):
     assert cache.get_seq_length(0) == before
     with pytest.raises(ValueError):
         cache.append(kt[:, :, :3], vt[:, :, :4], 0)
+
+
+# ---------------------------------------------------------------------------------------------
+# device-counter mode: the host shadow of the longest sequence
+# ---------------------------------------------------------------------------------------------
+def test_host_shadow_counters_follow_the_oracle():
+    """KVCache_Layer.step_host_counters + the flush bookkeeping advance the host ints exactly as
+    the oracle's update / quantize_decode do, from every phase of the state machine."""
+    from kitty_amd.kvcache.utils_kv_per_layer import KVCache_Layer
+    for T0 in (3, 32, 100, 32 + 128 + 5, 32 + 3 * 128):
+        k, v = make_kv(1, 1, T0 + 1, seed=T0)
+        ol = O.OracleLayer(1, 4096, 1)
+        ol.update(k[:, :, :T0], v[:, :, :T0])
+        ol.quantize_prefill()
+        L = KVCache_Layer(1, 4096, 1, 128, 32, 2, 4, 128, 32, device="cpu")
+        for f in KVCache_Layer.COUNT_FIELDS:
+            setattr(L, f, getattr(ol, f))
+        tok = (k[:, :, T0:T0 + 1], v[:, :, T0:T0 + 1])
+        for _ in range(700):
+            ol.update(*tok)
+            L.step_host_counters()
+            assert L.counts()[:7] == [getattr(ol, f) for f in KVCache_Layer.COUNT_FIELDS]
+            ol.quantize_decode()
+            for cnt, pages in (("Q_Buffer_Count_K", "PageCount_K"), ("Q_Buffer_Count_V", "PageCount_V")):
+                if getattr(L, cnt) == 128:          # what KittyCache._flush_full_device does on the host
+                    setattr(L, pages, getattr(L, pages) + 1)
+                    setattr(L, cnt, 0)
+            assert L.counts()[:7] == [getattr(ol, f) for f in KVCache_Layer.COUNT_FIELDS]
+        assert L.get_total_length() == T0 + 700
+
+
+def test_enable_device_counters_validates_and_shadows_the_longest():
+    from kitty_amd.kvcache.utils_kv_per_layer import KVCache_Layer
+    L = KVCache_Layer(3, 1024, 1, 128, 32, 2, 4, 128, 32, device="cpu")
+    rows = [[32, 1, 7, 0, 7, 128, 7, 0], [20, 0, 0, 0, 0, 0, 0, 0], [32, 2, 100, 1, 100, 128, 3, 0]]
+    sc = L.enable_device_counters(torch.tensor(rows, dtype=torch.int32))
+    assert L.device_counters and sc.dtype == torch.int32 and sc.tolist() == rows
+    assert L.counts() == rows[2] and L.get_total_length() == 32 + 2 * 128 + 100
+    for bad in ([[33, 0, 0, 0, 0, 0, 0, 0]] * 3, [[32, 0, 129, 0, 1, 128, 0, 0]] * 3, [[32, 0, 5, 0, 0, 4, 0, 0]] * 3,
+                [[32, 9, 0, 9, 0, 0, 0, 0]] * 3, [[32, 0, 1, 0, 0, 1, 128, 0]] * 3, [[-1, 0, 0, 0, 0, 0, 0, 0]] * 3):
+        with pytest.raises(ValueError):
+            L.enable_device_counters(torch.tensor(bad, dtype=torch.int32))
+    with pytest.raises(ValueError):
+        L.enable_device_counters(torch.zeros(2, 8, dtype=torch.int32))
+    M = KVCache_Layer(2, 1024, 1, 128, 32, 2, 4, 128, 32, device="cpu")
+    M.Sink_Count, M.Q_Buffer_Count_K, M.Local_Count_V = 32, 9, 9
+    assert M.enable_device_counters().tolist() == [[32, 0, 9, 0, 0, 9, 0, 0]] * 2
