@@ -212,16 +212,23 @@ def bench_end_to_end(args):
                    n2=torch.ones(HID, device=dev, dtype=torch.float16)) for _ in range(LAYERS)]
     emb, head = rnd(VOCAB, HID), rnd(VOCAB, HID)
     nf = torch.ones(HID, device=dev, dtype=torch.float16)
-    steps = args.warmup + args.steps
-    cache = kitty_amd.KittyCache(cfg, B, T0 + steps + 256, device=dev)
-    K, V = synth_kv(B, H_KV, T0, D, 1004, dev)
-    for li in range(LAYERS):              # a context of T0 tokens in every layer (same synthetic K/V)
-        cache.update(K, V, li)
-        cache.quantize_prefill(li)
-    del K, V
+    mode = args.e2e_mode
+    CHECK = 6 if mode == "graph" else 0   # steps of an eager twin the graph's tokens are checked against
+    steps = args.warmup + args.steps + CHECK + 4
+
+    def make_cache():
+        cache = kitty_amd.KittyCache(cfg, B, T0 + steps + 256, device=dev)
+        K, V = synth_kv(B, H_KV, T0, D, 1004, dev)
+        for li in range(LAYERS):          # a context of T0 tokens in every layer (same synthetic K/V)
+            cache.update(K, V, li)
+            cache.quantize_prefill(li)
+        if mode != "host":
+            cache.enable_device_counters()
+        return cache
+
     inv_freq = 1.0 / (500000.0 ** (torch.arange(0, D, 2, device=dev, dtype=torch.float32) / D))
 
-    def rope(x, pos):                     # x [B, H, 1, D], rotate-half convention
+    def rope(x, pos):                     # x [B, H, 1, D], rotate-half convention; pos: float or 0-d tensor
         ang = pos * inv_freq
         cos, sin = torch.cat([ang.cos(), ang.cos()]).half(), torch.cat([ang.sin(), ang.sin()]).half()
         x1, x2 = x[..., : D // 2], x[..., D // 2:]
@@ -232,7 +239,7 @@ def bench_end_to_end(args):
         return (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + 1e-5)).half() * w
 
     @torch.no_grad()
-    def step(tok, pos):
+    def step(cache, tok, pos):
         x = emb[tok]                      # [B, HID]: 2-D activations keep the GEMM launches cheap
         for li, w in enumerate(layers):
             h = rms(x, w["n1"])
@@ -248,23 +255,75 @@ def bench_end_to_end(args):
             x = x + F.linear(F.silu(gu[..., :FF]) * gu[..., FF:], w["wd"])
         return F.linear(rms(x, nf), head).argmax(-1).view(B)
 
+    cache = make_cache()
     tok = torch.zeros(B, dtype=torch.long, device=dev)
+    graph_ok = None
+    if mode == "graph":
+        # Device counters make the launch sequence of a step independent of the sequence lengths, so one
+        # captured graph serves every step; position and token live in device buffers it updates itself.
+        pos_t = torch.full((), float(T0), device=dev, dtype=torch.float32)
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):     # eager steps first: workspaces exist, libraries are initialised
+            for _ in range(3):
+                tok.copy_(step(cache, tok, pos_t))
+                pos_t += 1
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        saved = cache.host_counters()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            tok.copy_(step(cache, tok, pos_t))
+            pos_t += 1
+        cache.restore_host_counters(saved)   # capture ran the host bookkeeping of a step that did not execute
+
+        def run_step(i):
+            graph.replay()
+            cache.step_host_counters()
+
+        # every replay against an eager twin started from the same state, with eager work in between
+        twin = make_cache()
+        ttok = torch.zeros(B, dtype=torch.long, device=dev)
+        for i in range(3):
+            ttok = step(twin, ttok, float(T0 + i))
+        graph_ok = True
+        for i in range(CHECK):
+            run_step(i)
+            ttok = step(twin, ttok, float(T0 + 3 + i))
+            torch.cuda.synchronize()
+            graph_ok = graph_ok and bool(torch.equal(tok, ttok))
+        graph_ok = graph_ok and twin.host_counters() == cache.host_counters() and all(
+            torch.equal(a.seq_counts, b.seq_counts) for a, b in zip(cache.kv_cache, twin.kv_cache))
+        del twin
+        done = 3 + CHECK
+    else:
+        done = 0
+
+        def run_step(i):
+            nonlocal tok
+            tok = step(cache, tok, float(T0 + done + i))
+
     for i in range(args.warmup):
-        tok = step(tok, T0 + i)
+        run_step(i)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for i in range(args.steps):
-        tok = step(tok, T0 + args.warmup + i)
+        run_step(args.warmup + i)
     torch.cuda.synchronize()
     dt = (time.perf_counter() - t0) / args.steps
+    notes = {"host": "dense layers are torch (hipBLASLt); one Python-driven launch sequence per layer, host counters "
+                     "(the reference's mode), not graph-captured",
+             "device": "as host mode, but per-sequence counters on the device (fused append + flush launches)",
+             "graph": "per-sequence counters on the device; the whole step captured once in a HIP graph and replayed"}
     print(json.dumps({
         "metric": "end_to_end_decode_tokens_per_s", "value": B / dt, "unit": "tokens/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": dt * 1e3, "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "f16 model, 2/4-bit packed KV",
         "data": "synthetic (random-init Llama-3.1-8B shapes, synthetic KV context in every layer)",
         "config": {"workload": f"32-layer Llama-3.1-8B-shaped decode, batch {B}, context {T0}, greedy (configs[4] side number)",
-                   "batch": B, "context": T0, "layers": LAYERS},
-        "note": "dense layers are torch (hipBLASLt); one Python-driven launch sequence per layer, not graph-captured",
+                   "batch": B, "context": T0, "layers": LAYERS, "mode": mode},
+        "graph_tokens_match_eager": graph_ok, "final_length": cache.get_seq_length(0),
+        "note": notes[mode],
     }))
 
 
@@ -276,6 +335,9 @@ def main():
     ap.add_argument("--workload", default="c1", choices=sorted(WORKLOADS) + ["c3", "e2e"])
     ap.add_argument("--e2e-batch", type=int, default=16)
     ap.add_argument("--e2e-context", type=int, default=32768)
+    ap.add_argument("--e2e-mode", default="host", choices=["host", "device", "graph"],
+                    help="host: the reference's shared host counters; device: per-sequence counters on the device; "
+                         "graph: device counters and the whole step replayed from one captured HIP graph")
     ap.add_argument("--copies", type=int, default=0, help="independent cache copies to rotate over (0 = auto)")
     ap.add_argument("--splits", type=int, default=0)
     ap.add_argument("--variant", type=int, default=0)

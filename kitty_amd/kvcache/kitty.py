@@ -163,6 +163,37 @@ class KittyCache(_HFCache):
         for L in self.kv_cache:
             L.enable_device_counters(seq_counts)
 
+    def step_host_counters(self) -> None:
+        """Advance every layer's host shadow by one decode step (append + flush) without launching
+        anything.  For callers that replay a captured HIP graph of the decode step: the replay
+        advances the device counters, this keeps ``get_seq_length`` and the capacity checks in
+        step.  Capturing runs the Python of one step without executing its kernels: save
+        ``host_counters()`` before a capture and ``restore_host_counters`` after it."""
+        for L in self.kv_cache:
+            if not L.device_counters:
+                raise ValueError("step_host_counters is for layers with device counters")
+            P = L.PAGE_SIZE
+            if L.Sink_Count >= L.S and L.Q_Buffer_Count_K >= P:
+                raise ValueError("Q-buffer is full")
+            L.step_host_counters()
+            if (L.Q_Buffer_Count_K == P and L.PageCount_K >= L.MAX_PAGE) or \
+                    (L.Q_Buffer_Count_V == P and L.PageCount_V >= L.MAX_PAGE):
+                raise ValueError(f"cache is full (max_length={L.MAX_LEN})")
+            if L.Q_Buffer_Count_K == P:
+                L.PageCount_K += 1
+                L.Q_Buffer_Count_K = 0
+            if L.Q_Buffer_Count_V == P:
+                L.PageCount_V += 1
+                L.Q_Buffer_Count_V = 0
+
+    def host_counters(self) -> list:
+        return [L.counts() for L in self.kv_cache]
+
+    def restore_host_counters(self, saved: list) -> None:
+        for L, row in zip(self.kv_cache, saved):
+            for f, v in zip(L.COUNT_FIELDS, row):
+                setattr(L, f, int(v))
+
     def _append_token_device(self, L: KVCache_Layer, key_states: torch.Tensor, value_states: torch.Tensor) -> None:
         B = key_states.shape[0]
         for name, t in (("key_states", key_states), ("value_states", value_states)):
