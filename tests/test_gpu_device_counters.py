@@ -191,3 +191,63 @@ def test_device_counter_calls_reject_bad_arguments(K):
     assert lib.kitty_append_token(L.descriptor(), k.data_ptr() + 2, k.data_ptr(), 256, 256, 2, st) == -4
     with pytest.raises(NotImplementedError):
         c.append(k, k, 0)
+
+
+def test_decode_step_replays_from_one_captured_graph(K):
+    """update -> attend -> quantize_decode captured once and replayed 150 times (across a K flush,
+    a V flush and the ring wrap), with eager work and a synchronisation between replays; every
+    replay's output and the final state equal those of an eager twin."""
+    B, H_KV, H_Q, T, steps = 3, 2, 8, 32 + 128 + 120, 150
+    k, v = make_kv(B, H_KV, T + steps + 2, seed=41)
+    mod = K.u.module(H_KV, H_Q)
+
+    def make():
+        c = K.KittyCache(K.u.cfg(H_KV, H_Q), B, 1024)
+        c.update(K.u.to_dev(k[:, :, :T]), K.u.to_dev(v[:, :, :T]), 0)
+        c.quantize_prefill(0)
+        c.enable_device_counters()
+        return c
+
+    def step(c, kk, vv, qq):
+        c.update(kk, vv, 0)
+        out, _ = K.attn(mod, qq, c.kv_cache[0], 128 ** -0.5, num_splits=3)
+        c.quantize_decode(0)
+        return out
+
+    cg, ce = make(), make()
+    kin = torch.zeros(B, H_KV, 1, 128, dtype=torch.float16, device="cuda")
+    vin, qin = torch.zeros_like(kin), torch.zeros(B, H_Q, 1, 128, dtype=torch.float16, device="cuda")
+
+    def feed(s):
+        kin.copy_(K.u.to_dev(k[:, :, T + s:T + s + 1]))
+        vin.copy_(K.u.to_dev(v[:, :, T + s:T + s + 1]))
+        qin.copy_(K.u.to_dev(make_q(B, H_Q, seed=1000 + s)))
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    for s in range(2):                      # eager steps first: the workspace exists before the capture
+        feed(s)
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            step(cg, kin, vin, qin)
+        torch.cuda.current_stream().wait_stream(side)
+        step(ce, kin, vin, qin)
+    torch.cuda.synchronize()
+    saved = cg.host_counters()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out_g = step(cg, kin, vin, qin)
+    cg.restore_host_counters(saved)
+    for s in range(2, 2 + steps):
+        feed(s)
+        graph.replay()
+        cg.step_host_counters()
+        out_e = step(ce, kin, vin, qin)
+        torch.cuda.synchronize()
+        assert torch.equal(out_g, out_e), f"replay {s - 2}"
+    a, d = ce.kv_cache[0], cg.kv_cache[0]
+    for name in ("KeyCache", "KeyCache_metadata", "ValueCache", "ValueCache_metadata", "Sink_Buffer_K",
+                 "Sink_Buffer_V", "Q_Buffer_K", "Q_Buffer_V", "Local_Buffer_V", "seq_counts"):
+        assert torch.equal(getattr(a, name).view(torch.uint8), getattr(d, name).view(torch.uint8)), name
+    assert a.counts() == d.counts() and d.get_total_length() == T + 2 + steps
+    assert d.PageCount_K == 3 and d.PageCount_V == 2      # both flushes happened inside replays
