@@ -330,8 +330,9 @@ def bench_end_to_end(args):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=20)
+    # the defaults are long enough for the clocks to settle: the first ~100 launches after idle run 5-8 % slower
+    ap.add_argument("--steps", type=int, default=2000)
+    ap.add_argument("--warmup", type=int, default=500)
     ap.add_argument("--workload", default="c1", choices=sorted(WORKLOADS) + ["c3", "e2e"])
     ap.add_argument("--e2e-batch", type=int, default=16)
     ap.add_argument("--e2e-context", type=int, default=32768)

@@ -10,9 +10,10 @@
 //   S^T[token][col] = sum_ch  code[token][ch]            * (q[col][ch] * scale_k[ch])     (QK)
 //   O^T[ch][col]    = sum_tok code[tok][ch]               * (p[tok][col] * scale_v[tok])   (PV)
 //
-// The 16 columns hold the G query heads of the kv head (col n -> head n % G, replicated).  The
-// zero points never touch the codes: sum_ch q*zero_k is one dot product per page and column,
-// sum_tok p*zero_v one scalar per column, both on the vector ALU.
+// The 16 columns hold the G query heads of the kv head, replicated (col n -> head n % G; with at
+// most 8 heads col n -> head (n % 8) % G, and columns 8..15 carry the low-order part of the QK
+// operand, see qk_packed).  The zero points never touch the codes: sum_ch q*zero_k and
+// sum_tok p*zero_v are one more small matrix product each.
 //
 // Codes as operands.  A 32-bit word of a packed plane holds 16 two-bit codes of ONE row (K: one
 // channel, 16 tokens; V: one token, 16 channels) but an MFMA register must hold two consecutive k
@@ -160,7 +161,8 @@ struct Ctx {
   int b, h, lane, kg, n;
   uint32_t lane_off;    // register-fed tiles: byte offset of this lane's word relative to plane row krow(pi, 0)
   uint32_t sel;         // v_perm selector merging own / partner halves
-  int g;                // query head of this column (n % G)
+  int g;                // query head of this column
+  bool lo_part;         // split columns: this column carries the low part of q * scale (see qk_packed)
   uint32_t ktr;         // LDS: this lane's corner of a transposing read of K plane rows 4kg .. 4kg+3
   uint32_t vtr;         // LDS: same for V rows 32kg .. 32kg+3
   float sc2;            // scaling * log2(e)
@@ -282,9 +284,20 @@ __device__ __forceinline__ void stage_k_meta(LDS& S, const Ctx& x, const KSRC& k
   wave_lds_fence();
 }
 
+__device__ __forceinline__ float ror8(float v) {   // value of column n ^ 8 (rotation by 8 within the row of 16 lanes)
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x128 /* row_ror:8 */,
+                                                                0xf, 0xf, false));
+}
+
 // logits of one packed K page: C[u][j] = sum_ch code * q * scale, still in subnormal units
-// (multiply by code_unscale(u)); cz = q . zero
-template <bool BOOST, class LDS, class KSRC>
+// (multiply by code_unscale(u)); cz = q . zero.
+// q * scale does not fit an fp16 operand (the product of two fp16 numbers has 22 significant bits
+// and the logits need more than 11), so it enters as a rounded part and its exact remainder.
+// SPLIT_COLS (at most 8 query heads per kv head): the two parts sit in different columns of the
+// same B operand - column n carries the rounded part of head n % 8, column n + 8 the remainder -
+// and the two partial sums are added across the columns afterwards: one matrix instruction per
+// tile of codes instead of two, none of them waiting for the one before it.
+template <bool BOOST, bool SPLIT_COLS, class LDS, class KSRC>
 __device__ __forceinline__ void qk_packed(LDS& S, const Ctx& x, const KSRC& kb, float4v (&C)[8], float& cz) {
   stage_k_meta<BOOST>(S, x, kb);
   // q . zero_k on the matrix core as well: an A tile whose 16 rows all hold the zero points
@@ -302,14 +315,15 @@ __device__ __forceinline__ void qk_packed(LDS& S, const Ctx& x, const KSRC& kb, 
       const half2v qq = as_h2(x.qpair[kc * 4 + pi]), s2 = as_h2(sp[pi]);
       const half2v hi = qq * s2;                                   // q*scale rounded to fp16 ...
       const half2v lo = __builtin_elementwise_fma(qq, s2, -hi);    // ... and its exact remainder
-      bh[pi] = as_u32(hi);
+      bh[pi] = SPLIT_COLS ? (x.lo_part ? as_u32(lo) : as_u32(hi)) : as_u32(hi);
       bl[pi] = as_u32(lo);
       bq[pi] = x.qpair[kc * 4 + pi];
       az[pi] = zp[pi];
       Y[pi] = X[pi] >> 10;
     }
     Cz = mfma16(az, bq, Cz);
-    unpack_mfma2(X, Y, bh, bl, C);
+    if (SPLIT_COLS) unpack_mfma1(X, Y, bh, C);
+    else unpack_mfma2(X, Y, bh, bl, C);
   }
   if (BOOST) {
     // fifth chunk: the 32 high-plane slots; slot krow(pi, kg) + h carries bits 3:2 of the channel
@@ -324,11 +338,18 @@ __device__ __forceinline__ void qk_packed(LDS& S, const Ctx& x, const KSRC& kb, 
       const half2v s2 = {S.ks4_nat[c0], S.ks4_nat[c1]};
       const half2v hi = qq * s2;
       const half2v lo = __builtin_elementwise_fma(qq, s2, -hi);
-      bh[pi] = as_u32(hi);
+      bh[pi] = SPLIT_COLS ? (x.lo_part ? as_u32(lo) : as_u32(hi)) : as_u32(hi);
       bl[pi] = as_u32(lo);
       Y[pi] = X[pi] >> 10;
     }
-    unpack_mfma2(X, Y, bh, bl, C);
+    if (SPLIT_COLS) unpack_mfma1(X, Y, bh, C);
+    else unpack_mfma2(X, Y, bh, bl, C);
+  }
+  if (SPLIT_COLS) {
+#pragma unroll
+    for (int u = 0; u < 8; ++u)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) C[u][j] += ror8(C[u][j]);
   }
   cz = Cz[0];
 }
@@ -470,8 +491,8 @@ __device__ __forceinline__ void pv_packed(LDS& S, const Ctx& x, float4v (&out)[8
     for (int pi = 0; pi < 4; ++pi) {
       const half2v p2 = {(_Float16)P[2 * pi][j], (_Float16)P[2 * pi + 1][j]};   // tokens 32kg + 8j + 2pi + {0,1}
       p16[pi] = as_u32(p2);
-      alz[pi] = zr[pi];
       bp[pi] = as_u32(p2 * as_h2(sp[pi]));
+      alz[pi] = zr[pi];
       Y[pi] = X[pi] >> 10;
     }
     lz = mfma16(alz, p16, lz);
@@ -579,7 +600,9 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(kitty_kv_layer L, co
   x.sel = (x.n & 1) ? 0x03020706u : 0x05040100u;
   x.sc2 = scaling * kLog2e;
   const int G = H_Q / L.H_KV;
-  x.g = x.n % G;
+  constexpr bool SPLIT_COLS = DMA;   // both mean "at most 8 query heads per kv head"
+  x.g = SPLIT_COLS ? (x.n & 7) % G : x.n % G;
+  x.lo_part = SPLIT_COLS && (x.n & 8);
   x.ktr = (4 * x.kg + (x.n >> 2)) * kRowBytes + (x.n & 3) * 8;
   x.vtr = (32 * x.kg + (x.n >> 2)) * kRowBytes + (x.n & 3) * 8;
 
@@ -654,7 +677,7 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(kitty_kv_layer L, co
         const int buf = (i - t0) & 1;
         if (i == t0) wait_vmcnt<nK + kDmaV>(); else wait_vmcnt<nK + 2 * kDmaV>();
         __builtin_amdgcn_s_setprio(KITTY_PRIO_MFMA);
-        qk_packed<BOOST>(S, x, KLds{S.kbuf[buf]}, C, cz);
+        qk_packed<BOOST, SPLIT_COLS>(S, x, KLds{S.kbuf[buf]}, C, cz);
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
         dma_k<BOOST>(x, min(i + 2, t1 - 1), buf ? lk1 : lk0);
         __builtin_amdgcn_s_setprio(KITTY_PRIO_VALU);
@@ -677,7 +700,7 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(kitty_kv_layer L, co
     for (int i = t0; i < t1; ++i) {
       float cz;
       v_load_regs(x, i, vb);
-      qk_packed<BOOST>(S, x, kb, C, cz);
+      qk_packed<BOOST, SPLIT_COLS>(S, x, kb, C, cz);
       // unconditional (the last iteration re-loads its own tile) so that the number of loads in
       // flight is static and the PV phase only waits for the V words, not for this prefetch
       k_load_regs<BOOST>(x, min(i + 1, t1 - 1), kb);
@@ -695,7 +718,7 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(kitty_kv_layer L, co
       const int ntok = min(kPage, x.c.nbody - i * kPage);
       if (i < x.c.pk) {
         k_load_regs<BOOST>(x, i, kb);
-        qk_packed<BOOST>(S, x, kb, C, cz);
+        qk_packed<BOOST, SPLIT_COLS>(S, x, kb, C, cz);
         softmax_tile<true>(x, A, C, cz, ntok);
       } else {
         qk_fp16(x, qbuf_k, kPage, C);
