@@ -89,7 +89,19 @@ __device__ __forceinline__ uint32_t as_u32(half2v h) { return __builtin_bit_cast
 __device__ __forceinline__ uint32_t swap_pair(uint32_t v) {   // value of lane n^1
   return (uint32_t)__builtin_amdgcn_mov_dpp((int)v, 0xB1 /* quad_perm [1,0,3,2] */, 0xf, 0xf, true);
 }
-__device__ __forceinline__ float xor_lanes(float v, int mask) { return __shfl_xor(v, mask); }
+// Maximum over the four lane groups (lanes l, l^16, l^32, l^48) with the row-swap instructions of
+// gfx950: two vector instructions per step, where a shuffle would be a round trip through LDS.
+// v_permlane16_swap exchanges rows 1 and 3 of its first operand with rows 0 and 2 of its second.
+__device__ __forceinline__ float max_over_lane_groups(float v) {
+  const unsigned b = __builtin_bit_cast(unsigned, v);
+  const auto r = __builtin_amdgcn_permlane16_swap(b, b, false, false);
+  const unsigned r0 = r[0], r1 = r[1];   // as scalars first: a bit_cast of r[1] itself reads element 0
+  const float m = fmaxf(__builtin_bit_cast(float, r0), __builtin_bit_cast(float, r1));
+  const unsigned c = __builtin_bit_cast(unsigned, m);
+  const auto q = __builtin_amdgcn_permlane32_swap(c, c, false, false);
+  const unsigned q0 = q[0], q1 = q[1];
+  return fmaxf(__builtin_bit_cast(float, q0), __builtin_bit_cast(float, q1));
+}
 
 // The workgroup is one wavefront, and the LDS unit executes a wavefront's instructions in order:
 // a write followed by a read needs no hardware wait, only the compiler must keep the order.
@@ -265,6 +277,7 @@ template <bool BOOST, class LDS, class KSRC>
 __device__ __forceinline__ void stage_k_meta(LDS& S, const Ctx& x, const KSRC& kb) {
   const int l = x.lane;
   const uint2 km = kb.meta2(x);
+  const uint32_t ib = BOOST ? kb.idx(x) : 0u;   // both reads first: one round trip through LDS, not two
   const uint32_t ss = __builtin_amdgcn_perm(km.y, km.x, 0x05040100u);   // (s0, s1)
   const uint32_t zz = __builtin_amdgcn_perm(km.y, km.x, 0x07060302u);   // (z0, z1)
   const int pos = (l >> 4) * 16 + ((l >> 1) & 3) * 4 + 2 * ((l >> 3) & 1) + (l & 1);
@@ -275,8 +288,7 @@ __device__ __forceinline__ void stage_k_meta(LDS& S, const Ctx& x, const KSRC& k
     const half2v four = {(_Float16)4.0f, (_Float16)4.0f};
     ((uint32_t*)S.ks4_nat)[l] = as_u32(as_h2(ss) * four);
     if (l < 8) ((uint32_t*)S.inv)[l] = 0x80808080u;
-    wave_lds_fence();
-    const uint32_t ib = kb.idx(x);
+    wave_lds_fence();   // LDS executes a wave's instructions in order: the scatter below lands on the cleared bytes
     const uint32_t i0 = ib & 0xffu, i1 = ib >> 8;
     if (i0 < 32) S.inv[i0] = (uint8_t)(2 * l);
     if (i1 < 32) S.inv[i1] = (uint8_t)(2 * l + 1);
@@ -299,17 +311,45 @@ __device__ __forceinline__ float ror8(float v) {   // value of column n ^ 8 (rot
 // tile of codes instead of two, none of them waiting for the one before it.
 template <bool BOOST, bool SPLIT_COLS, class LDS, class KSRC>
 __device__ __forceinline__ void qk_packed(LDS& S, const Ctx& x, const KSRC& kb, float4v (&C)[8], float& cz) {
+  // One chunk of 32 plane rows ahead: the LDS reads of chunk kc + 1 are issued before the vector
+  // and matrix work of chunk kc, so that their latency is covered by this wave's own work.
+  uint32_t Xn[4];
+  kb.x4_lo(x, 0, Xn);                       // does not depend on the tables staged below
   stage_k_meta<BOOST>(S, x, kb);
+  uint4v spn = *(const uint4v*)&S.ks_perm[x.kg * 4];
+  uint4v zpn = *(const uint4v*)&S.kz_perm[x.kg * 4];
+  uint32_t inv2[4];                          // high-plane chunk: channels behind this lane's slots
+  half2v qh[4], sh[4];                       // high-plane chunk: gathered q and 4 * scale
   // q . zero_k on the matrix core as well: an A tile whose 16 rows all hold the zero points
   float4v Cz = float4v{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
   for (int u = 0; u < 8; ++u) C[u] = float4v{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
   for (int kc = 0; kc < 4; ++kc) {
-    const uint4v sp = *(const uint4v*)&S.ks_perm[kc * 16 + x.kg * 4];
-    const uint4v zp = *(const uint4v*)&S.kz_perm[kc * 16 + x.kg * 4];
     uint32_t bh[4], bl[4], bq[4], az[4], X[4], Y[4];
-    kb.x4_lo(x, kc, X);
+    const uint4v sp = spn, zp = zpn;
+#pragma unroll
+    for (int pi = 0; pi < 4; ++pi) X[pi] = Xn[pi];
+    if (kc < 3) {
+      kb.x4_lo(x, kc + 1, Xn);
+      spn = *(const uint4v*)&S.ks_perm[(kc + 1) * 16 + x.kg * 4];
+      zpn = *(const uint4v*)&S.kz_perm[(kc + 1) * 16 + x.kg * 4];
+    } else if (BOOST) {
+      kb.x4_hi(x, Xn);
+    }
+    if (BOOST && kc == 2) {
+#pragma unroll
+      for (int pi = 0; pi < 4; ++pi) inv2[pi] = *(const uint16_t*)&S.inv[krow(pi, x.kg)];
+    }
+    if (BOOST && kc == 3) {
+#pragma unroll
+      for (int pi = 0; pi < 4; ++pi) {
+        const uint32_t c0 = inv2[pi] & 0xffu, c1 = inv2[pi] >> 8;
+        qh[pi] = half2v{S.q_nat[x.g][c0], S.q_nat[x.g][c1]};
+        sh[pi] = half2v{S.ks4_nat[c0], S.ks4_nat[c1]};
+      }
+    }
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int pi = 0; pi < 4; ++pi) {
       const half2v qq = as_h2(x.qpair[kc * 4 + pi]), s2 = as_h2(sp[pi]);
@@ -329,15 +369,11 @@ __device__ __forceinline__ void qk_packed(LDS& S, const Ctx& x, const KSRC& kb, 
     // fifth chunk: the 32 high-plane slots; slot krow(pi, kg) + h carries bits 3:2 of the channel
     // inv[slot], weight 4 * scale
     uint32_t bh[4], bl[4], X[4], Y[4];
-    kb.x4_hi(x, X);
 #pragma unroll
     for (int pi = 0; pi < 4; ++pi) {
-      const uint32_t cc = *(const uint16_t*)&S.inv[krow(pi, x.kg)];
-      const uint32_t c0 = cc & 0xffu, c1 = cc >> 8;
-      const half2v qq = {S.q_nat[x.g][c0], S.q_nat[x.g][c1]};
-      const half2v s2 = {S.ks4_nat[c0], S.ks4_nat[c1]};
-      const half2v hi = qq * s2;
-      const half2v lo = __builtin_elementwise_fma(qq, s2, -hi);
+      X[pi] = Xn[pi];
+      const half2v hi = qh[pi] * sh[pi];
+      const half2v lo = __builtin_elementwise_fma(qh[pi], sh[pi], -hi);
       bh[pi] = SPLIT_COLS ? (x.lo_part ? as_u32(lo) : as_u32(hi)) : as_u32(hi);
       bl[pi] = as_u32(lo);
       Y[pi] = X[pi] >> 10;
@@ -392,8 +428,7 @@ __device__ __forceinline__ void softmax_tile(const Ctx& x, Acc& A, float4v (&C)[
     }
 #pragma unroll
   for (int u = 0; u < 8; ++u) mt = fmaxf(fmaxf(mt, fmaxf(C[u][0], C[u][1])), fmaxf(C[u][2], C[u][3]));
-  mt = fmaxf(mt, xor_lanes(mt, 16));
-  mt = fmaxf(mt, xor_lanes(mt, 32));
+  mt = max_over_lane_groups(mt);
   if (__any(A.first || mt > 0.f)) {
     // the column's max moves: shift this tile's logits and rescale what is accumulated
     const float dm = A.first ? mt : fmaxf(mt, 0.f);
@@ -481,18 +516,29 @@ __device__ __forceinline__ void pv_packed(LDS& S, const Ctx& x, float4v (&out)[8
   // sum p and sum p*zero_v ride along as one more A tile: even rows are ones, odd rows the zero
   // points, so row 0 of the product is the column's sum of p and row 1 its sum of p * zero_v
   const uint32_t* lz_rows = (x.n & 1) ? S.vz_nat : S.ones;
+  // one chunk of 8 plane rows per lane group ahead, as in qk_packed
+  uint32_t Xn[4];
+  vb.x4(x, 0, Xn);
+  uint4v spn = *(const uint4v*)&S.vs_nat[16 * x.kg];
+  uint4v zrn = *(const uint4v*)&lz_rows[16 * x.kg];
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
-    const uint4v sp = *(const uint4v*)&S.vs_nat[16 * x.kg + 4 * j];
-    const uint4v zr = *(const uint4v*)&lz_rows[16 * x.kg + 4 * j];
+    const uint4v sp = spn, zr = zrn;
     uint32_t bp[4], p16[4], alz[4], X[4], Y[4];
-    vb.x4(x, j, X);
+#pragma unroll
+    for (int pi = 0; pi < 4; ++pi) X[pi] = Xn[pi];
+    if (j < 3) {
+      vb.x4(x, j + 1, Xn);
+      spn = *(const uint4v*)&S.vs_nat[16 * x.kg + 4 * (j + 1)];
+      zrn = *(const uint4v*)&lz_rows[16 * x.kg + 4 * (j + 1)];
+    }
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int pi = 0; pi < 4; ++pi) {
       const half2v p2 = {(_Float16)P[2 * pi][j], (_Float16)P[2 * pi + 1][j]};   // tokens 32kg + 8j + 2pi + {0,1}
       p16[pi] = as_u32(p2);
-      bp[pi] = as_u32(p2 * as_h2(sp[pi]));
       alz[pi] = zr[pi];
+      bp[pi] = as_u32(p2 * as_h2(sp[pi]));
       Y[pi] = X[pi] >> 10;
     }
     lz = mfma16(alz, p16, lz);

@@ -93,6 +93,20 @@ __device__ __forceinline__ half8 load_a(const uint8_t* p) {
   return __builtin_shufflevector(a0, a1, 0, 1, 2, 3, 4, 5, 6, 7);
 }
 
+// Maximum over the four lane groups (lanes l, l^16, l^32, l^48) with the row-swap instructions of
+// gfx950: two vector instructions per step, where a shuffle would be a round trip through LDS.
+// v_permlane16_swap exchanges rows 1 and 3 of its first operand with rows 0 and 2 of its second.
+__device__ __forceinline__ float max_over_lane_groups(float v) {
+  const unsigned b = __builtin_bit_cast(unsigned, v);
+  const auto r = __builtin_amdgcn_permlane16_swap(b, b, false, false);
+  const unsigned r0 = r[0], r1 = r[1];   // as scalars first: a bit_cast of r[1] itself reads element 0
+  const float m = fmaxf(__builtin_bit_cast(float, r0), __builtin_bit_cast(float, r1));
+  const unsigned c = __builtin_bit_cast(unsigned, m);
+  const auto q = __builtin_amdgcn_permlane32_swap(c, c, false, false);
+  const unsigned q0 = q[0], q1 = q[1];
+  return fmaxf(__builtin_bit_cast(float, q0), __builtin_bit_cast(float, q1));
+}
+
 __device__ __forceinline__ float xor_lanes(float v, int mask) { return __shfl_xor(v, mask); }
 
 // fp16(code) * scale + zero with both roundings, for two codes at a time; `c` holds the codes as
@@ -330,8 +344,7 @@ struct TileAttend {
     for (int nt = 0; nt < kNT; ++nt) {
       float mx = fmaxf(fmaxf(S[0][nt][0], S[0][nt][1]), fmaxf(S[0][nt][2], S[0][nt][3]));
       mx = fmaxf(mx, fmaxf(fmaxf(S[1][nt][0], S[1][nt][1]), fmaxf(S[1][nt][2], S[1][nt][3])));
-      mx = fmaxf(mx, xor_lanes(mx, 16));
-      mx = fmaxf(mx, xor_lanes(mx, 32));
+      mx = max_over_lane_groups(mx);
       mt_[nt] = mx;
     }
     bool move = A.first;
