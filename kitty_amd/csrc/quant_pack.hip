@@ -69,6 +69,29 @@ __device__ __forceinline__ float div_by(float n, Divisor k) {
 __device__ __forceinline__ float code_of(float x_minus_min, Divisor k, float qlim) {
   return __builtin_floorf(fminf(div_by(x_minus_min, k) + 0.5f, qlim));
 }
+// The same codes for 8 values of one group at a time, mostly without the division: t = x * (1 /
+// scale) + 0.5 in one fma is within 4e-6 of the reference's (x / scale) + 0.5 (quotients are below
+// 16.5, the reciprocal is good to 2^-23), so unless a t lies within 2^-16 of an integer its floor is
+// the reference's code.  If any lane of the wave has such a t among its 8, the wave redoes these
+// 8 values with the exact division (about one case in seventy).
+__device__ __forceinline__ void codes_of_8(const float (&x)[8], float mn, Divisor k, float qlim, float (&c)[8]) {
+  float t[8], fmn = 1.0f, fmx = 0.0f;
+#pragma unroll
+  for (int r = 0; r < 8; ++r) {
+    t[r] = __builtin_fmaf(x[r] - mn, k.r, 0.5f);
+    const float f = __builtin_amdgcn_fractf(t[r]);
+    fmn = fminf(fmn, f);
+    fmx = fmaxf(fmx, f);
+  }
+  constexpr float kEps = 1.52587890625e-05f;   // 2^-16
+  if (__any(!(fmn >= kEps && fmx <= 1.0f - kEps))) {
+#pragma unroll
+    for (int r = 0; r < 8; ++r) c[r] = code_of(x[r] - mn, k, qlim);
+  } else {
+#pragma unroll
+    for (int r = 0; r < 8; ++r) c[r] = __builtin_floorf(fminf(t[r], qlim));
+  }
+}
 // Bits {1,0} (SHIFT = 0) or {3,2} (SHIFT = 2) of the 8 nibbles of n, packed into 16 bits.
 template <int SHIFT>
 __device__ __forceinline__ uint32_t gather_fields(uint32_t n) {
@@ -95,7 +118,7 @@ __device__ __forceinline__ void quant_k_page(const uint8_t* __restrict__ src_pag
   __shared__ float s_pmax[16][kD];
   __shared__ double s_psum[MODE == 0 ? 1 : 16][kD];
   __shared__ float4 s_q[kD];   // per channel: min, scale, refined reciprocal of the scale, qmax + 0.5
-  __shared__ uint16_t s_score[kD];
+  __shared__ __attribute__((aligned(16))) uint32_t s_key[kD];   // score << 8 | (127 - channel): larger sorts first
   __shared__ __attribute__((aligned(16))) uint8_t s_idx[kD];
   __shared__ __attribute__((aligned(16))) uint16_t s_lo[kD * 16];
 
@@ -139,7 +162,8 @@ __device__ __forceinline__ void quant_k_page(const uint8_t* __restrict__ src_pag
 #pragma unroll
       for (int i = 0; i < 16; ++i) sum += s_psum[i][tid];
       // an integer below 2^47 (or inf / nan for non-finite inputs, which saturate)
-      s_score[tid] = mean_abs_fp16_bits(sum < 1.8e19 ? (uint64_t)(sum * 16777216.0) : ~0ull);
+      s_key[tid] = ((uint32_t)mean_abs_fp16_bits(sum < 1.8e19 ? (uint64_t)(sum * 16777216.0) : ~0ull) << 8) |
+                   (uint32_t)(kD - 1 - tid);
     } else {
       s_idx[tid] = slot_in[tid];
     }
@@ -149,11 +173,12 @@ __device__ __forceinline__ void quant_k_page(const uint8_t* __restrict__ src_pag
     if (tid < kD) {
       // rank = number of channels that sort before this one: higher score, or equal score and
       // lower channel index
-      const uint16_t mine = s_score[tid];
+      const uint32_t mine = s_key[tid];
       int rank = 0;
-      for (int d = 0; d < kD; ++d) {
-        const uint16_t o = s_score[d];
-        rank += (o > mine) || (o == mine && d < tid);
+#pragma unroll 8
+      for (int d = 0; d < kD; d += 4) {
+        const uint4 o = *(const uint4*)&s_key[d];
+        rank += (o.x > mine) + (o.y > mine) + (o.z > mine) + (o.w > mine);
       }
       const uint8_t slot = (uint8_t)(rank < d_boost ? rank : d_boost);
       s_idx[tid] = slot;
@@ -181,8 +206,7 @@ __device__ __forceinline__ void quant_k_page(const uint8_t* __restrict__ src_pag
     const Divisor k = {qp.y, qp.z};
     // the 8 codes (0..15) as one word of nibbles, built in floating point (exact: 16 bits per half)
     float c[8];
-#pragma unroll
-    for (int r = 0; r < 8; ++r) c[r] = code_of(xs[j][r] - qp.x, k, qp.w);
+    codes_of_8(xs[j], qp.x, k, qp.w, c);
     const float h0 = __builtin_fmaf(__builtin_fmaf(__builtin_fmaf(c[3], 16.f, c[2]), 16.f, c[1]), 16.f, c[0]);
     const float h1 = __builtin_fmaf(__builtin_fmaf(__builtin_fmaf(c[7], 16.f, c[6]), 16.f, c[5]), 16.f, c[4]);
     const uint32_t nib = (uint32_t)h0 | ((uint32_t)h1 << 16);
