@@ -151,51 +151,60 @@ __device__ __forceinline__ void quant_k_page(const uint8_t* __restrict__ src_pag
   }
   __syncthreads();
 
-  float ch_min = 0.f, ch_max = 0.f;
-  if (tid < kD) {
-    float mn = s_pmin[0][tid], mx = s_pmax[0][tid];
+  // Second stage on lane pairs: lanes 2c and 2c+1 each fold 8 of channel c's 16 partials, then
+  // exchange; with selection they also split the 128 comparisons of the ranking.
+  const int ch = tid >> 1, hf = tid & 1;
+  float ch_min = s_pmin[hf][ch], ch_max = s_pmax[hf][ch];
 #pragma unroll
-    for (int i = 1; i < 16; ++i) { mn = fminf(mn, s_pmin[i][tid]); mx = fmaxf(mx, s_pmax[i][tid]); }
-    ch_min = mn; ch_max = mx;
-    if (MODE != 0) {
-      double sum = 0.0;
-#pragma unroll
-      for (int i = 0; i < 16; ++i) sum += s_psum[i][tid];
-      // an integer below 2^47 (or inf / nan for non-finite inputs, which saturate)
-      s_key[tid] = ((uint32_t)mean_abs_fp16_bits(sum < 1.8e19 ? (uint64_t)(sum * 16777216.0) : ~0ull) << 8) |
-                   (uint32_t)(kD - 1 - tid);
-    } else {
-      s_idx[tid] = slot_in[tid];
-    }
+  for (int i = 2; i < 16; i += 2) {
+    ch_min = fminf(ch_min, s_pmin[i + hf][ch]);
+    ch_max = fmaxf(ch_max, s_pmax[i + hf][ch]);
   }
+  ch_min = fminf(ch_min, __shfl_xor(ch_min, 1));
+  ch_max = fmaxf(ch_max, __shfl_xor(ch_max, 1));
   if (MODE != 0) {
+    double sum = 0.0;
+#pragma unroll
+    for (int i = 0; i < 16; i += 2) sum += s_psum[i + hf][ch];
+    sum += __shfl_xor(sum, 1);
+    // an integer below 2^47 (or inf / nan for non-finite inputs, which saturate)
+    if (hf == 0)
+      s_key[ch] = ((uint32_t)mean_abs_fp16_bits(sum < 1.8e19 ? (uint64_t)(sum * 16777216.0) : ~0ull) << 8) |
+                  (uint32_t)(kD - 1 - ch);
     __syncthreads();
-    if (tid < kD) {
-      // rank = number of channels that sort before this one: higher score, or equal score and
-      // lower channel index
-      const uint32_t mine = s_key[tid];
-      int rank = 0;
+    // rank = number of channels that sort before this one: higher score, or equal score and
+    // lower channel index
+    const uint32_t mine = s_key[ch];
+    int rank = 0;
 #pragma unroll 8
-      for (int d = 0; d < kD; d += 4) {
-        const uint4 o = *(const uint4*)&s_key[d];
-        rank += (o.x > mine) + (o.y > mine) + (o.z > mine) + (o.w > mine);
-      }
-      const uint8_t slot = (uint8_t)(rank < d_boost ? rank : d_boost);
-      s_idx[tid] = slot;
-      if (slot_out) slot_out[tid] = slot;
+    for (int d = hf * (kD / 2); d < (hf + 1) * (kD / 2); d += 4) {
+      const uint4 o = *(const uint4*)&s_key[d];
+      rank += (o.x > mine) + (o.y > mine) + (o.z > mine) + (o.w > mine);
+    }
+    rank += __shfl_xor(rank, 1);
+    const uint8_t slot = (uint8_t)(rank < d_boost ? rank : d_boost);
+    if (hf == 0) {
+      s_idx[ch] = slot;
+      if (slot_out) slot_out[ch] = slot;
     }
     if (MODE == 2) return;
-  }
-
-  if (tid < kD) {
-    const bool boosted = s_idx[tid] < d_boost;
-    const float qmax = boosted ? 15.0f : 3.0f;
+    if (hf == 0) {
+      const float qmax = slot < d_boost ? 15.0f : 3.0f;
+      float scale = (ch_max - ch_min) / qmax;
+      scale = scale < 1e-6f ? 1e-6f : scale;
+      const Divisor k = make_divisor(scale);
+      s_q[ch] = float4{ch_min, k.d, k.r, qmax + 0.5f};
+      *(__half2*)(meta_dst + ch * 4) = __halves2half2(__float2half_rn(scale), __float2half_rn(ch_min));
+    }
+  } else if (hf == 0) {
+    const uint8_t slot = slot_in[ch];
+    s_idx[ch] = slot;
+    const float qmax = slot < d_boost ? 15.0f : 3.0f;
     float scale = (ch_max - ch_min) / qmax;
     scale = scale < 1e-6f ? 1e-6f : scale;
     const Divisor k = make_divisor(scale);
-    s_q[tid] = float4{ch_min, k.d, k.r, qmax + 0.5f};
-    __half2 m2 = __halves2half2(__float2half_rn(scale), __float2half_rn(ch_min));
-    *(__half2*)(meta_dst + tid * 4) = m2;
+    s_q[ch] = float4{ch_min, k.d, k.r, qmax + 0.5f};
+    *(__half2*)(meta_dst + ch * 4) = __halves2half2(__float2half_rn(scale), __float2half_rn(ch_min));
   }
   __syncthreads();
 
