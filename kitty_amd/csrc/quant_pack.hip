@@ -69,27 +69,36 @@ __device__ __forceinline__ float div_by(float n, Divisor k) {
 __device__ __forceinline__ float code_of(float x_minus_min, Divisor k, float qlim) {
   return __builtin_floorf(fminf(div_by(x_minus_min, k) + 0.5f, qlim));
 }
-// The same codes for 8 values of one group at a time, mostly without the division: t = x * (1 /
-// scale) + 0.5 in one fma is within 4e-6 of the reference's (x / scale) + 0.5 (quotients are below
-// 16.5, the reciprocal is good to 2^-23), so unless a t lies within 2^-16 of an integer its floor is
-// the reference's code.  If any lane of the wave has such a t among its 8, the wave redoes these
-// 8 values with the exact division (about one case in seventy).
-__device__ __forceinline__ void codes_of_8(const float (&x)[8], float mn, Divisor k, float qlim, float (&c)[8]) {
-  float t[8], fmn = 1.0f, fmx = 0.0f;
+// The same codes for N values of one group at a time, mostly without the division:
+//   t = fma(x, r, c0),  c0 = fma(-min, r, 0.5),  r = the refined reciprocal of the scale.
+// Against the reference's fl(fl((x - min) / scale) + 0.5) this differs by the roundings of x - min,
+// of the quotient and of the sum (1e-6 each for quotients below 16.5), the reciprocal's last bit
+// (2e-6), the rounding of c0 (1.9e-6 while |min * r| <= 32) and its own (1e-6): under 8e-6.  So
+// unless t lies within 2^-16 of an integer, floor(t) is the reference's code; the reference's upper
+// clamp never changes a floor for finite inputs (the largest quotient is qmax * (1 + 2^-24)).  If any
+// lane of the wave has such a t among its N, or a group whose c0 is NaN (fast_offset returns that
+// when |min * r| > 32 or the scale is not finite), the wave redoes these N values with the exact
+// division: about one group in seventy on gaussian data.
+__device__ __forceinline__ float fast_offset(float mn, Divisor k) {
+  const float c0 = __builtin_fmaf(-mn, k.r, 0.5f);
+  return (fabsf(mn * k.r) <= 32.0f && k.d < 3.0e38f) ? c0 : __builtin_nanf("");
+}
+template <int N>
+__device__ __forceinline__ void codes_of(const float (&x)[N], float mn, float c0, Divisor k, float qlim, float (&c)[N]) {
+  float fmn = 1.0f, fmx = 0.0f;
 #pragma unroll
-  for (int r = 0; r < 8; ++r) {
-    t[r] = __builtin_fmaf(x[r] - mn, k.r, 0.5f);
-    const float f = __builtin_amdgcn_fractf(t[r]);
+  for (int r = 0; r < N; ++r) {
+    const float t = __builtin_fmaf(x[r], k.r, c0);
+    c[r] = __builtin_floorf(t);
+    const float f = t - c[r];
     fmn = fminf(fmn, f);
     fmx = fmaxf(fmx, f);
   }
   constexpr float kEps = 1.52587890625e-05f;   // 2^-16
-  if (__any(!(fmn >= kEps && fmx <= 1.0f - kEps))) {
+  // (min / max skip NaNs, so the group's NaN offset is tested by itself)
+  if (__any(!(c0 == c0 && fmn >= kEps && fmx <= 1.0f - kEps))) {
 #pragma unroll
-    for (int r = 0; r < 8; ++r) c[r] = code_of(x[r] - mn, k, qlim);
-  } else {
-#pragma unroll
-    for (int r = 0; r < 8; ++r) c[r] = __builtin_floorf(fminf(t[r], qlim));
+    for (int r = 0; r < N; ++r) c[r] = code_of(x[r] - mn, k, qlim);
   }
 }
 // Bits {1,0} (SHIFT = 0) or {3,2} (SHIFT = 2) of the 8 nibbles of n, packed into 16 bits.
@@ -118,6 +127,7 @@ __device__ __forceinline__ void quant_k_page(const uint8_t* __restrict__ src_pag
   __shared__ float s_pmax[16][kD];
   __shared__ double s_psum[MODE == 0 ? 1 : 16][kD];
   __shared__ float4 s_q[kD];   // per channel: min, scale, refined reciprocal of the scale, qmax + 0.5
+  __shared__ float s_c0[kD];   // per channel: the fast path's offset (fast_offset)
   __shared__ __attribute__((aligned(16))) uint32_t s_key[kD];   // score << 8 | (127 - channel): larger sorts first
   __shared__ __attribute__((aligned(16))) uint8_t s_idx[kD];
   __shared__ __attribute__((aligned(16))) uint16_t s_lo[kD * 16];
@@ -194,6 +204,8 @@ __device__ __forceinline__ void quant_k_page(const uint8_t* __restrict__ src_pag
       scale = scale < 1e-6f ? 1e-6f : scale;
       const Divisor k = make_divisor(scale);
       s_q[ch] = float4{ch_min, k.d, k.r, qmax + 0.5f};
+    s_c0[ch] = fast_offset(ch_min, k);
+      s_c0[ch] = fast_offset(ch_min, k);
       *(__half2*)(meta_dst + ch * 4) = __halves2half2(__float2half_rn(scale), __float2half_rn(ch_min));
     }
   } else if (hf == 0) {
@@ -204,6 +216,7 @@ __device__ __forceinline__ void quant_k_page(const uint8_t* __restrict__ src_pag
     scale = scale < 1e-6f ? 1e-6f : scale;
     const Divisor k = make_divisor(scale);
     s_q[ch] = float4{ch_min, k.d, k.r, qmax + 0.5f};
+    s_c0[ch] = fast_offset(ch_min, k);
     *(__half2*)(meta_dst + ch * 4) = __halves2half2(__float2half_rn(scale), __float2half_rn(ch_min));
   }
   __syncthreads();
@@ -215,7 +228,7 @@ __device__ __forceinline__ void quant_k_page(const uint8_t* __restrict__ src_pag
     const Divisor k = {qp.y, qp.z};
     // the 8 codes (0..15) as one word of nibbles, built in floating point (exact: 16 bits per half)
     float c[8];
-    codes_of_8(xs[j], qp.x, k, qp.w, c);
+    codes_of<8>(xs[j], qp.x, s_c0[d], k, qp.w, c);
     const float h0 = __builtin_fmaf(__builtin_fmaf(__builtin_fmaf(c[3], 16.f, c[2]), 16.f, c[1]), 16.f, c[0]);
     const float h1 = __builtin_fmaf(__builtin_fmaf(__builtin_fmaf(c[7], 16.f, c[6]), 16.f, c[5]), 16.f, c[4]);
     const uint32_t nib = (uint32_t)h0 | ((uint32_t)h1 << 16);
@@ -281,12 +294,14 @@ __device__ __forceinline__ void quant_v_page(const uint8_t* __restrict__ src_pag
     float scale = (mx - mn) / 3.0f;
     scale = scale < 1e-6f ? 1e-6f : scale;
     const Divisor kd = make_divisor(scale);
+    float code[16];
+    codes_of<16>(x, mn, fast_offset(mn, kd), kd, 3.5f, code);
     // 16 codes (0..3), 2 bits each, built in floating point in two exact 16-bit halves
     float h0 = 0.f, h1 = 0.f;
 #pragma unroll
     for (int k = 7; k >= 0; --k) {
-      h0 = __builtin_fmaf(h0, 4.f, code_of(x[k] - mn, kd, 3.5f));
-      h1 = __builtin_fmaf(h1, 4.f, code_of(x[8 + k] - mn, kd, 3.5f));
+      h0 = __builtin_fmaf(h0, 4.f, code[k]);
+      h1 = __builtin_fmaf(h1, 4.f, code[8 + k]);
     }
     const uint32_t packed = (uint32_t)h0 | ((uint32_t)h1 << 16);
     *(uint32_t*)(dst + t * kRowBytes + cg * 4) = packed;

@@ -117,6 +117,57 @@ def test_quantize_pack_bit_exact_random(K, student_t):
     assert np.array_equal(_np16(kc2), okc2)      # unmapped high-plane rows keep their old bytes
 
 
+def _awkward_page(rng):
+    """[128 tokens, 128 channels] fp16 whose channel groups exercise the quantizer's exact-division
+    fallback: offsets far larger than the range, constant groups (scale floor), values that sit
+    exactly on bin boundaries, fp16 extremes, subnormals; the rest gaussian."""
+    P = rng.standard_normal((128, 128)).astype(np.float32)
+    P[:, 0:16] = 100.0 + 0.01 * rng.standard_normal((128, 16))           # |min / scale| >> 32
+    P[:, 16:24] = rng.choice([0.0, 1.0, -3.5, 6.1e-5], size=(1, 8))      # constant per channel
+    P[:, 24:32] = 0.0
+    P[:, 32:48] = rng.integers(0, 7, size=(128, 16)) * 0.5               # (x - min) / scale = k + 0.5
+    P[0, 32:48], P[1, 32:48] = 0.0, 3.0
+    P[:, 48:56] = rng.choice([65504.0, -65504.0, 1.0, 0.0], size=(128, 8))
+    P[:, 56:64] = rng.integers(0, 1024, size=(128, 8)) * 2.0 ** -24      # subnormals only
+    P[:, 64:72] = rng.integers(0, 31, size=(128, 8)) / 2.0               # 4-bit boundaries if boosted
+    P[0, 64:72], P[1, 64:72] = 0.0, 15.0
+    return P.astype(np.float16)
+
+
+def test_quantize_pack_bit_exact_awkward_groups(K):
+    """Channel groups (K) and token groups (V) built to hit the slow paths of the code computation."""
+    rng = np.random.default_rng(77)
+    B, H, P, t0 = 1, 2, 3, 32
+    T = t0 + P * 128
+    k = rng.standard_normal((B, H, T, 128)).astype(np.float16)
+    v = k.copy()
+    for h in range(H):
+        for p in range(P):
+            pg = _awkward_page(rng)
+            k[0, h, t0 + p * 128:t0 + (p + 1) * 128] = pg          # groups along channels
+            v[0, h, t0 + p * 128:t0 + (p + 1) * 128] = pg.T        # the same groups along tokens
+    pt = np.arange(B * 4, dtype=np.int64).reshape(B, 4)
+    lay = O.Layout(H_KV=H)
+    okc = np.zeros((B * 4, lay.bytes_per_page_K), np.uint8)
+    okm = np.zeros((B * 4, H, 128, 2), np.float16)
+    ovc = np.zeros((B * 4, lay.bytes_per_page_V), np.uint8)
+    ovm = np.zeros((B * 4, H, 128, 2), np.float16)
+    used = O.quantize_pack_k(k, t0, P, pt, 0, okc, okm, 128, 32)
+    O.quantize_pack_v(v, t0, P, pt, 0, ovc, ovm, 128)
+    kc, km = K.u.to_dev(np.zeros_like(okc)), K.u.to_dev(np.zeros_like(okm))
+    vc, vm = K.u.to_dev(np.zeros_like(ovc)), K.u.to_dev(np.zeros_like(ovm))
+    kd, vd, ptd = K.u.to_dev(k), K.u.to_dev(v), K.u.to_dev(pt)
+    K.qk(kd, t0, P, ptd, 0, kc, km, 128, 32)
+    K.qv(vd, t0, P, ptd, 0, vc, vm, 128)
+    sm = K.sel(kd, t0, P, 128, 32)
+    torch.cuda.synchronize()
+    assert np.array_equal(_np16(sm), used)
+    assert np.array_equal(_np16(km).view(np.uint16), okm.view(np.uint16))
+    assert np.array_equal(_np16(kc), okc)
+    assert np.array_equal(_np16(vm).view(np.uint16), ovm.view(np.uint16))
+    assert np.array_equal(_np16(vc), ovc)
+
+
 def test_quantize_strided_source_no_copy(K):
     """[B, T, H, D] projections transposed to [B, H, T, D] are read through their strides."""
     B, H, T = 1, 2, 128 * 2
