@@ -100,11 +100,11 @@ __device__ __forceinline__ float max_over_lane_groups(float v) {
   const unsigned b = __builtin_bit_cast(unsigned, v);
   const auto r = __builtin_amdgcn_permlane16_swap(b, b, false, false);
   const unsigned r0 = r[0], r1 = r[1];   // as scalars first: a bit_cast of r[1] itself reads element 0
-  const float m = fmaxf(__builtin_bit_cast(float, r0), __builtin_bit_cast(float, r1));
+  const float m = vmax(__builtin_bit_cast(float, r0), __builtin_bit_cast(float, r1));
   const unsigned c = __builtin_bit_cast(unsigned, m);
   const auto q = __builtin_amdgcn_permlane32_swap(c, c, false, false);
   const unsigned q0 = q[0], q1 = q[1];
-  return fmaxf(__builtin_bit_cast(float, q0), __builtin_bit_cast(float, q1));
+  return vmax(__builtin_bit_cast(float, q0), __builtin_bit_cast(float, q1));
 }
 
 __device__ __forceinline__ float xor_lanes(float v, int mask) { return __shfl_xor(v, mask); }
@@ -342,8 +342,8 @@ struct TileAttend {
     float mt_[kNT];
 #pragma unroll
     for (int nt = 0; nt < kNT; ++nt) {
-      float mx = fmaxf(fmaxf(S[0][nt][0], S[0][nt][1]), fmaxf(S[0][nt][2], S[0][nt][3]));
-      mx = fmaxf(mx, fmaxf(fmaxf(S[1][nt][0], S[1][nt][1]), fmaxf(S[1][nt][2], S[1][nt][3])));
+      float mx = vmax3(vmax3(S[0][nt][0], S[0][nt][1], S[0][nt][2]), S[0][nt][3], S[1][nt][0]);
+      mx = vmax3(vmax3(mx, S[1][nt][1], S[1][nt][2]), S[1][nt][3], mx);
       mx = max_over_lane_groups(mx);
       mt_[nt] = mx;
     }
