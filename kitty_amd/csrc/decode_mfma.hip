@@ -65,16 +65,28 @@ struct Tables {
 };
 // LDS of one wave.  With tiles streamed through LDS (DMA) the budget is 160 KB / 8 waves per CU,
 // which leaves room for the q rows of 8 heads; larger groups use the register-fed variant.
-template <bool DMA>
+// QUARTER (1, 2 or 4 query heads per kv head, see softmax_quarter): four more V scale tables, q rows
+// of 4 heads.
+template <bool DMA, bool QUARTER>
 struct WaveLds;
 template <>
-struct WaveLds<true> : Tables {
+struct WaveLds<true, false> : Tables {
   __attribute__((aligned(16))) uint8_t kbuf[2][kKTile];
   __attribute__((aligned(16))) uint8_t vbuf[kVTile];
   __attribute__((aligned(16))) _Float16 q_nat[8][kQPad];   // [head][channel]; [..][128] = 0 ("no channel")
 };
 template <>
-struct WaveLds<false> : Tables {
+struct WaveLds<true, true> : Tables {
+  __attribute__((aligned(16))) uint8_t kbuf[2][kKTile];
+  __attribute__((aligned(16))) uint8_t vbuf[kVTile];
+  __attribute__((aligned(16))) _Float16 q_nat[4][kQPad];
+  // vs_q[t][e]: the V scale pair of token pair e if e % 4 == t, else 0 (cleared once per kernel):
+  // a column that owns operand register t of every chunk multiplies by table t and so feeds
+  // zeros for the tokens of the other columns
+  __attribute__((aligned(16))) uint32_t vs_q[4][64];
+};
+template <>
+struct WaveLds<false, false> : Tables {
   __attribute__((aligned(16))) _Float16 q_nat[16][kQPad];
   __attribute__((aligned(16))) uint8_t kbuf[1][10240];     // staging of fp16 V rows (pv_fp16)
 };
@@ -175,6 +187,8 @@ struct Ctx {
   uint32_t sel;         // v_perm selector merging own / partner halves
   int g;                // query head of this column
   bool lo_part;         // split columns: this column carries the low part of q * scale (see qk_packed)
+  int pi_own;           // quarter columns: the operand register (token pairs 2 pi_own + {0,1} of every octet) of this column
+  float usc[2];         // quarter columns: code_unscale(2 pi_own + i) * sc2
   uint32_t ktr;         // LDS: this lane's corner of a transposing read of K plane rows 4kg .. 4kg+3
   uint32_t vtr;         // LDS: same for V rows 32kg .. 32kg+3
   float sc2;            // scaling * log2(e)
@@ -301,6 +315,11 @@ __device__ __forceinline__ float ror8(float v) {   // value of column n ^ 8 (rot
                                                                 0xf, 0xf, false));
 }
 
+__device__ __forceinline__ float ror4(float v) {   // value of column n - 4 (mod 16)
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x124 /* row_ror:4 */,
+                                                                0xf, 0xf, false));
+}
+
 // logits of one packed K page: C[u][j] = sum_ch code * q * scale, still in subnormal units
 // (multiply by code_unscale(u)); cz = q . zero.
 // q * scale does not fit an fp16 operand (the product of two fp16 numbers has 22 significant bits
@@ -309,7 +328,8 @@ __device__ __forceinline__ float ror8(float v) {   // value of column n ^ 8 (rot
 // same B operand - column n carries the rounded part of head n % 8, column n + 8 the remainder -
 // and the two partial sums are added across the columns afterwards: one matrix instruction per
 // tile of codes instead of two, none of them waiting for the one before it.
-template <bool BOOST, bool SPLIT_COLS, class LDS, class KSRC>
+// COMBINE = false leaves the two partial sums of split columns apart (combine_quarter adds them).
+template <bool BOOST, bool SPLIT_COLS, bool COMBINE = true, class LDS, class KSRC>
 __device__ __forceinline__ void qk_packed(LDS& S, const Ctx& x, const KSRC& kb, float4v (&C)[8], float& cz) {
   // One chunk of 32 plane rows ahead: the LDS reads of chunk kc + 1 are issued before the vector
   // and matrix work of chunk kc, so that their latency is covered by this wave's own work.
@@ -381,13 +401,39 @@ __device__ __forceinline__ void qk_packed(LDS& S, const Ctx& x, const KSRC& kb, 
     if (SPLIT_COLS) unpack_mfma1(X, Y, bh, C);
     else unpack_mfma2(X, Y, bh, bl, C);
   }
-  if (SPLIT_COLS) {
+  if (SPLIT_COLS && COMBINE) {
 #pragma unroll
     for (int u = 0; u < 8; ++u)
 #pragma unroll
       for (int j = 0; j < 4; ++j) C[u][j] += ror8(C[u][j]);
   }
   cz = Cz[0];
+}
+
+// Quarter columns.  With 1, 2 or 4 query heads per kv head the 16 columns of a tile hold every
+// head at least four times (columns n, n ^ 4, n ^ 8, n ^ 12; n and n ^ 8 carry the two parts of
+// q * scale), and the softmax of a page would be computed four times over.  Instead each of the four
+// columns keeps two of the eight 16-token tiles - tiles 2 pi_own + {0, 1}, i.e. operand register
+// pi_own of every PV chunk - does the softmax of those 32 tokens only, and feeds zeros for the other
+// tokens into PV; its accumulators then hold a partial sum over its tokens, and the four are added
+// once, when the split is written.  The running maximum is shared, so the partials are compatible.
+//
+// own[i][j] = the full logit (both parts) of tile 2 pi_own + i, still in code units.  Two selects
+// around the cross-column add: columns n and n ^ 8 must hold the same tiles when they are added.
+__device__ __forceinline__ void combine_quarter(const Ctx& x, const float4v (&C)[8], float4v (&own)[2]) {
+  const bool upper = x.pi_own & 2, odd = x.pi_own & 1;   // pi_own = 2 * bit 2 of n + bit 3 of n
+  float4v T[4];
+#pragma unroll
+  for (int k = 0; k < 4; ++k)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const float v = upper ? C[4 + k][j] : C[k][j];
+      T[k][j] = v + ror8(v);
+    }
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) own[i][j] = odd ? T[2 + i][j] : T[i][j];
 }
 
 // logits of up to 128 fp16 rows (sink or K Q-buffer): A = the rows themselves, B = q
@@ -449,6 +495,39 @@ __device__ __forceinline__ void softmax_tile(const Ctx& x, Acc& A, float4v (&C)[
   for (int u = 0; u < 8; ++u)
 #pragma unroll
     for (int j = 0; j < 4; ++j) C[u][j] = __builtin_amdgcn_exp2f(C[u][j]);
+}
+
+// The same for the two tiles a quarter column owns (full packed pages only: nothing to mask).
+__device__ __forceinline__ void softmax_quarter(const Ctx& x, Acc& A, float4v (&own)[2], float cz) {
+  const float cst = cz * x.sc2 - A.m;
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) own[i][j] = own[i][j] * x.usc[i] + cst;
+  float mt = fmaxf(fmaxf(fmaxf(own[0][0], own[0][1]), fmaxf(own[0][2], own[0][3])),
+                   fmaxf(fmaxf(own[1][0], own[1][1]), fmaxf(own[1][2], own[1][3])));
+  mt = fmaxf(mt, ror4(mt));            // the four columns of a head ...
+  mt = fmaxf(mt, ror8(mt));
+  mt = max_over_lane_groups(mt);       // ... and the four lane groups: the page's maximum for this head
+  if (__any(A.first || mt > 0.f)) {
+    const float dm = A.first ? mt : fmaxf(mt, 0.f);
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) own[i][j] -= dm;
+    if (!A.first) {
+      const float alpha = __builtin_amdgcn_exp2f(-dm);
+      A.lz *= alpha;
+#pragma unroll
+      for (int u = 0; u < 8; ++u) A.out[u] *= alpha;
+    }
+    A.m += dm;
+    A.first = false;
+  }
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) own[i][j] = __builtin_amdgcn_exp2f(own[i][j]);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -546,6 +625,56 @@ __device__ __forceinline__ void pv_packed(LDS& S, const Ctx& x, float4v (&out)[8
   }
 }
 
+// PV for quarter columns: P holds the probabilities of the column's own tokens only (register j:
+// tokens 32kg + 8j + 2 pi_own + {0,1}).  The B operand of chunk j is that pair times the masked
+// scale table of pi_own: zero in the other three registers.  Sum p and sum p * zero_v take ONE more
+// tile per page: its B registers are the four own pairs themselves, and A row 2t + 1 holds the zero
+// points in the token order of a column with pi_own = t (even rows: ones), so column n finds its
+// sum of p in every even row and its sum of p * zero_v in row 2 pi_own + 1.
+template <class LDS>
+__device__ __forceinline__ void pv_quarter(LDS& S, const Ctx& x, float4v (&out)[8], float4v& lz, const VLds& vb,
+                                           const float4v (&P)[2]) {
+  const uint2 vm = vb.meta2(x);   // token pair e = lane: lane group e / 16, chunk (e / 4) % 4, register e % 4
+  wave_lds_fence();
+  S.vs_q[x.lane & 3][x.lane] = __builtin_amdgcn_perm(vm.y, vm.x, 0x05040100u);
+  S.vz_nat[(x.lane & 48) + 4 * (x.lane & 3) + ((x.lane >> 2) & 3)] = __builtin_amdgcn_perm(vm.y, vm.x, 0x07060302u);
+  wave_lds_fence();
+  const uint32_t* sq = &S.vs_q[x.pi_own][16 * x.kg];
+  const uint32_t* lz_rows = (x.n & 1) ? &S.vz_nat[16 * x.kg + 4 * ((x.n >> 1) & 3)] : &S.ones[0];
+  uint32_t Xn[4];
+  vb.x4(x, 0, Xn);
+  uint4v spn = *(const uint4v*)&sq[0];
+  const uint4v zr = *(const uint4v*)lz_rows;
+  uint32_t p16[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const half2v p2 = {(_Float16)P[0][j], (_Float16)P[1][j]};
+    p16[j] = as_u32(p2);
+  }
+  {
+    const uint32_t alz[4] = {zr[0], zr[1], zr[2], zr[3]};
+    lz = mfma16(alz, p16, lz);
+  }
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const uint4v sp = spn;
+    uint32_t bp[4], X[4], Y[4];
+#pragma unroll
+    for (int pi = 0; pi < 4; ++pi) X[pi] = Xn[pi];
+    if (j < 3) {
+      vb.x4(x, j + 1, Xn);
+      spn = *(const uint4v*)&sq[4 * (j + 1)];
+    }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int pi = 0; pi < 4; ++pi) {
+      bp[pi] = as_u32(as_h2(p16[j]) * as_h2(sp[pi]));
+      Y[pi] = X[pi] >> 10;
+    }
+    unpack_mfma1(X, Y, bp, out);
+  }
+}
+
 // fp16 V rows (sink, V Q-buffer, local ring), accumulators in true units.  The matrix core wants
 // A[row = channel][k = token], i.e. the rows transposed: 32 tokens at a time (the tokens of one
 // lane group) are copied into LDS as [channel][token] with 16-bit stores, after which the eight
@@ -553,7 +682,8 @@ __device__ __forceinline__ void pv_packed(LDS& S, const Ctx& x, float4v (&out)[8
 constexpr int kVtPitch = 80;                 // bytes per channel row: 32 tokens + padding
 constexpr int kVtBytes = kD * kVtPitch;      // 10240
 static_assert(kVtBytes <= 2 * kKTile && kVtBytes <= 10240, "the staging area reuses the K tile buffers");
-template <bool SINK>
+// QUARTER: the tail's tiles keep whole columns; only the columns with pi_own = 0 accumulate them.
+template <bool SINK, bool QUARTER>
 __device__ __forceinline__ void pv_fp16(uint8_t* vt, const Ctx& x, Acc& A, int tail_first_row, int ntok,
                                         const float4v (&P)[8]) {
   const kitty_kv_layer& L = *x.L;
@@ -592,7 +722,7 @@ __device__ __forceinline__ void pv_fp16(uint8_t* vt, const Ctx& x, Acc& A, int t
     }
     if (32 * (qt + 1) < ntok) fetch(qt + 1, piece);
     wave_lds_fence();
-    const bool mine = x.kg == qt;
+    const bool mine = x.kg == qt && (!QUARTER || x.pi_own == 0);
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       uint32_t bp[4], alz[4];
@@ -628,11 +758,14 @@ __device__ __forceinline__ void wait_vmcnt() {
 }
 
 // DMA: packed tiles are streamed global -> LDS (G <= 8); otherwise they are loaded into registers.
-template <bool BOOST, bool DMA>
+// QUARTER (needs DMA; 1, 2 or 4 query heads per kv head): body pages go through combine_quarter /
+// softmax_quarter / pv_quarter.
+template <bool BOOST, bool DMA, bool QUARTER>
 __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(kitty_kv_layer L, const __half* __restrict__ q, int H_Q,
                                                             float scaling, float* __restrict__ ws_ml,
                                                             float* __restrict__ ws_acc, int num_splits) {
-  __shared__ WaveLds<DMA> S;
+  static_assert(DMA || !QUARTER, "quarter columns are a variant of the LDS-streamed kernel");
+  __shared__ WaveLds<DMA, QUARTER> S;
   Ctx x;
   x.L = &L;
   x.b = blockIdx.z;
@@ -649,6 +782,18 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(kitty_kv_layer L, co
   constexpr bool SPLIT_COLS = DMA;   // both mean "at most 8 query heads per kv head"
   x.g = SPLIT_COLS ? (x.n & 7) % G : x.n % G;
   x.lo_part = SPLIT_COLS && (x.n & 8);
+  x.pi_own = ((x.n >> 2) & 1) * 2 + (x.n >> 3);
+  {
+    const int u_own = 2 * x.pi_own;   // code_unscale wants a constant: pick from the eight
+    float us[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) us[u] = code_unscale(u) * x.sc2;
+    x.usc[0] = x.usc[1] = 0.f;
+#pragma unroll
+    for (int u = 0; u < 8; u += 2) {
+      if (u == u_own) { x.usc[0] = us[u]; x.usc[1] = us[u + 1]; }
+    }
+  }
   x.ktr = (4 * x.kg + (x.n >> 2)) * kRowBytes + (x.n & 3) * 8;
   x.vtr = (32 * x.kg + (x.n >> 2)) * kRowBytes + (x.n & 3) * 8;
 
@@ -667,6 +812,10 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(kitty_kv_layer L, co
   }
   if (x.lane == 0) S.ks4_nat[128] = (_Float16)0.0f;
   S.ones[x.lane] = 0x3C003C00u;
+  if constexpr (QUARTER) {
+#pragma unroll
+    for (int t = 0; t < 4; ++t) S.vs_q[t][x.lane] = 0u;
+  }
   wave_lds_fence();
 
   Acc A;
@@ -723,14 +872,23 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(kitty_kv_layer L, co
         const int buf = (i - t0) & 1;
         if (i == t0) wait_vmcnt<nK + kDmaV>(); else wait_vmcnt<nK + 2 * kDmaV>();
         __builtin_amdgcn_s_setprio(KITTY_PRIO_MFMA);
-        qk_packed<BOOST, SPLIT_COLS>(S, x, KLds{S.kbuf[buf]}, C, cz);
+        qk_packed<BOOST, SPLIT_COLS, !QUARTER>(S, x, KLds{S.kbuf[buf]}, C, cz);
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
         dma_k<BOOST>(x, min(i + 2, t1 - 1), buf ? lk1 : lk0);
         __builtin_amdgcn_s_setprio(KITTY_PRIO_VALU);
-        softmax_tile<true>(x, A, C, cz, kPage);
-        wait_vmcnt<nK>();
-        __builtin_amdgcn_s_setprio(KITTY_PRIO_MFMA);
-        pv_packed(S, x, A.out, A.lz, VLds{S.vbuf}, C);
+        if constexpr (QUARTER) {
+          float4v own[2];
+          combine_quarter(x, C, own);
+          softmax_quarter(x, A, own, cz);
+          wait_vmcnt<nK>();
+          __builtin_amdgcn_s_setprio(KITTY_PRIO_MFMA);
+          pv_quarter(S, x, A.out, A.lz, VLds{S.vbuf}, own);
+        } else {
+          softmax_tile<true>(x, A, C, cz, kPage);
+          wait_vmcnt<nK>();
+          __builtin_amdgcn_s_setprio(KITTY_PRIO_MFMA);
+          pv_packed(S, x, A.out, A.lz, VLds{S.vbuf}, C);
+        }
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
         dma_v(x, min(i + 1, t1 - 1), lv);
       }
@@ -777,24 +935,49 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(kitty_kv_layer L, co
 #pragma unroll
         for (int u = 0; u < 8; ++u) tmp[u] = float4v{0.f, 0.f, 0.f, 0.f};
         v_load_regs(x, i, vb);
+        if (QUARTER && x.pi_own != 0) {
+#pragma unroll
+          for (int u = 0; u < 8; ++u) C[u] = float4v{0.f, 0.f, 0.f, 0.f};
+        }
         pv_packed(S, x, tmp, A.lz, vb, C);
 #pragma unroll
         for (int u = 0; u < 8; ++u) A.out[u] += tmp[u] * code_unscale(u);
       } else {
-        pv_fp16<false>(&S.kbuf[0][0], x, A, (i - x.c.pv) * kPage, ntok, C);
+        pv_fp16<false, QUARTER>(&S.kbuf[0][0], x, A, (i - x.c.pv) * kPage, ntok, C);
       }
     }
     if (do_sink && x.c.sink > 0) {
       const uint8_t* sink_k = (const uint8_t*)L.sink_k + (int64_t)x.b * L.sink_stride_b + (int64_t)x.h * L.sink_stride_h;
       qk_fp16(x, sink_k, L.S, C);
       softmax_tile<false>(x, A, C, 0.f, x.c.sink);
-      pv_fp16<true>(&S.kbuf[0][0], x, A, 0, x.c.sink, C);
+      pv_fp16<true, QUARTER>(&S.kbuf[0][0], x, A, 0, x.c.sink, C);
     }
   }
   to_true_units(A);
 
   // ---- partial of this split: columns n < G are the G heads -----------------------------------
-  const float l = A.lz[0], z = A.lz[1];
+  float l = A.lz[0], z = A.lz[1];
+  if constexpr (QUARTER) {
+    // the four columns of a head hold partial sums over their own tokens (the tail's tiles went to
+    // pi_own = 0 alone); sum p * zero_v of a column sits in row 2 pi_own + 1, which this lane holds
+    // if its lane group is even (pi_own 0, 1) or odd (pi_own 2, 3) accordingly
+    l += ror4(l);
+    l += ror8(l);
+    z = (x.pi_own & 1) ? A.lz[3] : A.lz[1];
+    z = ((x.pi_own >> 1) == (x.kg & 1)) ? z : 0.f;
+    z += ror4(z);
+    z += ror8(z);
+    z += __shfl_xor(z, 16);
+#pragma unroll
+    for (int u = 0; u < 8; ++u)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        float v = A.out[u][j];
+        v += ror4(v);
+        v += ror8(v);
+        A.out[u][j] = v;
+      }
+  }
   if (x.n < G) {
     const int64_t row = ((int64_t)x.b * H_Q + (int64_t)x.h * G + x.n) * num_splits + split;
     if (x.kg == 0) {
@@ -817,14 +1000,17 @@ bool decode_mfma_supported(const kitty_kv_layer& L, int H_Q) {
 void launch_decode_mfma(const kitty_kv_layer& L, const void* q, int B, int H_Q, float scaling, float* ws_ml,
                         float* ws_acc, int num_splits, hipStream_t stream) {
   const dim3 grid(num_splits, L.H_KV, B), block(64);
-  const bool boost = L.D_BOOSTED == 32, dma = H_Q / L.H_KV <= 8;
-#define KITTY_LAUNCH(BOOST, DMA)                                                                            \
-  hipLaunchKernelGGL((decode_mfma_kernel<BOOST, DMA>), grid, block, 0, stream, L, (const __half*)q, H_Q, scaling, \
-                     ws_ml, ws_acc, num_splits)
-  if (boost && dma) KITTY_LAUNCH(true, true);
-  else if (boost) KITTY_LAUNCH(true, false);
-  else if (dma) KITTY_LAUNCH(false, true);
-  else KITTY_LAUNCH(false, false);
+  const int G = H_Q / L.H_KV;
+  const bool boost = L.D_BOOSTED == 32, dma = G <= 8, quarter = G == 1 || G == 2 || G == 4;
+#define KITTY_LAUNCH(BOOST, DMA, QUARTER)                                                                   \
+  hipLaunchKernelGGL((decode_mfma_kernel<BOOST, DMA, QUARTER>), grid, block, 0, stream, L, (const __half*)q, H_Q, \
+                     scaling, ws_ml, ws_acc, num_splits)
+  if (boost && quarter) KITTY_LAUNCH(true, true, true);
+  else if (boost && dma) KITTY_LAUNCH(true, true, false);
+  else if (boost) KITTY_LAUNCH(true, false, false);
+  else if (quarter) KITTY_LAUNCH(false, true, true);
+  else if (dma) KITTY_LAUNCH(false, true, false);
+  else KITTY_LAUNCH(false, false, false);
 #undef KITTY_LAUNCH
 }
 
