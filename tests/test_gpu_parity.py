@@ -325,6 +325,30 @@ def test_group_sizes(K, G):
         _attend_both(K, cache, ol, H_KV, H_Q, q, variant=variant)
 
 
+@pytest.mark.parametrize("G", [1, 4, 8, 16])
+def test_no_boosted_channels(K, G):
+    """D_BOOSTED = 0 (no high plane): the other half of the kernel instantiations.  The reference's
+    cache always boosts head_dim / 4 channels, so the layer is built by hand."""
+    from kitty_amd.kvcache.utils_kv_per_layer import KVCache_Layer
+    B, H_KV, T, max_len = 2, 2, 32 + 128 * 4 + 77, 1024
+    H_Q = H_KV * G
+    k, v = make_kv(B, H_KV, T, seed=70 + G)
+    cache = K.KittyCache(K.u.cfg(H_KV, H_Q), B, max_len)
+    cache.d_boosted = 0
+    cache.kv_cache[0] = KVCache_Layer(MAX_BS=B, MAX_LEN=max_len, H_KV=H_KV, D=128, D_BOOSTED=0, LOW_BIT=2, HIGH_BIT=4,
+                                      PAGE_SIZE=128, S=32, device="cuda")
+    assert cache.update(K.u.to_dev(k), K.u.to_dev(v), 0) is True
+    cache.quantize_prefill(0)
+    ol = O.OracleLayer(B, max_len, H_KV, D_BOOSTED=0)
+    assert ol.update(k, v) is True
+    ol.quantize_prefill()
+    assert K.u.layer_bytes_equal(cache.kv_cache[0], ol) == []
+    q = make_q(B, H_Q, seed=G)
+    for variant in (0, 1):
+        for splits in (0, 1, 5):
+            _attend_both(K, cache, ol, H_KV, H_Q, q, variant=variant, num_splits=splits)
+
+
 def test_decode_steps_cross_flushes(K):
     """Prefill, then 300 decode steps (update -> attend -> quantize_decode, the caller's order):
     sink fill, ring wrap, K and V flushes at different steps.  State bit-exact at every step,
