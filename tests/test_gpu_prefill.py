@@ -99,6 +99,31 @@ def test_chunk_group_sizes(K, G):
     _run(K, cache, ol, H_KV, H_KV * G, B, Tq, seed=G, what=f"G={G}")
 
 
+def test_chunk_without_boosted_channels(K):
+    """D_BOOSTED = 0: the other instantiation of the kernel (the reference's cache always boosts
+    head_dim / 4 channels, so the layer is built by hand); the append of the chunk too."""
+    from kitty_amd.kvcache.utils_kv_per_layer import KVCache_Layer
+    B, H_KV, H_Q, T0, Tq, max_len = 2, 2, 8, 32 + 128 * 3 + 40, 170, 1024
+    cache = K.KittyCache(K.u.cfg(H_KV, H_Q), B, max_len)
+    cache.d_boosted = 0
+    cache.kv_cache[0] = KVCache_Layer(MAX_BS=B, MAX_LEN=max_len, H_KV=H_KV, D=128, D_BOOSTED=0, LOW_BIT=2, HIGH_BIT=4,
+                                      PAGE_SIZE=128, S=32, device="cuda")
+    ol = O.OracleLayer(B, max_len, H_KV, D_BOOSTED=0)
+    k, v = make_kv(B, H_KV, T0, seed=91)
+    cache.update(K.u.to_dev(k), K.u.to_dev(v), 0)
+    cache.quantize_prefill(0)
+    ol.update(k, v)
+    ol.quantize_prefill()
+    assert K.u.layer_bytes_equal(cache.kv_cache[0], ol) == []
+    got, q, kc, vc = _run(K, cache, ol, H_KV, H_Q, B, Tq, seed=92, what="no boosted channels")
+    cache.append(K.u.to_dev(kc), K.u.to_dev(vc), 0)
+    for t in range(Tq):
+        ol.update(kc[:, :, t:t + 1], vc[:, :, t:t + 1])
+        ol.quantize_decode()
+    torch.cuda.synchronize()
+    assert K.u.layer_bytes_equal(cache.kv_cache[0], ol) == []
+
+
 def test_one_token_chunk_equals_decode(K):
     """T_q = 1 is a decode step: same result as appending the token and calling decode attention."""
     B, H_KV, H_Q, T0 = 2, 2, 8, 32 + 128 * 4 + 9
