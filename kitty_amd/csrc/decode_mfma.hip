@@ -14,6 +14,8 @@
 // most 8 heads col n -> head (n % 8) % G, and columns 8..15 carry the low-order part of the QK
 // operand, see qk_packed).  The zero points never touch the codes: sum_ch q*zero_k and
 // sum_tok p*zero_v are one more small matrix product each.
+// With 1, 2 or 4 heads per kv head every head sits in at least four columns; each of the four then
+// does the softmax and feeds PV for a quarter of a page's tokens only (see combine_quarter).
 //
 // Codes as operands.  A 32-bit word of a packed plane holds 16 two-bit codes of ONE row (K: one
 // channel, 16 tokens; V: one token, 16 channels) but an MFMA register must hold two consecutive k

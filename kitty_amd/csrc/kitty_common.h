@@ -19,28 +19,18 @@ constexpr int kVBytes = kPage * kRowBytes;               // 4096: a V page-head
 
 __host__ __device__ inline int k_head_bytes(int d_boost) { return kRowBytes * (kD + d_boost) + kD; }
 
-// v_max_f32 / v_min_f32 (and the three-operand forms) as single instructions.  In front of fmaxf /
-// fminf the compiler puts a NaN-quieting `v_max_f32 x, x, x` for every operand it cannot prove
-// canonical (anything that crosses a basic block), which doubles the cost of a reduction.  The
-// hardware instruction already returns the other operand when one is a NaN, like fmaxf.
+// v_max_f32 / v_max3_f32 as single instructions.  In front of fmaxf the compiler puts a NaN-quieting
+// `v_max_f32 x, x, x` for every operand it cannot prove canonical (anything that crosses a basic
+// block), which doubles the cost of a reduction.  The hardware instruction already returns the
+// other operand when one is a NaN, like fmaxf.
 __device__ __forceinline__ float vmax(float a, float b) {
   float r;
   asm("v_max_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
   return r;
 }
-__device__ __forceinline__ float vmin(float a, float b) {
-  float r;
-  asm("v_min_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
-  return r;
-}
 __device__ __forceinline__ float vmax3(float a, float b, float c) {
   float r;
   asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
-  return r;
-}
-__device__ __forceinline__ float vmin3(float a, float b, float c) {
-  float r;
-  asm("v_min3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
   return r;
 }
 
