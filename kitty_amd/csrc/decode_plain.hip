@@ -172,28 +172,38 @@ __global__ __launch_bounds__(256) void decode_plain_kernel(kitty_kv_layer L, con
 }
 
 // out[b, 0, hq, :] = sum_s acc_s * 2^(m_s - m) / sum_s l_s * 2^(m_s - m); the running maxima of
-// the partials are in log2 units.  One block per (32 channels, query head, batch row): 8 groups
-// of 32 lanes stride over the splits, then combine through LDS in a fixed order.
-constexpr int kMergeGroups = 8, kMergeChannels = 32;
-__global__ __launch_bounds__(kMergeGroups * kMergeChannels) void decode_merge_kernel(
+// the partials are in log2 units.  One block per (32 channels, query head, batch row).  The maximum
+// over the splits is taken with one load per thread and a block reduction; then GROUPS groups of
+// 32 lanes stride over the splits, four loads in flight each, and combine through LDS in a fixed
+// order.  GROUPS = 8 up to 32 splits (2 when there are thousands of blocks), 32 beyond (a long
+// sequence at batch 1 has hundreds of splits).
+constexpr int kMergeChannels = 32;
+template <int GROUPS>
+__global__ __launch_bounds__(GROUPS * kMergeChannels) void decode_merge_kernel(
     const float* __restrict__ ws_ml, const float* __restrict__ ws_acc, __half* __restrict__ out, int num_splits) {
-  __shared__ float s_m[kMergeGroups], s_l[kMergeGroups], s_o[kMergeGroups][kMergeChannels];
+  constexpr int kThreads = GROUPS * kMergeChannels, kWaves = kThreads / 64;
+  __shared__ float s_m[kWaves], s_l[GROUPS], s_o[GROUPS][kMergeChannels];
   const int64_t head = (int64_t)blockIdx.z * gridDim.y + blockIdx.y;
   const int64_t row0 = head * num_splits;
   const int lane = threadIdx.x & (kMergeChannels - 1), grp = threadIdx.x / kMergeChannels;
   const int d = blockIdx.x * kMergeChannels + lane;
   float m = -INFINITY;
-  for (int s = grp; s < num_splits; s += kMergeGroups) m = fmaxf(m, ws_ml[(row0 + s) * 2]);
-  if (lane == 0) s_m[grp] = m;
+  for (int s = threadIdx.x; s < num_splits; s += kThreads) m = fmaxf(m, ws_ml[(row0 + s) * 2]);
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o));
+  if ((threadIdx.x & 63) == 0) s_m[threadIdx.x >> 6] = m;
   __syncthreads();
 #pragma unroll
-  for (int g = 0; g < kMergeGroups; ++g) m = fmaxf(m, s_m[g]);
+  for (int w = 0; w < kWaves; ++w) m = fmaxf(m, s_m[w]);
   float l = 0.f, o = 0.f;
-  for (int s = grp; s < num_splits; s += kMergeGroups) {
+#pragma unroll 4
+  for (int s = grp; s < num_splits; s += GROUPS) {
     const float ms = ws_ml[(row0 + s) * 2];
+    const float ls = ws_ml[(row0 + s) * 2 + 1];
+    const float as = ws_acc[(row0 + s) * kD + d];
     const float w = (ms == -INFINITY) ? 0.f : exp2f(ms - m);
-    l += ws_ml[(row0 + s) * 2 + 1] * w;
-    o += ws_acc[(row0 + s) * kD + d] * w;
+    l += ls * w;
+    o += as * w;
   }
   if (lane == 0) s_l[grp] = l;
   s_o[grp][lane] = o;
@@ -201,7 +211,7 @@ __global__ __launch_bounds__(kMergeGroups * kMergeChannels) void decode_merge_ke
   if (grp == 0) {
     l = 0.f, o = 0.f;
 #pragma unroll
-    for (int g = 0; g < kMergeGroups; ++g) { l += s_l[g]; o += s_o[g][lane]; }
+    for (int g = 0; g < GROUPS; ++g) { l += s_l[g]; o += s_o[g][lane]; }
     out[head * kD + d] = __float2half_rn(l > 0.f ? o / l : 0.f);
   }
 }
@@ -214,8 +224,16 @@ void launch_decode_plain(const kitty_kv_layer& L, const void* q, int B, int H_Q,
 
 void launch_decode_merge(const float* ws_ml, const float* ws_acc, void* out, int B, int H_Q, int num_splits,
                          hipStream_t stream) {
-  hipLaunchKernelGGL(decode_merge_kernel, dim3(kD / kMergeChannels, H_Q, B), dim3(kMergeGroups * kMergeChannels), 0,
-                     stream, ws_ml, ws_acc, (__half*)out, num_splits);
+  const dim3 grid(kD / kMergeChannels, H_Q, B);
+  if (num_splits <= 32 && (int64_t)grid.x * grid.y * grid.z >= 4096)   // large batch: one wave per block, all resident at once
+    hipLaunchKernelGGL(decode_merge_kernel<2>, grid, dim3(2 * kMergeChannels), 0, stream, ws_ml, ws_acc, (__half*)out,
+                       num_splits);
+  else if (num_splits <= 32)
+    hipLaunchKernelGGL(decode_merge_kernel<8>, grid, dim3(8 * kMergeChannels), 0, stream, ws_ml, ws_acc, (__half*)out,
+                       num_splits);
+  else
+    hipLaunchKernelGGL(decode_merge_kernel<32>, grid, dim3(32 * kMergeChannels), 0, stream, ws_ml, ws_acc,
+                       (__half*)out, num_splits);
 }
 
 }  // namespace kitty
