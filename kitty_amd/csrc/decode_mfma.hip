@@ -832,7 +832,8 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(kitty_kv_layer L, co
   // ("tail": the sink, and the one or two tiles with fp16 rows on either side).  The tail takes the
   // FIRST splits, so that its long-latency waves start with the launch and run beside the body: one
   // split when a body split is long enough to hide it (12 tiles or more), else three (sink / first
-  // tail tile / the others).  The remaining splits share the body evenly.  1 split: everything.
+  // tail tile / the others).  The remaining splits share the body evenly (tile counts differ by at
+  // most one).  1 split: everything.
   const int nbt = c_div_up(x.c.nbody, kPage);
   const int npp = min(min(x.c.pv, x.c.pk), nbt);
   const int n_tail = num_splits >= 4 && npp < 12 * (num_splits - 3) ? 3 : (num_splits >= 2 ? 1 : 0);
@@ -847,9 +848,11 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(kitty_kv_layer L, co
     else if (split == 1) { u0 = npp; u1 = min(nbt, npp + 1); }
     else u0 = min(nbt, npp + 1);
   } else {
-    const int n_body = num_splits - n_tail;
-    const int per = (npp + n_body - 1) / n_body;
-    t0 = min(npp, (split - n_tail) * per); t1 = min(npp, t0 + per);
+    // even shares: the first npp % n_body splits take one tile more
+    const int n_body = num_splits - n_tail, i_body = split - n_tail;
+    const int base = npp / n_body, rem = npp - base * n_body;
+    t0 = i_body * base + min(i_body, rem);
+    t1 = t0 + base + (i_body < rem ? 1 : 0);
   }
   const bool tail = do_sink || u0 < u1;
   const uint8_t* qbuf_k = (const uint8_t*)L.qbuf_k + (int64_t)x.b * L.win_stride_b + (int64_t)x.h * L.win_stride_h;
