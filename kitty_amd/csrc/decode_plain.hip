@@ -201,7 +201,8 @@ __global__ __launch_bounds__(GROUPS * kMergeChannels) void decode_merge_kernel(
     const float ms = ws_ml[(row0 + s) * 2];
     const float ls = ws_ml[(row0 + s) * 2 + 1];
     const float as = ws_acc[(row0 + s) * kD + d];
-    const float w = (ms == -INFINITY) ? 0.f : exp2f(ms - m);
+    if (ms == -INFINITY) continue;   // an empty split: its accumulator row may never have been written
+    const float w = exp2f(ms - m);
     l += ls * w;
     o += as * w;
   }
