@@ -123,14 +123,22 @@ __device__ __forceinline__ void quant_k_page(const uint8_t* __restrict__ src_pag
   const int tg = tid >> 4;   // tokens tg*8 .. tg*8+7
   const int c8 = tid & 15;   // channels c8*8 .. c8*8+7
 
-  __shared__ float s_pmin[16][kD];
-  __shared__ float s_pmax[16][kD];
-  __shared__ double s_psum[MODE == 0 ? 1 : 16][kD];
-  __shared__ float4 s_q[kD];   // per channel: min, scale, refined reciprocal of the scale, qmax + 0.5
-  __shared__ float s_c0[kD];   // per channel: the fast path's offset (fast_offset)
+  // LDS layouts are chosen so that the 64 lanes of an access fall on 64 different banks.  Per-channel
+  // tables are indexed by pos(channel) = (channel % 8) * 16 + channel / 8: the 16 lanes that share a
+  // token group work on channels 8 apart and so read / write consecutive entries.  Rows of partials
+  // (one per token group) are 144 entries apart, which moves each of the four token groups of a
+  // wave to its own quarter (floats) or half (doubles, two passes) of the banks.
+  constexpr int kPitch = kD + 16;
+  __shared__ __attribute__((aligned(16))) float s_pmin[16][kPitch];   // later: the low plane on its way out
+  __shared__ float s_pmax[16][kPitch];
+  __shared__ double s_psum[MODE == 0 ? 1 : 16][kPitch];
+  __shared__ float4 s_q[kD];   // [pos]: min, scale, refined reciprocal of the scale, qmax + 0.5
+  __shared__ float s_c0[kD];   // [pos]: the fast path's offset (fast_offset)
   __shared__ __attribute__((aligned(16))) uint32_t s_key[kD];   // score << 8 | (127 - channel): larger sorts first
-  __shared__ __attribute__((aligned(16))) uint8_t s_idx[kD];
-  __shared__ __attribute__((aligned(16))) uint16_t s_lo[kD * 16];
+  __shared__ __attribute__((aligned(16))) uint8_t s_idx[kD];    // slot by channel, as it is stored
+  __shared__ uint8_t s_idx_p[kD];                               // [pos]
+  static_assert(sizeof(s_pmin) >= kD * 32, "the low plane reuses the minima");
+  uint8_t* const s_lo = (uint8_t*)&s_pmin[0][0];
 
   const uint8_t* src = src_page + (int64_t)(tg * 8) * stride_t + c8 * 16;
   uint4 rows[8];
@@ -155,27 +163,29 @@ __device__ __forceinline__ void quant_k_page(const uint8_t* __restrict__ src_pag
       mx = fmaxf(mx, xs[j][r]);
       if (MODE != 0) sum += (double)fabsf(xs[j][r]);
     }
-    s_pmin[tg][c8 * 8 + j] = mn;
-    s_pmax[tg][c8 * 8 + j] = mx;
-    if (MODE != 0) s_psum[tg][c8 * 8 + j] = sum;
+    s_pmin[tg][j * 16 + c8] = mn;
+    s_pmax[tg][j * 16 + c8] = mx;
+    if (MODE != 0) s_psum[tg][j * 16 + c8] = sum;
   }
   __syncthreads();
 
   // Second stage on lane pairs: lanes 2c and 2c+1 each fold 8 of channel c's 16 partials, then
   // exchange; with selection they also split the 128 comparisons of the ranking.
-  const int ch = tid >> 1, hf = tid & 1;
-  float ch_min = s_pmin[hf][ch], ch_max = s_pmax[hf][ch];
+  // (the pair's channel follows the table order, so that its reads are consecutive too)
+  const int pos = tid >> 1, hf = tid & 1;
+  const int ch = (pos & 15) * 8 + (pos >> 4);
+  float ch_min = s_pmin[hf][pos], ch_max = s_pmax[hf][pos];
 #pragma unroll
   for (int i = 2; i < 16; i += 2) {
-    ch_min = fminf(ch_min, s_pmin[i + hf][ch]);
-    ch_max = fmaxf(ch_max, s_pmax[i + hf][ch]);
+    ch_min = fminf(ch_min, s_pmin[i + hf][pos]);
+    ch_max = fmaxf(ch_max, s_pmax[i + hf][pos]);
   }
   ch_min = fminf(ch_min, __shfl_xor(ch_min, 1));
   ch_max = fmaxf(ch_max, __shfl_xor(ch_max, 1));
   if (MODE != 0) {
     double sum = 0.0;
 #pragma unroll
-    for (int i = 0; i < 16; i += 2) sum += s_psum[i + hf][ch];
+    for (int i = 0; i < 16; i += 2) sum += s_psum[i + hf][pos];
     sum += __shfl_xor(sum, 1);
     // an integer below 2^47 (or inf / nan for non-finite inputs, which saturate)
     if (hf == 0)
@@ -195,6 +205,7 @@ __device__ __forceinline__ void quant_k_page(const uint8_t* __restrict__ src_pag
     const uint8_t slot = (uint8_t)(rank < d_boost ? rank : d_boost);
     if (hf == 0) {
       s_idx[ch] = slot;
+      s_idx_p[pos] = slot;
       if (slot_out) slot_out[ch] = slot;
     }
     if (MODE == 2) return;
@@ -203,41 +214,43 @@ __device__ __forceinline__ void quant_k_page(const uint8_t* __restrict__ src_pag
       float scale = (ch_max - ch_min) / qmax;
       scale = scale < 1e-6f ? 1e-6f : scale;
       const Divisor k = make_divisor(scale);
-      s_q[ch] = float4{ch_min, k.d, k.r, qmax + 0.5f};
-    s_c0[ch] = fast_offset(ch_min, k);
-      s_c0[ch] = fast_offset(ch_min, k);
+      s_q[pos] = float4{ch_min, k.d, k.r, qmax + 0.5f};
+      s_c0[pos] = fast_offset(ch_min, k);
       *(__half2*)(meta_dst + ch * 4) = __halves2half2(__float2half_rn(scale), __float2half_rn(ch_min));
     }
   } else if (hf == 0) {
     const uint8_t slot = slot_in[ch];
     s_idx[ch] = slot;
+    s_idx_p[pos] = slot;
     const float qmax = slot < d_boost ? 15.0f : 3.0f;
     float scale = (ch_max - ch_min) / qmax;
     scale = scale < 1e-6f ? 1e-6f : scale;
     const Divisor k = make_divisor(scale);
-    s_q[ch] = float4{ch_min, k.d, k.r, qmax + 0.5f};
-    s_c0[ch] = fast_offset(ch_min, k);
+    s_q[pos] = float4{ch_min, k.d, k.r, qmax + 0.5f};
+    s_c0[pos] = fast_offset(ch_min, k);
     *(__half2*)(meta_dst + ch * 4) = __halves2half2(__float2half_rn(scale), __float2half_rn(ch_min));
   }
-  __syncthreads();
+  __syncthreads();   // the tables are complete, and nobody reads the partial minima any more (s_lo takes their place)
 
 #pragma unroll
   for (int j = 0; j < 8; ++j) {
-    const int d = c8 * 8 + j;
-    const float4 qp = s_q[d];
+    const int d = c8 * 8 + j, dp = j * 16 + c8;
+    const float4 qp = s_q[dp];
     const Divisor k = {qp.y, qp.z};
     // the 8 codes (0..15) as one word of nibbles, built in floating point (exact: 16 bits per half)
     float c[8];
-    codes_of<8>(xs[j], qp.x, s_c0[d], k, qp.w, c);
+    codes_of<8>(xs[j], qp.x, s_c0[dp], k, qp.w, c);
     const float h0 = __builtin_fmaf(__builtin_fmaf(__builtin_fmaf(c[3], 16.f, c[2]), 16.f, c[1]), 16.f, c[0]);
     const float h1 = __builtin_fmaf(__builtin_fmaf(__builtin_fmaf(c[7], 16.f, c[6]), 16.f, c[5]), 16.f, c[4]);
     const uint32_t nib = (uint32_t)h0 | ((uint32_t)h1 << 16);
-    s_lo[d * 16 + tg] = (uint16_t)gather_fields<0>(nib);
-    const uint8_t slot = s_idx[d];
+    // plane row d, tokens 8 tg ..: byte d * 32 + 2 tg, with the row's 16-byte pieces and its three
+    // row-in-octet bits flipped by c8 so that the 16 rows written at once (8 apart) spread over the banks
+    *(uint16_t*)(s_lo + ((d * 32 + tg * 2) ^ (c8 << 4))) = (uint16_t)gather_fields<0>(nib);
+    const uint8_t slot = s_idx_p[dp];
     if (slot < d_boost) *(uint16_t*)(dst + kLoBytes + slot * kRowBytes + tg * 2) = (uint16_t)gather_fields<2>(nib);
   }
   __syncthreads();
-  ((uint4*)dst)[tid] = ((const uint4*)s_lo)[tid];
+  ((uint4*)dst)[tid] = *(const uint4*)(s_lo + ((tid * 16) ^ (((tid >> 4) & 15) << 4)));   // piece tid of the plane: row tid / 2, c8 = row / 8
   if (tid < kD / 4) ((uint32_t*)(dst + kRowBytes * (kD + d_boost)))[tid] = ((const uint32_t*)s_idx)[tid];
 }
 
