@@ -284,11 +284,17 @@ __device__ __forceinline__ void quant_v_page(const uint8_t* __restrict__ src_pag
   const int tid = threadIdx.x;
   const int cg = tid & 7;
   const uint8_t* src = src_page + cg * 32;
+  uint4 la[4], lc[4];   // all eight loads of the thread are in flight before the first is used
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int t = (tid >> 3) + 32 * i;
-    const uint4 a = *(const uint4*)(src + (int64_t)t * stride_t);
-    const uint4 c = *(const uint4*)(src + (int64_t)t * stride_t + 16);
+    la[i] = *(const uint4*)(src + (int64_t)t * stride_t);
+    lc[i] = *(const uint4*)(src + (int64_t)t * stride_t + 16);
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int t = (tid >> 3) + 32 * i;
+    const uint4 a = la[i], c = lc[i];
     const uint32_t w[8] = {a.x, a.y, a.z, a.w, c.x, c.y, c.z, c.w};
     float x[16];
     float mn = INFINITY, mx = -INFINITY;
