@@ -253,7 +253,8 @@ __device__ __forceinline__ void k_load_regs(const Ctx& x, int page_index, KRegs&
 
 // Global -> LDS loads of one K page-head (no registers involved): scalar base + per-lane offset,
 // the LDS destination is M0 + instruction offset + lane * size.  8 instructions with the high
-// plane, 6 without.
+// plane, 6 without.  Every tile is read exactly once, so the loads are marked non-temporal (2 % on the
+// whole launch; a read-only stream runs at 6.5 TB/s with the hint and 5.9 TB/s without).
 template <bool BOOST>
 constexpr int kDmaK = BOOST ? 8 : 6;
 constexpr int kDmaV = 6;
@@ -267,21 +268,21 @@ __device__ __forceinline__ void dma_k(const Ctx& x, int page_index, uint32_t lds
   const uint32_t off16 = x.lane * 16, off4 = x.lane * 4, off4dup = (x.lane & 31) * 4;
   asm volatile(
       "s_mov_b32 m0, %2\n\t"
-      "global_load_lds_dwordx4 %0, %1\n\t"
-      "global_load_lds_dwordx4 %0, %1 offset:1024\n\t"
-      "global_load_lds_dwordx4 %0, %1 offset:2048\n\t"
-      "global_load_lds_dwordx4 %0, %1 offset:3072"
+      "global_load_lds_dwordx4 %0, %1 nt\n\t"
+      "global_load_lds_dwordx4 %0, %1 offset:1024 nt\n\t"
+      "global_load_lds_dwordx4 %0, %1 offset:2048 nt\n\t"
+      "global_load_lds_dwordx4 %0, %1 offset:3072 nt"
       :: "v"(off16), "s"(page), "s"(lds) : "memory", "m0");
   if (BOOST) {
-    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1"
+    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1 nt"
                  :: "v"(off16), "s"(page + kLoBytes), "s"(lds + kKOffHi) : "memory", "m0");
-    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dword %0, %1"
+    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dword %0, %1 nt"
                  :: "v"(off4dup), "s"(page + kLoBytes + 1024), "s"(lds + kKOffIdx) : "memory", "m0");
   }
   asm volatile(
       "s_mov_b32 m0, %2\n\t"
-      "global_load_lds_dword %0, %1\n\t"
-      "global_load_lds_dword %0, %1 offset:256"
+      "global_load_lds_dword %0, %1 nt\n\t"
+      "global_load_lds_dword %0, %1 offset:256 nt"
       :: "v"(off4), "s"(meta), "s"(lds + kKOffMeta) : "memory", "m0");
 }
 
@@ -573,16 +574,16 @@ __device__ __forceinline__ void dma_v(const Ctx& x, int page_index, uint32_t lds
   const uint32_t off16 = x.lane * 16;
   asm volatile(
       "s_mov_b32 m0, %2\n\t"
-      "global_load_lds_dwordx4 %0, %1\n\t"
-      "global_load_lds_dwordx4 %0, %1 offset:1024\n\t"
-      "global_load_lds_dwordx4 %0, %1 offset:2048\n\t"
-      "global_load_lds_dwordx4 %0, %1 offset:3072"
+      "global_load_lds_dwordx4 %0, %1 nt\n\t"
+      "global_load_lds_dwordx4 %0, %1 offset:1024 nt\n\t"
+      "global_load_lds_dwordx4 %0, %1 offset:2048 nt\n\t"
+      "global_load_lds_dwordx4 %0, %1 offset:3072 nt"
       :: "v"(off16), "s"(page), "s"(lds) : "memory", "m0");
   const uint32_t off4 = x.lane * 4;
   asm volatile(
       "s_mov_b32 m0, %2\n\t"
-      "global_load_lds_dword %0, %1\n\t"
-      "global_load_lds_dword %0, %1 offset:256"
+      "global_load_lds_dword %0, %1 nt\n\t"
+      "global_load_lds_dword %0, %1 offset:256 nt"
       :: "v"(off4), "s"(meta), "s"(lds + kVOffMeta) : "memory", "m0");
 }
 

@@ -40,6 +40,14 @@ __device__ inline uint16_t mean_abs_fp16_bits(uint64_t S) {
   return (uint16_t)q;
 }
 
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+// 16 bytes of the source, which is read exactly once: a non-temporal load (a read-only stream
+// reaches 6.5 TB/s with them on this part, 5.9 TB/s without)
+__device__ __forceinline__ uint4 nt_load16(const uint8_t* p) {
+  const u32x4 v = __builtin_nontemporal_load((const u32x4*)p);
+  return uint4{v.x, v.y, v.z, v.w};
+}
+
 __device__ inline float h2f(uint16_t bits) { return __half2float(__ushort_as_half(bits)); }
 
 // IEEE fp32 division by a divisor that is shared by a whole group.  This is the correctly rounded
@@ -143,7 +151,7 @@ __device__ __forceinline__ void quant_k_page(const uint8_t* __restrict__ src_pag
   const uint8_t* src = src_page + (int64_t)(tg * 8) * stride_t + c8 * 16;
   uint4 rows[8];
 #pragma unroll
-  for (int r = 0; r < 8; ++r) rows[r] = *(const uint4*)(src + (int64_t)r * stride_t);
+  for (int r = 0; r < 8; ++r) rows[r] = nt_load16(src + (int64_t)r * stride_t);
 
   // this thread's 8 tokens x 8 channels as floats, and per channel the partial min / max (/ sum
   // of |x|: exact in fp64, every term is a multiple of 2^-24 below 2^16)
@@ -288,8 +296,8 @@ __device__ __forceinline__ void quant_v_page(const uint8_t* __restrict__ src_pag
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int t = (tid >> 3) + 32 * i;
-    la[i] = *(const uint4*)(src + (int64_t)t * stride_t);
-    lc[i] = *(const uint4*)(src + (int64_t)t * stride_t + 16);
+    la[i] = nt_load16(src + (int64_t)t * stride_t);
+    lc[i] = nt_load16(src + (int64_t)t * stride_t + 16);
   }
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
