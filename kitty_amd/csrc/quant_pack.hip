@@ -331,7 +331,7 @@ __device__ __forceinline__ void quant_v_page(const uint8_t* __restrict__ src_pag
       h1 = __builtin_fmaf(h1, 4.f, code[8 + k]);
     }
     const uint32_t packed = (uint32_t)h0 | ((uint32_t)h1 << 16);
-    *(uint32_t*)(dst + t * kRowBytes + cg * 4) = packed;
+    __builtin_nontemporal_store(packed, (uint32_t*)(dst + t * kRowBytes + cg * 4));   // written once, read much later
     if (cg == 0) *(__half2*)(mdst + t * 4) = __halves2half2(__float2half_rn(scale), __float2half_rn(mn));
   }
 }
