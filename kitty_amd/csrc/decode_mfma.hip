@@ -862,41 +862,47 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(kitty_kv_layer L, co
   if constexpr (DMA) {
     // Tiles stream through LDS: two K buffers, one V buffer.  Issue order
     //   K(t0) K(t0+1) V(t0) | QK(i) -> K(i+2) -> softmax -> PV(i) -> V(i+1) | ...
-    // so K(i) has a lead of one and a half iterations and V(i) of half an iteration.  Loads past
-    // the end re-read the last tile, which keeps the number in flight static: the waits below
-    // count instructions issued AFTER the tile that is needed.
+    // so K(i) has a lead of one and a half iterations and V(i) of half an iteration.  The waits
+    // count the instructions issued AFTER the tile that is needed; nothing is loaded past the end
+    // of the range (the last two iterations wait on shorter queues).
     if (t0 < t1) {
       constexpr int nK = kDmaK<BOOST>;
       const uint32_t lk0 = (uint32_t)(uintptr_t)&S.kbuf[0][0], lk1 = (uint32_t)(uintptr_t)&S.kbuf[1][0];
       const uint32_t lv = (uint32_t)(uintptr_t)&S.vbuf[0];
       dma_k<BOOST>(x, t0, lk0);
-      dma_k<BOOST>(x, min(t0 + 1, t1 - 1), lk1);
+      if (t0 + 1 < t1) dma_k<BOOST>(x, t0 + 1, lk1);
       dma_v(x, t0, lv);
 #pragma unroll 1
       for (int i = t0; i < t1; ++i) {
         float cz;
         const int buf = (i - t0) & 1;
-        if (i == t0) wait_vmcnt<nK + kDmaV>(); else wait_vmcnt<nK + 2 * kDmaV>();
+        const bool k1 = i + 1 < t1, k2 = i + 2 < t1;   // K(i+1) has been, K(i+2) will be asked for
+        // K(i) is followed in the queue by V(i-1) (not in the first iteration), K(i+1) if any, V(i)
+        if (i == t0) {
+          if (k1) wait_vmcnt<nK + kDmaV>(); else wait_vmcnt<kDmaV>();
+        } else {
+          if (k1) wait_vmcnt<nK + 2 * kDmaV>(); else wait_vmcnt<2 * kDmaV>();
+        }
         __builtin_amdgcn_s_setprio(KITTY_PRIO_MFMA);
         qk_packed<BOOST, SPLIT_COLS, !QUARTER>(S, x, KLds{S.kbuf[buf]}, C, cz);
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-        dma_k<BOOST>(x, min(i + 2, t1 - 1), buf ? lk1 : lk0);
+        if (k2) dma_k<BOOST>(x, i + 2, buf ? lk1 : lk0);
         __builtin_amdgcn_s_setprio(KITTY_PRIO_VALU);
         if constexpr (QUARTER) {
           float4v own[2];
           combine_quarter(x, C, own);
           softmax_quarter(x, A, own, cz);
-          wait_vmcnt<nK>();
+          if (k2) wait_vmcnt<nK>(); else wait_vmcnt<0>();   // V(i) is followed by K(i+2) if any
           __builtin_amdgcn_s_setprio(KITTY_PRIO_MFMA);
           pv_quarter(S, x, A.out, A.lz, VLds{S.vbuf}, own);
         } else {
           softmax_tile<true>(x, A, C, cz, kPage);
-          wait_vmcnt<nK>();
+          if (k2) wait_vmcnt<nK>(); else wait_vmcnt<0>();
           __builtin_amdgcn_s_setprio(KITTY_PRIO_MFMA);
           pv_packed(S, x, A.out, A.lz, VLds{S.vbuf}, C);
         }
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-        dma_v(x, min(i + 1, t1 - 1), lv);
+        if (k1) dma_v(x, i + 1, lv);
       }
       wait_vmcnt<0>();
     }
