@@ -103,6 +103,12 @@ def test_host_side_rejection_without_gpu(lib):
     assert lib.kitty_decode_attn_workspace_bytes(16, 32, 64, 16) == 0
     assert 1 <= lib.kitty_decode_attn_default_splits(16, 8, 257) <= 257
     assert lib.kitty_decode_attn_default_splits(1, 8, 1025) > lib.kitty_decode_attn_default_splits(16, 8, 1025)
+    # long splits: two waves per SIMD of the 256 CUs; short splits (under 8 tiles): 15/16 of that;
+    # never fewer than 4 tiles per body split
+    assert lib.kitty_decode_attn_default_splits(16, 8, 257) == 16
+    assert lib.kitty_decode_attn_default_splits(1, 8, 1025) == 240
+    assert lib.kitty_decode_attn_default_splits(1, 8, 33) == 33 // 4 + 1 + 3
+    assert lib.kitty_decode_attn_default_splits(0, 8, 33) == 1
 
 
 def test_missing_library_fails_loudly(monkeypatch, tmp_path):
