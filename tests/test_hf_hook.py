@@ -1,0 +1,116 @@
+"""The hook for stock transformers attention modules (kitty_amd/hf.py)."""
+import numpy as np
+import pytest
+import torch
+
+transformers = pytest.importorskip("transformers")
+
+
+def _tiny_llama(attn):
+    from transformers import LlamaConfig, LlamaForCausalLM
+    cfg = LlamaConfig(vocab_size=256, hidden_size=256, intermediate_size=512, num_hidden_layers=2,
+                      num_attention_heads=2, num_key_value_heads=1, head_dim=128, max_position_embeddings=4096,
+                      attn_implementation=attn)
+    torch.manual_seed(0)
+    return LlamaForCausalLM(cfg)
+
+
+def test_register_and_cache_adapter_on_cpu():
+    from kitty_amd import hf
+    hf.register()
+    hf.register()                                   # idempotent
+    from transformers.modeling_utils import ALL_ATTENTION_FUNCTIONS
+    assert ALL_ATTENTION_FUNCTIONS[hf.NAME] is hf.kitty_attention
+    model = _tiny_llama("kitty")                    # the name is accepted by a stock model
+    assert model.config._attn_implementation == "kitty"
+    cache = hf.KittyHFCache(model.config, 1, 256, device="cpu")
+    k = torch.randn(1, 1, 40, 128, dtype=torch.float16)
+    v = torch.randn(1, 1, 40, 128, dtype=torch.float16)
+    rk, rv = cache.update(k, v, 0)
+    assert rk is k and rv is v and hf._current.phase == "prefill" and hf._current.cache is cache
+    assert cache.get_mask_sizes(40, 0) == (40, 0)
+    assert cache.get_seq_length(0) == 0             # nothing is counted before quantize_prefill, as in the reference
+
+
+@pytest.mark.gpu
+def test_stock_llama_matches_dense_attention_while_everything_is_fp16():
+    """Prompt of 20 tokens and 60 decode steps: 80 tokens fit the sink and the fp16 windows, nothing
+    is quantized, so the logits must agree with the same model on torch's dense attention."""
+    if not torch.cuda.is_available():
+        pytest.skip("needs a GPU")
+    from transformers import DynamicCache
+    from kitty_amd import hf
+    hf.register()
+    dev = torch.device("cuda")
+    ref = _tiny_llama("sdpa").to(dev).half().eval()
+    mod = _tiny_llama("kitty").to(dev).half().eval()
+    mod.load_state_dict(ref.state_dict())
+    B, T0, steps = 2, 20, 60
+    ids = torch.randint(0, 256, (B, T0), generator=torch.Generator().manual_seed(1)).to(dev)
+    c_ref, c_mod = DynamicCache(), hf.KittyHFCache(mod.config, B, 512, device=dev)
+    with torch.no_grad():
+        cur = ids
+        for s in range(steps + 1):
+            a = ref(input_ids=cur, past_key_values=c_ref, use_cache=True).logits[:, -1].float()
+            b = mod(input_ids=cur, past_key_values=c_mod, use_cache=True).logits[:, -1].float()
+            assert torch.isfinite(b).all()
+            assert (a - b).abs().max().item() <= 3e-2, (s, (a - b).abs().max().item())
+            cur = a.argmax(-1, keepdim=True)
+    assert c_mod.get_seq_length(0) == T0 + steps
+    L = c_mod.kv_cache[1]
+    assert (L.Sink_Count, L.PageCount_K, L.Q_Buffer_Count_K) == (32, 0, T0 + steps - 32)
+    # generate() drives the same cache (greedy tokens are not compared: with random weights the top
+    # two logits are often closer than fp16 attention kernels agree)
+    with torch.no_grad():
+        gen_cache = hf.KittyHFCache(mod.config, B, 512, device=dev)
+        got = mod.generate(ids, past_key_values=gen_cache, max_new_tokens=12, do_sample=False, pad_token_id=0)
+    assert tuple(got.shape) == (B, T0 + 12) and torch.equal(got[:, :T0], ids)
+    assert gen_cache.get_seq_length(0) == T0 + 11          # the last token is returned, not fed back
+
+
+@pytest.mark.gpu
+def test_stock_llama_long_prompt_decode_and_chunk():
+    """A prompt that is packed, decode steps across flushes, then a chunk of new tokens: the cache
+    goes through the reference's state machine and the logits stay close to dense attention."""
+    if not torch.cuda.is_available():
+        pytest.skip("needs a GPU")
+    from transformers import DynamicCache
+    from kitty_amd import hf
+    from oracle import kitty_oracle as O
+    hf.register()
+    dev = torch.device("cuda")
+    ref = _tiny_llama("sdpa").to(dev).half().eval()
+    mod = _tiny_llama("kitty").to(dev).half().eval()
+    mod.load_state_dict(ref.state_dict())
+    B, T0, steps, chunk = 1, 300, 150, 70
+    g = torch.Generator().manual_seed(2)
+    ids = torch.randint(0, 256, (B, T0), generator=g).to(dev)
+    c_ref, c_mod = DynamicCache(), hf.KittyHFCache(mod.config, B, 1024, device=dev)
+    ol = O.OracleLayer(B, 1024, 1)                                  # counters only: the state machine
+    zeros = lambda n: np.zeros((B, 1, n, 128), np.float16)
+    with torch.no_grad():
+        cur, cos = ids, []
+        for s in range(steps + 1):
+            a = ref(input_ids=cur, past_key_values=c_ref, use_cache=True).logits[:, -1].float()
+            b = mod(input_ids=cur, past_key_values=c_mod, use_cache=True).logits[:, -1].float()
+            assert torch.isfinite(b).all()
+            cos.append(torch.nn.functional.cosine_similarity(a, b, dim=-1).min().item())
+            n = cur.shape[1]
+            if s == 0:
+                ol.update(zeros(n), zeros(n)); ol.quantize_prefill()
+            else:
+                ol.update(zeros(1), zeros(1)); ol.quantize_decode()
+            cur = a.argmax(-1, keepdim=True)
+        L = c_mod.kv_cache[0]
+        for f in ("Sink_Count", "PageCount_K", "PageCount_V", "Q_Buffer_Count_K", "Q_Buffer_Count_V", "Local_Count_V",
+                  "Write_Offset_Local_V"):
+            assert getattr(L, f) == getattr(ol, f), f
+        more = torch.randint(0, 256, (B, chunk), generator=g).to(dev)
+        b = mod(input_ids=more, past_key_values=c_mod, use_cache=True).logits.float()
+        a = ref(input_ids=more, past_key_values=c_ref, use_cache=True).logits.float()
+        assert torch.isfinite(b).all() and b.shape == a.shape
+        assert c_mod.get_seq_length(0) == T0 + steps + chunk
+    # 2-bit pages disturb the logits only a little: every step's logit vector points the same way as
+    # dense attention's (random weights leave the argmax itself nearly tied, so it is not compared)
+    print("cosine similarity of the logits: min %.4f mean %.4f" % (min(cos), sum(cos) / len(cos)))
+    assert min(cos) >= 0.97, min(cos)
