@@ -216,6 +216,7 @@ struct Prefill {
       // thread = one channel, 16 kW tokens: plane words of 16 tokens each
       const half2v m2 = __builtin_bit_cast(half2v, g.kmeta);
       const half2v scale = {m2[0], m2[0]}, zero = {m2[1], m2[1]};
+      const uint32_t k01 = dequant_pair(0x00010000u, scale, zero), k23 = dequant_pair(0x00030002u, scale, zero);
       uint8_t* row = kt + e * kPitch + part * kPartBytes;
 #pragma unroll
       for (int w = 0; w < kW; ++w) {
@@ -223,8 +224,12 @@ struct Prefill {
 #pragma unroll
         for (int u = 0; u < 8; ++u) {
           uint32_t code = (g.klo[w] >> (2 * u)) & 0x00030003u;
-          if (BOOST) code |= ((g.khi[w] >> (2 * u)) & 0x00030003u) << 2;
-          o[u] = dequant_pair(code, scale, zero);
+          if (BOOST) {
+            code |= ((g.khi[w] >> (2 * u)) & 0x00030003u) << 2;
+            o[u] = dequant_pair(code, scale, zero);
+          } else {   // four values per channel: the table of the V side below
+            o[u] = __builtin_amdgcn_perm(k23, k01, code * 0x0202u + 0x01000100u);
+          }
         }
         *(uint4*)(row + w * 32) = uint4{o[0], o[1], o[2], o[3]};
         *(uint4*)(row + w * 32 + 16) = uint4{o[4], o[5], o[6], o[7]};
@@ -247,13 +252,20 @@ struct Prefill {
     uint8_t* vrow = vt + slot_of(e) * kPitch + part * kPartBytes;
     if (s.v_kind == SRC_PACKED) {
       // thread = one token, 16 kW channels: words of 16 channels each
+      // All of a token's codes share one (scale, zero) and take four values: the four dequantized
+      // numbers are computed once (same instructions as dequant_pair, so the same two roundings)
+      // and every pair of codes picks its two with a byte permute, selector bytes (2c, 2c+1).
       const half2v m2 = __builtin_bit_cast(half2v, g.vmeta);
       const half2v scale = {m2[0], m2[0]}, zero = {m2[1], m2[1]};
+      const uint32_t t01 = dequant_pair(0x00010000u, scale, zero), t23 = dequant_pair(0x00030002u, scale, zero);
 #pragma unroll
       for (int w = 0; w < kW; ++w) {
         uint32_t o[8];
 #pragma unroll
-        for (int u = 0; u < 8; ++u) o[u] = dequant_pair((g.v[w] >> (2 * u)) & 0x00030003u, scale, zero);
+        for (int u = 0; u < 8; ++u) {
+          const uint32_t codes = (g.v[w] >> (2 * u)) & 0x00030003u;
+          o[u] = __builtin_amdgcn_perm(t23, t01, codes * 0x0202u + 0x01000100u);
+        }
         *(uint4*)(vrow + w * 32) = uint4{o[0], o[1], o[2], o[3]};
         *(uint4*)(vrow + w * 32 + 16) = uint4{o[4], o[5], o[6], o[7]};
       }
