@@ -35,6 +35,8 @@
 //   C[u][j] of lane (kg, n) = token 32kg + 8j + u, column n.
 //   V plane rows are tokens: lane group kg owns rows 32kg .. 32kg+31 (its own tokens), k-chunk j
 //   = rows 32kg + 8j .. +7, d-tile u = channels {8n + u}; O^T[u][j] = channel 32kg + 8j + u.
+#include <type_traits>
+
 #include "decode_common.h"
 
 // Wave priority while a phase is dominated by matrix instructions / by vector instructions: the
@@ -872,38 +874,52 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(kitty_kv_layer L, co
       dma_k<BOOST>(x, t0, lk0);
       if (t0 + 1 < t1) dma_k<BOOST>(x, t0 + 1, lk1);
       dma_v(x, t0, lv);
+      // Of the two waves that share a SIMD the older one wins arbitration, and it is 8 % faster per
+      // tile.  When the launch is a single round (at most two workgroups per SIMD of the 256 CUs),
+      // the workgroups dispatched after every SIMD has one are the younger ones: they raise their
+      // priority by one level after the first quarter of their range, which evens out the finishes.
+      // (Two copies of the loop: the conditional priorities cost the other launches 1.5 %.)
+      constexpr uint32_t kSimds = 256 * 4;
+      const uint32_t n_wg = gridDim.x * gridDim.y * gridDim.z;
+      const uint32_t lin_id = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
+      const bool young = n_wg <= 2 * kSimds && lin_id >= kSimds;
+      auto loop = [&](auto switch_priority) {
+      constexpr bool SWITCH = decltype(switch_priority)::value;
 #pragma unroll 1
       for (int i = t0; i < t1; ++i) {
         float cz;
         const int buf = (i - t0) & 1;
         const bool k1 = i + 1 < t1, k2 = i + 2 < t1;   // K(i+1) has been, K(i+2) will be asked for
+        const bool fav = SWITCH && 4 * (i - t0) >= t1 - t0;
         // K(i) is followed in the queue by V(i-1) (not in the first iteration), K(i+1) if any, V(i)
         if (i == t0) {
           if (k1) wait_vmcnt<nK + kDmaV>(); else wait_vmcnt<kDmaV>();
         } else {
           if (k1) wait_vmcnt<nK + 2 * kDmaV>(); else wait_vmcnt<2 * kDmaV>();
         }
-        __builtin_amdgcn_s_setprio(KITTY_PRIO_MFMA);
+        if (fav) __builtin_amdgcn_s_setprio(KITTY_PRIO_MFMA + 1); else __builtin_amdgcn_s_setprio(KITTY_PRIO_MFMA);
         qk_packed<BOOST, SPLIT_COLS, !QUARTER>(S, x, KLds{S.kbuf[buf]}, C, cz);
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
         if (k2) dma_k<BOOST>(x, i + 2, buf ? lk1 : lk0);
-        __builtin_amdgcn_s_setprio(KITTY_PRIO_VALU);
+        if (fav) __builtin_amdgcn_s_setprio(KITTY_PRIO_VALU + 1); else __builtin_amdgcn_s_setprio(KITTY_PRIO_VALU);
         if constexpr (QUARTER) {
           float4v own[2];
           combine_quarter(x, C, own);
           softmax_quarter(x, A, own, cz);
           if (k2) wait_vmcnt<nK>(); else wait_vmcnt<0>();   // V(i) is followed by K(i+2) if any
-          __builtin_amdgcn_s_setprio(KITTY_PRIO_MFMA);
+          if (fav) __builtin_amdgcn_s_setprio(KITTY_PRIO_MFMA + 1); else __builtin_amdgcn_s_setprio(KITTY_PRIO_MFMA);
           pv_quarter(S, x, A.out, A.lz, VLds{S.vbuf}, own);
         } else {
           softmax_tile<true>(x, A, C, cz, kPage);
           if (k2) wait_vmcnt<nK>(); else wait_vmcnt<0>();
-          __builtin_amdgcn_s_setprio(KITTY_PRIO_MFMA);
+          if (fav) __builtin_amdgcn_s_setprio(KITTY_PRIO_MFMA + 1); else __builtin_amdgcn_s_setprio(KITTY_PRIO_MFMA);
           pv_packed(S, x, A.out, A.lz, VLds{S.vbuf}, C);
         }
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
         if (k1) dma_v(x, i + 1, lv);
       }
+      };
+      if (young) loop(std::true_type{}); else loop(std::false_type{});
       wait_vmcnt<0>();
     }
   } else {
