@@ -114,3 +114,31 @@ def test_stock_llama_long_prompt_decode_and_chunk():
     # dense attention's (random weights leave the argmax itself nearly tied, so it is not compared)
     print("cosine similarity of the logits: min %.4f mean %.4f" % (min(cos), sum(cos) / len(cos)))
     assert min(cos) >= 0.97, min(cos)
+
+
+@pytest.mark.gpu
+def test_stock_llama_with_device_side_counters():
+    """After the prompt the cache can keep its counters on the device (one append launch, one flush
+    launch pair per layer and step): the logits are those of the host-counter mode, bit for bit."""
+    if not torch.cuda.is_available():
+        pytest.skip("needs a GPU")
+    from kitty_amd import hf
+    hf.register()
+    dev = torch.device("cuda")
+    mod = _tiny_llama("kitty").to(dev).half().eval()
+    B, T0, steps = 2, 32 + 128 + 100, 60                       # the K Q-buffer fills and is flushed on the way
+    ids = torch.randint(0, 256, (B, T0), generator=torch.Generator().manual_seed(3)).to(dev)
+    host, devc = (hf.KittyHFCache(mod.config, B, 1024, device=dev) for _ in range(2))
+    with torch.no_grad():
+        a = mod(input_ids=ids, past_key_values=host, use_cache=True).logits[:, -1]
+        b = mod(input_ids=ids, past_key_values=devc, use_cache=True).logits[:, -1]
+        assert torch.equal(a, b)
+        devc.enable_device_counters()
+        cur = a.float().argmax(-1, keepdim=True)
+        for s in range(steps):
+            a = mod(input_ids=cur, past_key_values=host, use_cache=True).logits[:, -1]
+            b = mod(input_ids=cur, past_key_values=devc, use_cache=True).logits[:, -1]
+            assert torch.equal(a, b), s
+            cur = a.float().argmax(-1, keepdim=True)
+    torch.cuda.synchronize()
+    assert devc.kv_cache[0].seq_counts.cpu().tolist() == [host.kv_cache[0].counts()] * B
