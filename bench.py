@@ -343,6 +343,10 @@ def main():
     ap.add_argument("--splits", type=int, default=0)
     ap.add_argument("--variant", type=int, default=0)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--scatter-pages", action="store_true",
+                    help="place every packed page at a random position of the page arrays (page tables to match), "
+                         "as a page pool leaves them after sequences have come and gone; default: the reference's "
+                         "identity tables")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 1 GiB device copy a few times, so that a counter run of this command "
                          "holds a kernel of known traffic to scale FETCH_SIZE / WRITE_SIZE by")
@@ -403,6 +407,19 @@ def main():
         quant_ms.append(e0.elapsed_time(e1))
         if i < copies:
             caches.append(c)
+    if args.scatter_pages:
+        gen = torch.Generator(device=dev).manual_seed(5)
+        for c in caches:
+            L = c.kv_cache[0]
+            for codes, meta, table in ((L.KeyCache, L.KeyCache_metadata, L.PageTable_K),
+                                       (L.ValueCache, L.ValueCache_metadata, L.PageTable_V)):
+                perm = torch.randperm(codes.shape[0], generator=gen, device=dev)
+                for t in (codes, meta):
+                    moved = torch.empty_like(t)
+                    moved[perm] = t
+                    t.copy_(moved)
+                table.copy_(perm[table])
+        del moved
     L0 = probe.kv_cache[0]
     quant_in_bytes = 2 * B * H_KV * (L0.PageCount_K + L0.PageCount_V) * 128 * D
     quant_gbps = quant_in_bytes / (min(quant_ms) * 1e-3) / 1e9
@@ -478,7 +495,8 @@ def main():
         "data": "synthetic (seeded N(0,1) K with 8 outlier channels/head x10, N(0,1) V, random-init)",
         "config": {"workload": desc, "batch": B, "q_heads": H_Q, "kv_heads": H_KV, "head_dim": D, "context": T,
                    "pages_k": L0.PageCount_K, "pages_v": L0.PageCount_V, "num_splits": splits,
-                   "variant": args.variant, "cache_copies_rotated": len(caches)},
+                   "variant": args.variant, "cache_copies_rotated": len(caches),
+                   "page_placement": "scattered" if args.scatter_pages else "identity"},
         "roofline": {
             "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBPS, "traffic": measured_traffic(args.workload, splits),

@@ -50,9 +50,13 @@ enum {
   KITTY_CNT_QBUF_V = 4,     /* Q_Buffer_Count_V      (0..PAGE_SIZE)                           */
   KITTY_CNT_LOCAL_V = 5,    /* Local_Count_V         (0..PAGE_SIZE)                           */
   KITTY_CNT_LOCAL_OFF = 6,  /* Write_Offset_Local_V  (ring head = oldest row)                 */
-  KITTY_CNT_RESERVED = 7,
+  KITTY_CNT_FLAGS = 7,      /* KITTY_SEQ_* bits                                               */
   KITTY_SEQ_COUNT_FIELDS = 8
 };
+/* Flag bits of a sequence's counter row.  INACTIVE: the slot holds no sequence (or a paused one):
+ * kitty_append_token and kitty_flush_full leave it alone; attention still sees what its counters
+ * describe, nothing when they are zero. */
+enum { KITTY_SEQ_INACTIVE = 1 };
 
 typedef struct kitty_kv_layer {
   int32_t H_KV, D, D_BOOSTED, PAGE_SIZE, S, MAX_PAGE;
@@ -180,7 +184,8 @@ int kitty_prefill_attn(const kitty_kv_layer* layer,
  * kitty_flush_full: every sequence whose K (V) Q-buffer holds PAGE_SIZE rows gets it quantized,
  * with channel selection, into page page_table[b][PageCount] and its counters advanced; the
  * arithmetic is that of kitty_quant_pack_k / _v.  A sequence already at MAX_PAGE pages, or whose
- * page id is outside [0, cache_pages), is left as it is.
+ * page id is outside [0, cache_pages) (a page table entry of -1: no page assigned), is left as it
+ * is, Q-buffer full, and drops the tokens appended until a later call finds a page there.
  */
 int kitty_append_token(const kitty_kv_layer* layer, const void* k_new, const void* v_new,
                        int64_t stride_b, int64_t stride_h, int B, void* stream);

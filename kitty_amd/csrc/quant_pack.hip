@@ -360,6 +360,7 @@ __global__ __launch_bounds__(256) void append_token_kernel(kitty_kv_layer L, con
                                                            int64_t stride_h) {
   const int b = blockIdx.x;
   int32_t* cnt = const_cast<int32_t*>(L.seq_counts) + b * KITTY_SEQ_COUNT_FIELDS;
+  if (cnt[KITTY_CNT_FLAGS] & KITTY_SEQ_INACTIVE) return;   // the whole block: nobody reaches the barrier
   const int sink = cnt[KITTY_CNT_SINK], rk = cnt[KITTY_CNT_QBUF_K], rv = cnt[KITTY_CNT_QBUF_V];
   const int lv = cnt[KITTY_CNT_LOCAL_V], off = cnt[KITTY_CNT_LOCAL_OFF] & (kPage - 1);
   const bool to_sink = sink < L.S;
@@ -408,6 +409,7 @@ __global__ __launch_bounds__(256) void flush_full_kernel(kitty_kv_layer L, int64
   const int h = blockIdx.x, b = blockIdx.y;
   const int32_t* cnt = L.seq_counts + b * KITTY_SEQ_COUNT_FIELDS;
   const int64_t w = (int64_t)b * L.win_stride_b + (int64_t)h * L.win_stride_h;
+  if (cnt[KITTY_CNT_FLAGS] & KITTY_SEQ_INACTIVE) return;
   if (blockIdx.z == 0) {
     const int pk = cnt[KITTY_CNT_PAGES_K];
     if (cnt[KITTY_CNT_QBUF_K] != kPage || pk < 0 || pk >= L.MAX_PAGE) return;
@@ -427,18 +429,27 @@ __global__ __launch_bounds__(256) void flush_full_kernel(kitty_kv_layer L, int64
   }
 }
 
-// after flush_full_kernel: the flushed Q-buffers are empty, their pages count
-__global__ void advance_counts_kernel(kitty_kv_layer L, int B) {
+// after flush_full_kernel: the flushed Q-buffers are empty, their pages count.  The conditions are
+// those under which flush_full_kernel wrote the page.
+__global__ void advance_counts_kernel(kitty_kv_layer L, int B, int64_t cache_pages) {
   const int b = blockIdx.x * blockDim.x + threadIdx.x;
   if (b >= B) return;
   int32_t* cnt = const_cast<int32_t*>(L.seq_counts) + b * KITTY_SEQ_COUNT_FIELDS;
-  if (cnt[KITTY_CNT_QBUF_K] == kPage && cnt[KITTY_CNT_PAGES_K] >= 0 && cnt[KITTY_CNT_PAGES_K] < L.MAX_PAGE) {
-    cnt[KITTY_CNT_PAGES_K] += 1;
-    cnt[KITTY_CNT_QBUF_K] = 0;
+  if (cnt[KITTY_CNT_FLAGS] & KITTY_SEQ_INACTIVE) return;
+  const int pk = cnt[KITTY_CNT_PAGES_K], pv = cnt[KITTY_CNT_PAGES_V];
+  if (cnt[KITTY_CNT_QBUF_K] == kPage && pk >= 0 && pk < L.MAX_PAGE) {
+    const int64_t pg = L.page_table_k[(int64_t)b * L.page_table_k_stride_b + pk];
+    if (pg >= 0 && pg < cache_pages) {
+      cnt[KITTY_CNT_PAGES_K] = pk + 1;
+      cnt[KITTY_CNT_QBUF_K] = 0;
+    }
   }
-  if (cnt[KITTY_CNT_QBUF_V] == kPage && cnt[KITTY_CNT_PAGES_V] >= 0 && cnt[KITTY_CNT_PAGES_V] < L.MAX_PAGE) {
-    cnt[KITTY_CNT_PAGES_V] += 1;
-    cnt[KITTY_CNT_QBUF_V] = 0;
+  if (cnt[KITTY_CNT_QBUF_V] == kPage && pv >= 0 && pv < L.MAX_PAGE) {
+    const int64_t pg = L.page_table_v[(int64_t)b * L.page_table_v_stride_b + pv];
+    if (pg >= 0 && pg < cache_pages) {
+      cnt[KITTY_CNT_PAGES_V] = pv + 1;
+      cnt[KITTY_CNT_QBUF_V] = 0;
+    }
   }
 }
 
@@ -580,6 +591,7 @@ extern "C" int kitty_flush_full(const kitty_kv_layer* layer, int B, int64_t cach
   if (int rc = check_append_layer(layer, B)) return rc;
   KITTY_REQUIRE(cache_pages >= 0, KITTY_E_RANGE, "bad cache_pages");
   hipLaunchKernelGGL(flush_full_kernel, dim3(layer->H_KV, B, 2), dim3(256), 0, (hipStream_t)stream, *layer, cache_pages);
-  hipLaunchKernelGGL(advance_counts_kernel, dim3((B + 63) / 64), dim3(64), 0, (hipStream_t)stream, *layer, B);
+  hipLaunchKernelGGL(advance_counts_kernel, dim3((B + 63) / 64), dim3(64), 0, (hipStream_t)stream, *layer, B,
+                     cache_pages);
   return check_launch("kitty_flush_full");
 }

@@ -19,13 +19,27 @@ from .kernels.kitty_quant_pack import quantize_pack_k, quantize_pack_v
 from .utils_kv_per_layer import KVCache_Layer
 
 
+def prefill_split(len_prefill: int, S: int, P: int) -> dict:
+    """Where the tokens of a prefill go (kitty.py:126-192): the first ``sink`` stay fp16 for good;
+    of the keys, the newest ``(T - S) % P`` wait in the Q-buffer and whole pages in between are
+    packed; of the values, the newest ``min(P, T - S)`` fill the local ring, the ``% P`` remainder
+    before them waits in the Q-buffer, the rest is packed."""
+    sink = min(S, len_prefill)
+    qbuf_k = max(0, len_prefill - sink) % P
+    pages_k = (len_prefill - sink - qbuf_k) // P
+    local_v = max(0, min(P, len_prefill - sink))
+    qbuf_v = max(0, len_prefill - sink - local_v) % P
+    pages_v = (len_prefill - sink - local_v - qbuf_v) // P
+    return dict(sink=sink, qbuf_k=qbuf_k, pages_k=pages_k, local_v=local_v, qbuf_v=qbuf_v, pages_v=pages_v)
+
+
 class KittyCache(_HFCache):
     """Kitty KV cache: fp16 sink + packed 2-bit pages (25 % of key channels at 4 bit) + fp16
     residual windows that are flushed into packed pages when full."""
     is_compileable = False
 
     def __init__(self, config, max_batch_size: int, max_length: int, *, device="cuda",
-                 select: str = "hip") -> None:
+                 select: str = "hip", layer_kwargs: Optional[dict] = None) -> None:
         if _HFCache is not object:
             try:
                 super().__init__(layers=[])          # transformers >= 4.54
@@ -46,7 +60,7 @@ class KittyCache(_HFCache):
             self.kv_cache.append(KVCache_Layer(
                 MAX_BS=max_batch_size, MAX_LEN=max_length, H_KV=self.num_key_value_heads, D=self.head_dim,
                 D_BOOSTED=self.d_boosted, LOW_BIT=self.low_bit, HIGH_BIT=self.high_bit,
-                PAGE_SIZE=self.page_size, S=self.sink_length, device=device))
+                PAGE_SIZE=self.page_size, S=self.sink_length, device=device, **(layer_kwargs or {})))
 
     def update(self, key_states: torch.Tensor, value_states: torch.Tensor, layer_idx: int,
                cache_kwargs: Optional[dict[str, Any]] = None) -> bool:
@@ -91,44 +105,46 @@ class KittyCache(_HFCache):
         kvcache = self.kv_cache[layer_idx]
         if kvcache.key_states is None or kvcache.value_states is None:
             raise ValueError("No key_states or value_states to quantize. Please call update() first.")
-        K, V = kvcache.key_states, kvcache.value_states
+        n = self._store_prefill(kvcache, kvcache.key_states, kvcache.value_states, 0)
+        kvcache.Sink_Count = n["sink"]
+        kvcache.Q_Buffer_Count_K = n["qbuf_k"]
+        kvcache.PageCount_K += n["pages_k"]
+        kvcache.Local_Count_V = n["local_v"]
+        kvcache.Q_Buffer_Count_V = n["qbuf_v"]
+        kvcache.PageCount_V += n["pages_v"]
+        kvcache.key_states = None
+        kvcache.value_states = None
+
+    def _store_prefill(self, kvcache: KVCache_Layer, K: torch.Tensor, V: torch.Tensor, first_row: int) -> dict:
+        """Write a prefill ``[B, H_KV, T, D]`` into rows ``first_row .. first_row + B`` of an empty
+        layer: sink, packed pages (through those rows of the page tables, from entry 0) and fp16
+        residuals.  Returns ``prefill_split``'s counts; the caller owns the counters."""
         B, P = K.shape[0], kvcache.PAGE_SIZE
+        rows = slice(first_row, first_row + B)
         len_prefill = K.shape[-2]
-        len_sink = min(kvcache.S, len_prefill)
-        # K: newest (T-S) % P tokens stay fp16 in the Q-buffer, whole pages in between are packed
-        len_qbuf_k = max(0, len_prefill - len_sink) % P
-        pages_k = (len_prefill - len_sink - len_qbuf_k) // P
+        n = prefill_split(len_prefill, kvcache.S, P)
+        len_sink, len_qbuf_k, pages_k = n["sink"], n["qbuf_k"], n["pages_k"]
+        len_local_v, len_qbuf_v, pages_v = n["local_v"], n["qbuf_v"], n["pages_v"]
         if pages_k > kvcache.MAX_PAGE:
             raise ValueError(f"prefill of {len_prefill} tokens exceeds max_length={kvcache.MAX_LEN}")
-        kvcache.Sink_Buffer_K[:B, :, :len_sink, :].copy_(K[:, :, :len_sink, :])
-        kvcache.Sink_Count = len_sink
+        kvcache.Sink_Buffer_K[rows, :, :len_sink, :].copy_(K[:, :, :len_sink, :])
         if len_qbuf_k > 0:
-            kvcache.Q_Buffer_K[:B, :, :len_qbuf_k, :].copy_(K[:, :, len_prefill - len_qbuf_k:, :])
-            kvcache.Q_Buffer_Count_K = len_qbuf_k
+            kvcache.Q_Buffer_K[rows, :, :len_qbuf_k, :].copy_(K[:, :, len_prefill - len_qbuf_k:, :])
         if pages_k > 0:
-            quantize_pack_k(K, len_sink, pages_k, kvcache.PageTable_K, 0, kvcache.KeyCache,
+            quantize_pack_k(K, len_sink, pages_k, kvcache.PageTable_K[rows], 0, kvcache.KeyCache,
                             kvcache.KeyCache_metadata, P, kvcache.D_BOOSTED, select=self.select)
-            kvcache.PageCount_K += pages_k
-        # V: newest min(P, T-S) tokens -> local ring, the remainder before them -> Q-buffer, rest packed
-        len_local_v = max(0, min(P, len_prefill - len_sink))
-        len_qbuf_v = max(0, len_prefill - len_sink - len_local_v) % P
-        pages_v = (len_prefill - len_sink - len_local_v - len_qbuf_v) // P
-        kvcache.Sink_Buffer_V[:B, :, :len_sink, :].copy_(V[:, :, :len_sink, :])
+        kvcache.Sink_Buffer_V[rows, :, :len_sink, :].copy_(V[:, :, :len_sink, :])
         if len_local_v > 0:
-            kvcache.Local_Buffer_V[:B, :, :len_local_v, :].copy_(V[:, :, len_prefill - len_local_v:, :])
-            kvcache.Local_Count_V = len_local_v
+            kvcache.Local_Buffer_V[rows, :, :len_local_v, :].copy_(V[:, :, len_prefill - len_local_v:, :])
         if len_qbuf_v > 0:
             assert len_local_v > 0, "Local buffer must be filled before using Q-buffer."
             lo = len_prefill - len_local_v - len_qbuf_v
-            kvcache.Q_Buffer_V[:B, :, :len_qbuf_v, :].copy_(V[:, :, lo: lo + len_qbuf_v, :])
-            kvcache.Q_Buffer_Count_V = len_qbuf_v
+            kvcache.Q_Buffer_V[rows, :, :len_qbuf_v, :].copy_(V[:, :, lo: lo + len_qbuf_v, :])
         if pages_v > 0:
             assert len_prefill - len_sink - len_local_v - len_qbuf_v == pages_v * P
-            quantize_pack_v(V, len_sink, pages_v, kvcache.PageTable_V, 0, kvcache.ValueCache,
+            quantize_pack_v(V, len_sink, pages_v, kvcache.PageTable_V[rows], 0, kvcache.ValueCache,
                             kvcache.ValueCache_metadata, P)
-            kvcache.PageCount_V += pages_v
-        kvcache.key_states = None
-        kvcache.value_states = None
+        return n
 
     def quantize_decode(self, layer_idx: int = 0) -> None:
         """Flush a full Q-buffer into the next packed page; K and V fill up independently
@@ -195,6 +211,12 @@ class KittyCache(_HFCache):
                 setattr(L, f, int(v))
 
     def _append_token_device(self, L: KVCache_Layer, key_states: torch.Tensor, value_states: torch.Tensor) -> None:
+        if L.Sink_Count >= L.S and L.Q_Buffer_Count_K >= L.PAGE_SIZE:
+            raise ValueError("Q-buffer is full: call quantize_decode() after every decode step")
+        self._launch_append(L, key_states, value_states)
+        L.step_host_counters()
+
+    def _launch_append(self, L: KVCache_Layer, key_states: torch.Tensor, value_states: torch.Tensor) -> None:
         B = key_states.shape[0]
         for name, t in (("key_states", key_states), ("value_states", value_states)):
             _lib.require_hip(t, name)
@@ -206,29 +228,29 @@ class KittyCache(_HFCache):
             key_states = key_states.contiguous()
         if value_states.stride() != key_states.stride():
             key_states, value_states = key_states.contiguous(), value_states.contiguous()
-        if L.Sink_Count >= L.S and L.Q_Buffer_Count_K >= L.PAGE_SIZE:
-            raise ValueError("Q-buffer is full: call quantize_decode() after every decode step")
         rc = _lib.lib().kitty_append_token(L.descriptor(), key_states.data_ptr(), value_states.data_ptr(),
                                            key_states.stride(0) * 2, key_states.stride(1) * 2, B,
                                            _lib.current_stream_ptr(key_states.device))
         _lib.check(rc, "KittyCache.update")
         L.active_batch = B
-        L.step_host_counters()
 
     def _flush_full_device(self, L: KVCache_Layer) -> None:
         P = L.PAGE_SIZE
         if (L.Q_Buffer_Count_K == P and L.PageCount_K >= L.MAX_PAGE) or \
                 (L.Q_Buffer_Count_V == P and L.PageCount_V >= L.MAX_PAGE):
             raise ValueError(f"cache is full (max_length={L.MAX_LEN})")
-        rc = _lib.lib().kitty_flush_full(L.descriptor(), L.active_batch, L.KeyCache.size(0),
-                                         _lib.current_stream_ptr(L.device))
-        _lib.check(rc, "KittyCache.quantize_decode")
+        self._launch_flush(L)
         if L.Q_Buffer_Count_K == P:
             L.PageCount_K += 1
             L.Q_Buffer_Count_K = 0
         if L.Q_Buffer_Count_V == P:
             L.PageCount_V += 1
             L.Q_Buffer_Count_V = 0
+
+    def _launch_flush(self, L: KVCache_Layer) -> None:
+        rc = _lib.lib().kitty_flush_full(L.descriptor(), L.active_batch, L.KeyCache.size(0),
+                                         _lib.current_stream_ptr(L.device))
+        _lib.check(rc, "KittyCache.quantize_decode")
 
     def append(self, key_states: torch.Tensor, value_states: torch.Tensor, layer_idx: int = 0) -> None:
         """Append a chunk of T >= 1 tokens ``[B, H_KV, T, D]`` to a layer in one go.

@@ -11,7 +11,10 @@ against the reference keeps working.  Differences, all additive:
   ragged batches (the reference keeps one set of host ints for the whole batch, :53-54,65,71-72,
   79-80).  When it is ``None`` the shared counters are used, exactly like the reference;
 * ``enable_device_counters()`` - from then on decode steps advance ``seq_counts`` on the device
-  (one fused append kernel, one flush launch) and the host ints only shadow the longest sequence.
+  (one fused append kernel, one flush launch) and the host ints only shadow the longest sequence;
+* ``n_pages=`` / ``page_tables=`` - a page pool smaller (or larger) than the reference's static
+  ``MAX_BS * MAX_PAGE`` pages, with page tables handed in by the owner of the pool (entries of -1:
+  no page assigned); see ``paging.PagedKittyCache``.
 """
 import math
 from typing import Optional
@@ -25,7 +28,8 @@ class KVCache_Layer:
     """KV cache of a single layer; pages are statically allocated."""
 
     def __init__(self, MAX_BS: int, MAX_LEN: int, H_KV: int, D: int, D_BOOSTED: int, LOW_BIT: int, HIGH_BIT: int,
-                 PAGE_SIZE: int, S: int, device="cuda"):
+                 PAGE_SIZE: int, S: int, device="cuda", *, n_pages: Optional[int] = None,
+                 page_tables: Optional[tuple] = None):
         assert PAGE_SIZE % 128 == 0, "PAGE_SIZE must be a multiple of 128."
         self.BITS_PER_BYTE = 8
         self.HIGH_BIT = HIGH_BIT
@@ -44,16 +48,26 @@ class KVCache_Layer:
         self.bytes_per_page_K = (H_KV * D * PAGE_SIZE * LOW_BIT // 8             # low 2-bit plane
                                  + H_KV * D_BOOSTED * PAGE_SIZE * LOW_BIT // 8   # high 2-bit plane (boosted)
                                  + H_KV * D)                                     # channel -> slot map
-        n_pages = MAX_BS * self.MAX_PAGE
+        if n_pages is None:
+            n_pages = MAX_BS * self.MAX_PAGE
+        elif n_pages < 1 or page_tables is None:
+            raise ValueError("a page pool needs n_pages >= 1 and the page tables of its owner")
         self.KeyCache = torch.zeros((n_pages, self.bytes_per_page_K), dtype=torch.uint8, device=dev)
         self.KeyCache_metadata = torch.zeros((n_pages, H_KV, D, 2), dtype=torch.half, device=dev)
         self.bytes_per_page_V = H_KV * PAGE_SIZE * D * LOW_BIT // 8
         self.ValueCache = torch.zeros((n_pages, self.bytes_per_page_V), dtype=torch.uint8, device=dev)
         self.ValueCache_metadata = torch.zeros((n_pages, H_KV, PAGE_SIZE, 2), dtype=torch.half, device=dev)
-        ident = (torch.arange(self.MAX_PAGE, dtype=torch.int64).view(1, -1)
-                 + torch.arange(MAX_BS, dtype=torch.int64).view(-1, 1) * self.MAX_PAGE)
-        self.PageTable_K = ident.to(dev)
-        self.PageTable_V = ident.clone().to(dev)
+        if page_tables is None:
+            ident = (torch.arange(self.MAX_PAGE, dtype=torch.int64).view(1, -1)
+                     + torch.arange(MAX_BS, dtype=torch.int64).view(-1, 1) * self.MAX_PAGE)
+            self.PageTable_K = ident.to(dev)
+            self.PageTable_V = ident.clone().to(dev)
+        else:
+            self.PageTable_K, self.PageTable_V = page_tables
+            for t in page_tables:
+                if t.dtype != torch.int64 or tuple(t.shape) != (MAX_BS, self.MAX_PAGE) or not t.is_contiguous() \
+                        or t.device.type != dev.type:
+                    raise ValueError(f"page tables must be contiguous int64 [{MAX_BS}, {self.MAX_PAGE}] on {dev}")
         self.PageCount_K = 0
         self.PageCount_V = 0
         # fp16 windows
