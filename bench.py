@@ -10,6 +10,7 @@ Infinity Cache.  Prints ONE JSON line.
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c1|c0|c2|c4] [--copies N]
 
 ``--workload e2e`` times a whole 32-layer decoder step around the cache (tokens/s).
+``--workload fq`` times the accuracy simulator's fake-quantization kernel on the configs[1] shape.
 ``--workload c3`` measures the other kernel family instead (BASELINE.json configs[3]): a 2048-token
 chunk attending a 30720-token packed prefix, bound by the matrix cores, plus the append of the chunk.
 """
@@ -188,6 +189,75 @@ def bench_chunked_prefill(args):
     print(json.dumps(result))
 
 
+def bench_fake_quant(args):
+    """The accuracy simulator's kernel: a step = fake quantization of one layer's dense fp16 K and V
+    of the configs[1] shape as the simulator's prefill does it (keys in 128-token groups per
+    channel with 25 promoted channels per block, values per token), in place."""
+    import torch
+    from kitty_amd import _lib, sim
+    _lib.lib()
+    dev = torch.device("cuda:0")
+    B, H_Q, H_KV, T, desc = WORKLOADS["c1"]
+    D, sink = 128, 32
+    n = (T - sink) // 128 * 128
+    K, V = synth_kv(B, H_KV, T, D, 1001, dev)
+    blocks = K[:, :, sink:sink + n].unflatten(2, (-1, 128)).transpose(-1, -2)
+    mask = sim.build_promote_mask(blocks, 0.2, 1)
+    src = [(K.clone(), V.clone()) for _ in range(2)]       # 4 x 1 GiB: nothing stays in the Infinity Cache
+    steps, warmup = min(args.steps, 200), min(args.warmup, 20)
+
+    def step(i, ev=None):
+        k, v = src[i % 2]
+        if ev is not None:
+            ev[0].record()
+        sim.fake_quant_tokens_(k, sink, n, 0, 128, 2, mask, 4)
+        if ev is not None:
+            ev[1].record()
+        sim.fake_quant_tokens_(v, sink, n, 1, 128, 2)
+        if ev is not None:
+            ev[2].record()
+
+    for i in range(warmup):
+        step(i)
+    torch.cuda.synchronize()
+    evs = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(steps)]
+    t0 = time.perf_counter()
+    for i in range(steps):
+        step(i, evs[i])
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) / steps * 1e3
+    k_us = sum(e[0].elapsed_time(e[1]) for e in evs) / steps * 1e3
+    v_us = sum(e[1].elapsed_time(e[2]) for e in evs) / steps * 1e3
+    nbytes = 2 * B * H_KV * n * D * 2                        # read + write, per tensor
+    result = {
+        "metric": "fake_quant_ms_per_step", "value": ms_per_step, "unit": "ms/step", "n_gpus": 1, "steps": steps,
+        "warmup": warmup, "ms_per_step": ms_per_step, "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f16 (every operator of the reference's chain rounded to f16)", "data": "synthetic (as configs[1])",
+        "config": {"workload": "accuracy simulator: fake quantization of one layer's dense K and V, " + desc,
+                   "kbits": 2, "vbits": 2, "promote_bit": 4, "promote_ratio": 0.2, "group_size": 128},
+        "roofline": {"bound": "hbm", "achieved": nbytes / (k_us * 1e-6) / 1e9, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": nbytes / (k_us * 1e-6) / 1e9 / HBM_PEAK_GBPS, "traffic": None,
+                     "kernel": "fake_quant_kernel<0> (keys)", "kernel_avg_us": k_us,
+                     "algorithmic_bytes_per_launch": nbytes,
+                     "values_kernel": {"kernel": "fake_quant_kernel<1>", "kernel_avg_us": v_us,
+                                       "achieved": nbytes / (v_us * 1e-6) / 1e9,
+                                       "frac": nbytes / (v_us * 1e-6) / 1e9 / HBM_PEAK_GBPS}},
+    }
+    if not args.no_cpu_baseline:
+        from oracle import sim_baseline as SB
+        threads = min(os.cpu_count() or 1, 16)
+        torch.set_num_threads(threads)
+        kc, vc = K[:1].cpu(), V[:1].cpu()
+        SB.simulate_prefill(kc[:, :, :sink + 1024].clone(), vc[:, :, :sink + 1024].clone(), promote_ratio=0.2)   # warm-up
+        t1 = time.perf_counter()
+        SB.simulate_prefill(kc, vc, promote_ratio=0.2)
+        dt = time.perf_counter() - t1
+        result["cpu_baseline"] = {"value": dt * B * 1e3, "unit": "ms/step", "cores": threads, "kind": "port",
+                                  "sample": f"the reference's torch operators (fp16 CPU tensors) on 1 of {B} sequences "
+                                            f"of the workload ({dt:.2f} s), scaled x{B}"}
+    print(json.dumps(result))
+
+
 def bench_end_to_end(args):
     """The side number of configs[4]: decode tokens/s of a full 32-layer Llama-3.1-8B-shaped model
     with random weights, every layer's KV in the packed cache.  The dense parts (projections, MLP,
@@ -333,7 +403,7 @@ def main():
     # the defaults are long enough for the clocks to settle: the first ~100 launches after idle run 5-8 % slower
     ap.add_argument("--steps", type=int, default=2000)
     ap.add_argument("--warmup", type=int, default=500)
-    ap.add_argument("--workload", default="c1", choices=sorted(WORKLOADS) + ["c3", "e2e"])
+    ap.add_argument("--workload", default="c1", choices=sorted(WORKLOADS) + ["c3", "e2e", "fq"])
     ap.add_argument("--e2e-batch", type=int, default=16)
     ap.add_argument("--e2e-context", type=int, default=32768)
     ap.add_argument("--e2e-mode", default="host", choices=["host", "device", "graph"],
@@ -360,6 +430,8 @@ def main():
         return bench_chunked_prefill(args)
     if args.workload == "e2e":
         return bench_end_to_end(args)
+    if args.workload == "fq":
+        return bench_fake_quant(args)
     import torch
     import kitty_amd
     from kitty_amd import _lib

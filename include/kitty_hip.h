@@ -191,6 +191,25 @@ int kitty_append_token(const kitty_kv_layer* layer, const void* k_new, const voi
                        int64_t stride_b, int64_t stride_h, int B, void* stream);
 int kitty_flush_full(const kitty_kv_layer* layer, int B, int64_t cache_pages, void* stream);
 
+/*
+ * Fake quantization of dense fp16 keys or values in place: replaces fake_quant_groupwise_lastdim of
+ * the reference's accuracy simulator (src/kitty_sim/utils_quant.py:64-114) on the slices its cache
+ * hands it (src/kitty_sim/kitty_simulate.py:196-252).  Arithmetic as that function evaluates on a GPU
+ * for fp16 tensors: every operator rounds its result to fp16, the range is floored at 1e-4, the code
+ * is clamped to [0, 2^bit - 1] and then rounded half to even.
+ * data: fp16 [B,H,T,D], D contiguous, byte strides; tokens [t_offset, t_offset + n_tokens) are
+ * rewritten.  axis 0: groups of group_size consecutive tokens per channel (keys; n_tokens must be a
+ * multiple of group_size; groups are counted from t_offset); promote_mask (optional, uint8 / bool,
+ * nonzero = promote_bit instead of bit) is indexed [b][h][tile][channel] through its byte strides,
+ * tile = 128-token block from t_offset (mask_stride_tile 0: one mask for all tokens, as the reference's
+ * [B,nh,D] mask).  axis 1: groups of group_size consecutive channels per token (values), no mask.
+ * group_size 32, 64 or 128; bit widths 1..8.
+ */
+int kitty_fake_quant(void* data, int64_t stride_b, int64_t stride_h, int64_t stride_t, int B, int H, int T, int D,
+                     int t_offset, int n_tokens, int axis, int group_size, int bit,
+                     const uint8_t* promote_mask, int64_t mask_stride_b, int64_t mask_stride_h,
+                     int64_t mask_stride_tile, int promote_bit, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -58,6 +58,8 @@ _SIGNATURES = {
                                    c_int64, c_int64, c_int64, c_int, c_int, c_int, c_float, c_void_p, c_void_p]),
     "kitty_append_token": (c_int, [POINTER(KittyKVLayer), c_void_p, c_void_p, c_int64, c_int64, c_int, c_void_p]),
     "kitty_flush_full": (c_int, [POINTER(KittyKVLayer), c_int, c_int64, c_void_p]),
+    "kitty_fake_quant": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_int, c_int, c_int, c_int, c_int, c_int,
+                                 c_int, c_int, c_int, c_void_p, c_int64, c_int64, c_int64, c_int, c_void_p]),
 }
 
 EXPORTS = tuple(_SIGNATURES)
