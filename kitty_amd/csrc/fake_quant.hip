@@ -9,11 +9,14 @@
 //   q        = rint(clamp(fp16(fp16(x - mn) / scale), 0, qmax))     (:112: clamp first, then round half to even)
 //   result   = fp16(fp16(q * scale) + mn)                           (:113)
 //
-// A tile is 128 tokens x 128 channels of one (batch row, head): 256 threads, each owning 8 channels
-// (16 bytes) of the 8 tokens r*16 + tg, so that a wave's load covers four consecutive token rows.
+// A tile is 128 tokens x 128 channels of one (batch row, head), 256 threads.
 // AXIS 0: groups run along the tokens (keys: one channel over group_size tokens; the reference
 // transposes K to [B, nh, D, T] for this, kitty_simulate.py:204-207), optional promote mask per
-// channel.  AXIS 1: groups run along the channels (values: one token over group_size channels).
+// channel.  A thread owns two channels (4 bytes) of 32 consecutive tokens, a wave one quarter of the
+// tile's tokens: a wave's load is one whole token row, the minimum and maximum of a 32-token group
+// never leave the thread, and larger groups combine two or four waves through 4 KB of LDS.
+// AXIS 1: groups run along the channels (values: one token over group_size channels).  A thread owns
+// 8 channels (16 bytes) of the 8 tokens r*16 + tg, a token row is 16 lanes, groups combine by shuffles.
 #include "kitty_common.h"
 
 namespace kitty {
@@ -21,17 +24,27 @@ namespace {
 
 __device__ __forceinline__ float hr(float v) { return __half2float(__float2half_rn(v)); }
 
-struct GroupParams { float mn, scale, qmax; };
+struct GroupParams { float mn, scale, rscale, qmax; };
 
 __device__ __forceinline__ GroupParams group_params(float mn, float mx, float qmax, float inv_qmax) {
   float rng = hr(mx - mn);
   rng = hr(fmaxf(rng, 1e-4f));
-  return GroupParams{mn, hr(rng * inv_qmax), qmax};
+  const float scale = hr(rng * inv_qmax);
+  return GroupParams{mn, scale, __frcp_rn(scale), qmax};
 }
 
+// The quotient (x - mn) / scale is needed rounded to fp32 and then to fp16.  d * (1 / scale) is
+// within 3 ulp of the fp32 quotient, so both round to the same fp16 number unless the product
+// lies within 4 ulp of the midpoint of two fp16 numbers (the 13 bits fp16 drops read 0x1000 +- 4),
+// or in fp16's subnormal range, where more bits are dropped: a wave with such a lane (one in
+// twenty) divides.
 __device__ __forceinline__ float fake_quant_one(float x, const GroupParams& g) {
-  float q = hr(__fdiv_rn(hr(x - g.mn), g.scale));
-  q = rintf(fminf(fmaxf(q, 0.f), g.qmax));
+  const float d = hr(x - g.mn);
+  float q = d * g.rscale;
+  const uint32_t low = __float_as_uint(q) & 0x1fffu;
+  const bool unsure = (low - 0x0ffcu <= 8u) || (q != 0.f && q < 6.2e-5f) || !(q < 65000.f);
+  if (__builtin_expect(__any(unsure), 0)) q = __fdiv_rn(d, g.scale);
+  q = rintf(fminf(fmaxf(hr(q), 0.f), g.qmax));
   return hr(hr(q * g.scale) + g.mn);
 }
 
@@ -53,27 +66,26 @@ __device__ __forceinline__ uint4 pack8(const float (&x)[8]) {
   return raw;
 }
 
-template <int AXIS>
+template <int AXIS, int GS>
 __global__ __launch_bounds__(256) void fake_quant_kernel(uint8_t* __restrict__ data, int64_t stride_b, int64_t stride_h,
-                                                         int64_t stride_t, int t_offset, int n_tokens, int group_size,
-                                                         float qmax, float inv_qmax, float qmax_promote,
-                                                         float inv_qmax_promote, const uint8_t* __restrict__ mask,
-                                                         int64_t mask_stride_b, int64_t mask_stride_h,
-                                                         int64_t mask_stride_tile) {
+                                                         int64_t stride_t, int t_offset, int n_tokens, float qmax,
+                                                         float inv_qmax, float qmax_promote, float inv_qmax_promote,
+                                                         const uint8_t* __restrict__ mask, int64_t mask_stride_b,
+                                                         int64_t mask_stride_h, int64_t mask_stride_tile) {
   const int tile = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
-  const int cg = threadIdx.x & 15, tg = threadIdx.x >> 4;
   const int n_here = min(kPage, n_tokens - tile * kPage);
-  uint8_t* base = data + (int64_t)b * stride_b + (int64_t)h * stride_h +
-                  (int64_t)(t_offset + tile * kPage) * stride_t + cg * 16;
-  uint4 raw[8];
-#pragma unroll
-  for (int r = 0; r < 8; ++r) {
-    const int tok = r * 16 + tg;
-    raw[r] = tok < n_here ? *(const uint4*)(base + (int64_t)tok * stride_t) : uint4{0, 0, 0, 0};
-  }
+  uint8_t* tile_base = data + (int64_t)b * stride_b + (int64_t)h * stride_h + (int64_t)(t_offset + tile * kPage) * stride_t;
 
   if constexpr (AXIS == 1) {
-    // one token row = 16 lanes; a group = group_size / 8 neighbouring lanes
+    const int cg = threadIdx.x & 15, tg = threadIdx.x >> 4;
+    uint8_t* base = tile_base + cg * 16;
+    uint4 raw[8];
+#pragma unroll
+    for (int r = 0; r < 8; ++r) {
+      const int tok = r * 16 + tg;
+      raw[r] = tok < n_here ? *(const uint4*)(base + (int64_t)tok * stride_t) : uint4{0, 0, 0, 0};
+    }
+    // one token row = 16 lanes; a group = GS / 8 neighbouring lanes
 #pragma unroll
     for (int r = 0; r < 8; ++r) {
       float x[8];
@@ -81,7 +93,8 @@ __global__ __launch_bounds__(256) void fake_quant_kernel(uint8_t* __restrict__ d
       float mn = x[0], mx = x[0];
 #pragma unroll
       for (int j = 1; j < 8; ++j) { mn = fminf(mn, x[j]); mx = fmaxf(mx, x[j]); }
-      for (int o = 1; o * 8 < group_size; o <<= 1) {
+#pragma unroll
+      for (int o = 1; o * 8 < GS; o <<= 1) {
         mn = fminf(mn, __shfl_xor(mn, o));
         mx = fmaxf(mx, __shfl_xor(mx, o));
       }
@@ -92,63 +105,50 @@ __global__ __launch_bounds__(256) void fake_quant_kernel(uint8_t* __restrict__ d
       if (tok < n_here) *(uint4*)(base + (int64_t)tok * stride_t) = pack8(x);
     }
   } else {
-    // a group = group_size consecutive tokens of one channel = rows r in [g * rpg, (g + 1) * rpg) of all 16 tg
-    __shared__ float s_mn[4][4][kD], s_mx[4][4][kD];     // [group][wave][channel]
-    const int rpg = group_size / 16, n_groups = kPage / group_size;
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    for (int g = 0; g < n_groups; ++g) {
-      float mn[8], mx[8];
+    // channels 2cp, 2cp+1; tokens 32wq .. 32wq+31 (wq = the wave's number, uniform)
+    const int cp = threadIdx.x & 63, wq = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const bool live = wq * 32 < n_here;                            // n_tokens is a multiple of GS >= 32
+    uint8_t* base = tile_base + (int64_t)(wq * 32) * stride_t;
+    const uint32_t lane_off = cp * 4;
+    uint32_t raw[32];
 #pragma unroll
-      for (int j = 0; j < 8; ++j) { mn[j] = INFINITY; mx[j] = -INFINITY; }
+    for (int i = 0; i < 32; ++i) raw[i] = live ? *(const uint32_t*)(base + (int64_t)i * stride_t + lane_off) : 0u;
+    float mn0 = INFINITY, mx0 = -INFINITY, mn1 = INFINITY, mx1 = -INFINITY;
+    if (live) {
 #pragma unroll
-      for (int r = 0; r < 8; ++r) {
-        if (r / rpg != g || r * 16 + tg >= n_here) continue;
-        float x[8];
-        unpack8(raw[r], x);
-#pragma unroll
-        for (int j = 0; j < 8; ++j) { mn[j] = fminf(mn[j], x[j]); mx[j] = fmaxf(mx[j], x[j]); }
-      }
-#pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        mn[j] = fminf(mn[j], __shfl_xor(mn[j], 16));
-        mx[j] = fmaxf(mx[j], __shfl_xor(mx[j], 16));
-        mn[j] = fminf(mn[j], __shfl_xor(mn[j], 32));
-        mx[j] = fmaxf(mx[j], __shfl_xor(mx[j], 32));
-      }
-      if (lane < 16) {
-#pragma unroll
-        for (int j = 0; j < 8; ++j) { s_mn[g][wave][cg * 8 + j] = mn[j]; s_mx[g][wave][cg * 8 + j] = mx[j]; }
+      for (int i = 0; i < 32; ++i) {
+        const float2 f = __half22float2(*(const __half2*)&raw[i]);
+        mn0 = fminf(mn0, f.x); mx0 = fmaxf(mx0, f.x);
+        mn1 = fminf(mn1, f.y); mx1 = fmaxf(mx1, f.y);
       }
     }
-    __syncthreads();
-    uint8_t promoted[8];
+    if constexpr (GS > 32) {
+      __shared__ float4 s_mm[4][64];
+      s_mm[wq][cp] = float4{mn0, mx0, mn1, mx1};
+      __syncthreads();
+      constexpr int wpg = GS / 32;                                 // waves per group
+      const int w0 = wq / wpg * wpg;
 #pragma unroll
-    for (int j = 0; j < 8; ++j) promoted[j] = 0;
-    if (mask) {
-      const uint2 m = *(const uint2*)(mask + (int64_t)b * mask_stride_b + (int64_t)h * mask_stride_h +
-                                      (int64_t)tile * mask_stride_tile + cg * 8);
-#pragma unroll
-      for (int j = 0; j < 8; ++j) promoted[j] = ((j < 4 ? m.x >> (8 * j) : m.y >> (8 * (j - 4))) & 0xff) != 0;
+      for (int w = 0; w < wpg; ++w) {
+        const float4 o = s_mm[w0 + w][cp];
+        mn0 = fminf(mn0, o.x); mx0 = fmaxf(mx0, o.y);
+        mn1 = fminf(mn1, o.z); mx1 = fmaxf(mx1, o.w);
+      }
     }
-    for (int g = 0; g < n_groups; ++g) {
-      if (g * group_size >= n_here) break;      // n_tokens is a multiple of group_size: a group is whole or absent
-      GroupParams gp[8];
+    if (!live) return;
+    uint32_t promoted = 0;
+    if (mask)
+      promoted = *(const uint16_t*)(mask + (int64_t)b * mask_stride_b + (int64_t)h * mask_stride_h +
+                                    (int64_t)tile * mask_stride_tile + cp * 2);
+    const GroupParams g0 = (promoted & 0xffu) ? group_params(mn0, mx0, qmax_promote, inv_qmax_promote)
+                                              : group_params(mn0, mx0, qmax, inv_qmax);
+    const GroupParams g1 = (promoted >> 8) ? group_params(mn1, mx1, qmax_promote, inv_qmax_promote)
+                                           : group_params(mn1, mx1, qmax, inv_qmax);
 #pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        const int c = cg * 8 + j;
-        const float mn = fminf(fminf(s_mn[g][0][c], s_mn[g][1][c]), fminf(s_mn[g][2][c], s_mn[g][3][c]));
-        const float mx = fmaxf(fmaxf(s_mx[g][0][c], s_mx[g][1][c]), fmaxf(s_mx[g][2][c], s_mx[g][3][c]));
-        gp[j] = promoted[j] ? group_params(mn, mx, qmax_promote, inv_qmax_promote) : group_params(mn, mx, qmax, inv_qmax);
-      }
-#pragma unroll
-      for (int r = 0; r < 8; ++r) {
-        if (r / rpg != g) continue;
-        float x[8];
-        unpack8(raw[r], x);
-#pragma unroll
-        for (int j = 0; j < 8; ++j) x[j] = fake_quant_one(x[j], gp[j]);
-        *(uint4*)(base + (int64_t)(r * 16 + tg) * stride_t) = pack8(x);
-      }
+    for (int i = 0; i < 32; ++i) {
+      const float2 f = __half22float2(*(const __half2*)&raw[i]);
+      const __half2 o = __floats2half2_rn(fake_quant_one(f.x, g0), fake_quant_one(f.y, g1));
+      *(uint32_t*)(base + (int64_t)i * stride_t + lane_off) = *(const uint32_t*)&o;
     }
   }
 }
@@ -185,13 +185,20 @@ extern "C" int kitty_fake_quant(void* data, int64_t stride_b, int64_t stride_h, 
   if (B == 0 || n_tokens == 0) return 0;
   const float qmax = (float)((1 << bit) - 1), qmax_p = (float)((1 << (promote_mask ? promote_bit : bit)) - 1);
   const dim3 grid((n_tokens + kPage - 1) / kPage, H, B), block(256);
-  if (axis == 0)
-    hipLaunchKernelGGL(fake_quant_kernel<0>, grid, block, 0, (hipStream_t)stream, (uint8_t*)data, stride_b, stride_h,
-                       stride_t, t_offset, n_tokens, group_size, qmax, 1.0f / qmax, qmax_p, 1.0f / qmax_p, promote_mask,
-                       mask_stride_b, mask_stride_h, mask_stride_tile);
-  else
-    hipLaunchKernelGGL(fake_quant_kernel<1>, grid, block, 0, (hipStream_t)stream, (uint8_t*)data, stride_b, stride_h,
-                       stride_t, t_offset, n_tokens, group_size, qmax, 1.0f / qmax, qmax_p, 1.0f / qmax_p, nullptr, 0, 0,
-                       0);
+  const uint8_t* m = axis == 0 ? promote_mask : nullptr;
+#define KITTY_FQ_LAUNCH(AXIS, GS)                                                                                      \
+  hipLaunchKernelGGL((fake_quant_kernel<AXIS, GS>), grid, block, 0, (hipStream_t)stream, (uint8_t*)data, stride_b,     \
+                     stride_h, stride_t, t_offset, n_tokens, qmax, 1.0f / qmax, qmax_p, 1.0f / qmax_p, m,              \
+                     mask_stride_b, mask_stride_h, mask_stride_tile)
+  if (axis == 0) {
+    if (group_size == 32) KITTY_FQ_LAUNCH(0, 32);
+    else if (group_size == 64) KITTY_FQ_LAUNCH(0, 64);
+    else KITTY_FQ_LAUNCH(0, 128);
+  } else {
+    if (group_size == 32) KITTY_FQ_LAUNCH(1, 32);
+    else if (group_size == 64) KITTY_FQ_LAUNCH(1, 64);
+    else KITTY_FQ_LAUNCH(1, 128);
+  }
+#undef KITTY_FQ_LAUNCH
   return check_launch("kitty_fake_quant");
 }
