@@ -24,6 +24,11 @@ from typing import Any, Optional
 
 import torch
 
+try:  # usable as past_key_values of a stock transformers model when transformers is importable
+    from transformers.cache_utils import Cache as _HFCache
+except Exception:  # pragma: no cover - transformers is optional for the kernels themselves
+    _HFCache = object
+
 from . import _lib
 
 __all__ = ["build_promote_mask", "fake_quant_groupwise_lastdim", "fake_quant_tokens_", "KittyKVCacheConfig",
@@ -145,12 +150,20 @@ class KittyKVCacheConfig:
             raise ValueError(f"promote_bit must be in [kbits, 8], got {self.promote_bit}")
 
 
-class KittyKVCache:
+class KittyKVCache(_HFCache):
     """The simulator's cache: ``update(key_states, value_states, layer_idx)`` appends and returns
     the keys and values the attention of this step sees ([B, nh, T, D] views of the layer's
-    buffers, valid until the layer's next ``update``)."""
+    buffers, valid until the layer's next ``update``).  A ``transformers`` cache like the
+    reference's (a ``DynamicCache`` subclass there): stock models with any dense attention
+    implementation take it as ``past_key_values``."""
+    is_compileable = False
 
     def __init__(self, cache_config: KittyKVCacheConfig, max_length: int):
+        if _HFCache is not object:
+            try:
+                super().__init__(layers=[])          # transformers >= 4.54
+            except TypeError:
+                super().__init__()
         self.cfg = cache_config
         self.max_length = max_length
         self.key_cache: list[torch.Tensor] = []
@@ -160,6 +173,11 @@ class KittyKVCache:
 
     def get_seq_length(self, layer_idx: int = 0) -> int:
         return self._len[layer_idx] if layer_idx < len(self._len) else 0
+
+    def get_mask_sizes(self, query_length, layer_idx: int = 0):
+        """(kv_length, kv_offset) of the mask a stock model prepares for ``query_length`` new tokens."""
+        n = query_length if isinstance(query_length, int) else int(query_length.shape[0])
+        return self.get_seq_length(layer_idx) + n, 0
 
     # -- the three quantization steps of the reference, on [lo, hi) of a layer's buffers ----------
     def _quant_k(self, layer: int, lo: int, hi: int) -> None:

@@ -151,3 +151,81 @@ def test_cache_steps_like_the_oracle(S, post, bitdec, sel, group):
         S.KittyKVCacheConfig(buffer_length=64)
     with pytest.raises(ValueError):
         S.KittyKVCacheConfig(kbits=12)
+
+
+def _tiny_llama():
+    from transformers import LlamaConfig, LlamaForCausalLM
+    cfg = LlamaConfig(vocab_size=256, hidden_size=256, intermediate_size=512, num_hidden_layers=2,
+                      num_attention_heads=2, num_key_value_heads=1, head_dim=128, max_position_embeddings=4096,
+                      attn_implementation="sdpa")
+    torch.manual_seed(0)
+    return LlamaForCausalLM(cfg).cuda().half().eval()
+
+
+def test_stock_model_takes_the_simulator_cache(S):
+    """A stock transformers Llama (torch's dense attention) with the simulator's cache as
+    past_key_values, as the reference's evaluation runs it: at 16 bits the logits are those of
+    transformers' own DynamicCache; at 2 bits generate() runs and the layer buffers end up equal to
+    the oracle's, fed the keys and values the model handed to update()."""
+    pytest.importorskip("transformers")
+    from transformers import DynamicCache
+    model = _tiny_llama()
+    B, T0, steps = 2, 32 + 128 + 30, 140
+    ids = torch.randint(0, 256, (B, T0), generator=torch.Generator().manual_seed(2)).cuda()
+    plain = S.KittyKVCache(S.KittyKVCacheConfig(kbits=16, vbits=16, promote_ratio=0.0), max_length=T0 + 8)
+    ref = DynamicCache()
+    with torch.no_grad():
+        cur = ids
+        for s in range(6):
+            a = model(input_ids=cur, past_key_values=ref, use_cache=True).logits[:, -1].float()
+            b = model(input_ids=cur, past_key_values=plain, use_cache=True).logits[:, -1].float()
+            assert (a - b).abs().max().item() <= 2e-2, s
+            cur = a.argmax(-1, keepdim=True)
+    assert plain.get_seq_length() == T0 + 5
+
+    cache = S.KittyKVCache(S.KittyKVCacheConfig(promote_ratio=0.2), max_length=T0 + steps)
+    seen = [[], []]
+    inner = cache.update
+
+    def recording_update(k, v, layer_idx, cache_kwargs=None):
+        seen[layer_idx].append((k.detach().cpu().numpy().copy(), v.detach().cpu().numpy().copy()))
+        return inner(k, v, layer_idx, cache_kwargs)
+
+    cache.update = recording_update
+    # topk's order among equal scores is not pinned: the oracle takes the masks the product chose
+    # (selection itself is checked in test_promote_mask_equals_the_oracle), block by block in order
+    masks, last = [[], []], []
+    inner_mask, inner_quant_k = S.build_promote_mask, cache._quant_k
+
+    def recording_mask(*a):
+        last.append(inner_mask(*a))
+        return last[-1]
+
+    def recording_quant_k(layer, lo, hi):
+        inner_quant_k(layer, lo, hi)
+        m = last.pop().cpu().numpy()                     # [B, nh, blocks, D]
+        masks[layer].extend(m[:, :, i] for i in range(m.shape[2]))
+
+    S.build_promote_mask, cache._quant_k = recording_mask, recording_quant_k
+    try:
+        with torch.no_grad():
+            out = model.generate(ids, past_key_values=cache, max_new_tokens=steps, do_sample=False, use_cache=True,
+                                 pad_token_id=0, eos_token_id=None)
+        cache.flush_pending()
+    finally:
+        S.build_promote_mask = inner_mask
+    assert out.shape == (B, T0 + steps)
+    n = len(seen[0])
+    assert n == len(seen[1]) and cache.get_seq_length(0) == T0 + n - 1 >= T0 + steps - 1
+    for l in range(2):
+        assert len(masks[l]) == (T0 + n - 1 - 32 - 1) // 128 and all(int(m.sum()) == B * 25 for m in masks[l])
+        feed = iter(masks[l])
+        oc = SO.SimCache(promote_ratio=0.2, mask_fn=lambda ks: next(feed))
+        assert seen[l][0][0].shape[2] == T0
+        for k, v in seen[l]:
+            oc.update(k, v)
+        L = oc.K.shape[2]
+        assert np.array_equal(_bits(cache.key_cache[l][:, :, :L].contiguous()), oc.K.view(np.uint16)), l
+        assert np.array_equal(_bits(cache.value_cache[l][:, :, :L].contiguous()), oc.V.view(np.uint16)), l
+    quantized = (cache.key_cache[0][:, :, 32:32 + 128] != torch.from_numpy(seen[0][0][0][:, :, 32:32 + 128]).cuda()).any()
+    assert bool(quantized)
