@@ -31,6 +31,7 @@ from typing import Any, Optional
 import torch
 
 from .kvcache.kitty import KittyCache
+from .kvcache.paging import PagedKittyCache
 from .kvcache.kernels import kitty_attention_forward, kitty_prefill_attention
 
 NAME = "kitty"
@@ -57,6 +58,34 @@ class KittyHFCache(KittyCache):
         is ever looked at (and only for its shape), so the new tokens alone are reported."""
         n = query_length if isinstance(query_length, int) else int(query_length.shape[0])
         return n, 0
+
+
+class PagedKittyHFCache(PagedKittyCache):
+    """``PagedKittyCache`` for stock attention modules.  A prompt is admitted with a batch-1 forward
+    inside ``with cache.admitting(slot):``; decode forwards take all slots as the batch, with
+    ``position_ids=cache.position_ids()`` since the sequences differ in length (rows of free
+    slots are computed and ignored)."""
+
+    def update(self, key_states: torch.Tensor, value_states: torch.Tensor, layer_idx: int,
+               cache_kwargs: Optional[dict[str, Any]] = None):
+        if self._admit_slot is None and key_states.shape[-2] != 1:
+            raise ValueError("several new tokens per sequence: admit a prompt inside `with cache.admitting(slot):`")
+        _current.cache = self
+        _current.phase = "prefill" if super().update(key_states, value_states, layer_idx, cache_kwargs) else "decode"
+        return key_states, value_states
+
+    def get_seq_length(self, layer_idx: int = 0) -> int:
+        """What a stock model derives positions from: 0 while a prompt is being admitted (its
+        positions start at 0), else the longest active sequence."""
+        return 0 if self._admit_slot is not None else super().get_seq_length(layer_idx)
+
+    def get_mask_sizes(self, query_length, layer_idx: int = 0):
+        n = query_length if isinstance(query_length, int) else int(query_length.shape[0])
+        return n, 0
+
+    def position_ids(self) -> torch.Tensor:
+        """[slots, 1] int64 on the cache's device: the position of each slot's next token."""
+        return torch.from_numpy(self.seq_lengths().astype("int64")).view(-1, 1).to(self.seq_counts.device)
 
 
 def kitty_attention(module, query: torch.Tensor, key: torch.Tensor, value: torch.Tensor,

@@ -142,3 +142,52 @@ def test_stock_llama_with_device_side_counters():
             cur = a.float().argmax(-1, keepdim=True)
     torch.cuda.synchronize()
     assert devc.kv_cache[0].seq_counts.cpu().tolist() == [host.kv_cache[0].counts()] * B
+
+
+@pytest.mark.gpu
+def test_stock_llama_on_the_paged_cache():
+    """Two prompts of different lengths admitted into slots 0 and 2 of three, decoded together with
+    per-row positions; slot 0 is released and a third prompt admitted while slot 2 keeps decoding.
+    Every sequence's logits agree with the same model serving that sequence alone on a KittyHFCache
+    (same kernels, other split counts: 3e-2 on fp16 logits)."""
+    if not torch.cuda.is_available():
+        pytest.skip("needs a GPU")
+    from kitty_amd import hf
+    hf.register()
+    dev = torch.device("cuda")
+    mod = _tiny_llama("kitty").to(dev).half().eval()
+    g = torch.Generator().manual_seed(4)
+    prompts = {0: torch.randint(0, 256, (1, 32 + 128 + 70), generator=g).to(dev),
+               2: torch.randint(0, 256, (1, 45), generator=g).to(dev)}
+    late = torch.randint(0, 256, (1, 32 + 128 * 2 + 9), generator=g).to(dev)
+    paged = hf.PagedKittyHFCache(mod.config, 3, 1024, pool_pages=10, device=dev)
+    solo, cur = {}, torch.zeros(3, 1, dtype=torch.long, device=dev)
+
+    def admit(slot, ids):
+        solo[slot] = hf.KittyHFCache(mod.config, 1, 1024, device=dev)
+        with paged.admitting(slot):
+            a = mod(input_ids=ids, past_key_values=paged, use_cache=True).logits[:, -1].float()
+        b = mod(input_ids=ids, past_key_values=solo[slot], use_cache=True).logits[:, -1].float()
+        assert (a - b).abs().max().item() <= 3e-2
+        cur[slot] = b.argmax(-1)
+
+    def decode(steps):
+        for s in range(steps):
+            pos = paged.position_ids()
+            a = mod(input_ids=cur, position_ids=pos, past_key_values=paged, use_cache=True).logits[:, -1].float()
+            for slot in paged.active_slots():
+                b = mod(input_ids=cur[slot:slot + 1], past_key_values=solo[slot], use_cache=True).logits[:, -1].float()
+                assert int(pos[slot]) == solo[slot].get_seq_length(0) - 1
+                assert (a[slot:slot + 1] - b).abs().max().item() <= 3e-2, (s, slot)
+                cur[slot] = b.argmax(-1)
+
+    with torch.no_grad():
+        for slot, ids in prompts.items():
+            admit(slot, ids)
+        assert paged.active_slots() == [0, 2] and list(paged.seq_lengths()) == [230, 0, 45]
+        decode(70)                                   # slot 0 flushes keys, slot 2 leaves the sink behind
+        paged.release(0)
+        admit(1, late)
+        decode(40)
+    paged.check_tables()
+    assert paged.active_slots() == [1, 2] and list(paged.seq_lengths()) == [0, 297 + 40, 45 + 110]
