@@ -79,16 +79,35 @@ struct WaveLds<true, false> : Tables {
   __attribute__((aligned(16))) uint8_t vbuf[kVTile];
   __attribute__((aligned(16))) _Float16 q_nat[8][kQPad];   // [head][channel]; [..][128] = 0 ("no channel")
 };
+// Quarter variant: the B operands of QK (q * scale, both parts, for the four heads) are a table
+// built once per page (qs, see qk_packed_tab), so the per-page tables of the generic path are only
+// needed by the tail tiles, which run after the body loop: they share the space of the V tile.
+constexpr int kQsPitch = 72;   // dwords per row of qs: 64 channel pairs + 8, so that rows fall on different banks
 template <>
-struct WaveLds<true, true> : Tables {
+struct WaveLds<true, true> {
   __attribute__((aligned(16))) uint8_t kbuf[2][kKTile];
-  __attribute__((aligned(16))) uint8_t vbuf[kVTile];
-  __attribute__((aligned(16))) _Float16 q_nat[4][kQPad];
+  union {
+    __attribute__((aligned(16))) uint8_t vbuf[kVTile];
+    struct {   // tail tiles only (staged by stage_tail_tables)
+      __attribute__((aligned(16))) uint32_t ks_perm[64];
+      _Float16 ks4_nat[kQPad];
+      uint32_t vs_nat[64], ones[64];
+      uint8_t inv[32];
+      __attribute__((aligned(16))) _Float16 q_nat[4][kQPad];
+    };
+  };
+  __attribute__((aligned(16))) uint32_t kz_perm[64];
+  uint32_t vz_nat[64];
   // vs_q[t][e]: the V scale pair of token pair e if e % 4 == t, else 0 (cleared once per kernel):
   // a column that owns operand register t of every chunk multiplies by table t and so feeds
   // zeros for the tokens of the other columns
   __attribute__((aligned(16))) uint32_t vs_q[4][64];
+  __attribute__((aligned(16))) uint32_t ones4[4];      // fp16 (1, 1) pairs
+  // qs[r][l]: fp16 pair for channels 2l, 2l+1; rows 0..3 = fp16(q_head * scale) of the four heads,
+  // rows 4..7 = the exact remainders
+  __attribute__((aligned(16))) uint32_t qs[8][kQsPitch];
 };
+static_assert(sizeof(WaveLds<true, true>) <= 160 * 1024 / 8, "eight waves per CU");
 template <>
 struct WaveLds<false, false> : Tables {
   __attribute__((aligned(16))) _Float16 q_nat[16][kQPad];
@@ -197,6 +216,10 @@ struct Ctx {
   uint32_t vtr;         // LDS: same for V rows 32kg .. 32kg+3
   float sc2;            // scaling * log2(e)
   uint32_t qpair[16];   // q[col][32kc + 8pi + 2kg + {0,1}] as an fp16 pair, index 4kc + pi
+  // quarter columns (qk_packed_tab):
+  uint32_t q4[4];       // q[head r][2 lane + {0,1}] of the four heads behind the table rows
+  uint32_t qs_rd;       // byte offset of this lane's first read in the q * scale table: row, lane group
+  uint32_t qb_rd;       // the same in the table of the high-plane slots
 };
 
 // ---------------------------------------------------------------------------------------------
@@ -411,6 +434,108 @@ __device__ __forceinline__ void qk_packed(LDS& S, const Ctx& x, const KSRC& kb, 
     for (int u = 0; u < 8; ++u)
 #pragma unroll
       for (int j = 0; j < 4; ++j) C[u][j] += ror8(C[u][j]);
+  }
+  cz = Cz[0];
+}
+
+// The same for quarter columns (at most four heads), with the B operands from a table.  The generic
+// path has every lane multiply q by the scales of its own operand registers: 16 columns = 4 heads x
+// 2 parts, each computed twice, plus a gather of q and scale through the slot map for the high
+// plane.  Here lane l, which receives the (scale, zero) pairs of channels 2l and 2l + 1, computes
+// both parts for the four heads once and stores them in channel order (qs); an operand register
+// pair of a 32-channel chunk - channels 32kc + 16 (pi / 2) + 4kg + {0..3} - is then one 64-bit read,
+// and the pipeline spends no vector instruction on the B side.  The operands of the high plane are
+// scattered instead of gathered: a boosted channel's lane writes 4 * q * scale to its slot of a
+// [row][slot] table, which lies in the tile's slot-map and metadata bytes (in registers by then).
+template <bool BOOST, class LDS>
+__device__ __forceinline__ void qk_packed_tab(LDS& S, const Ctx& x, uint8_t* kt, float4v (&C)[8], float& cz) {
+  const KLds kb{kt};
+  uint32_t Xn[4];
+  kb.x4_lo(x, 0, Xn);
+  const int l = x.lane;
+  const uint2 km = kb.meta2(x);
+  const uint32_t ib = BOOST ? kb.idx(x) : 0u;
+  const uint32_t ss = __builtin_amdgcn_perm(km.y, km.x, 0x05040100u);   // (s0, s1)
+  const uint32_t zz = __builtin_amdgcn_perm(km.y, km.x, 0x07060302u);   // (z0, z1)
+  const int pos = (l >> 4) * 16 + ((l >> 1) & 3) * 4 + 2 * ((l >> 3) & 1) + (l & 1);   // see stage_k_meta
+  uint8_t* bt = kt + kKOffIdx;   // high-plane operands: 8 rows x 32 slots, fp16
+  wave_lds_fence();              // the reads above come first: LDS executes a wave's instructions in order
+  S.kz_perm[pos] = zz;
+  uint32_t hi[4], lo[4];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const half2v h = as_h2(x.q4[r]) * as_h2(ss);                                    // q*scale rounded to fp16 ...
+    hi[r] = as_u32(h);
+    lo[r] = as_u32(__builtin_elementwise_fma(as_h2(x.q4[r]), as_h2(ss), -h));       // ... and its exact remainder
+  }
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    S.qs[r][l] = hi[r];
+    S.qs[4 + r][l] = lo[r];
+  }
+  if (BOOST) {
+    *(uint2*)(bt + 8 * l) = uint2{0u, 0u};   // a slot no channel claims contributes nothing
+    wave_lds_fence();
+    const half2v four = {(_Float16)4.0f, (_Float16)4.0f};
+    const uint32_t i0 = ib & 0xffu, i1 = ib >> 8;
+    if (i0 < 32) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        *(uint16_t*)(bt + 64 * r + 2 * i0) = (uint16_t)(as_u32(as_h2(hi[r]) * four) & 0xffffu);
+        *(uint16_t*)(bt + 64 * (4 + r) + 2 * i0) = (uint16_t)(as_u32(as_h2(lo[r]) * four) & 0xffffu);
+      }
+    }
+    if (i1 < 32) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        *(uint16_t*)(bt + 64 * r + 2 * i1) = (uint16_t)(as_u32(as_h2(hi[r]) * four) >> 16);
+        *(uint16_t*)(bt + 64 * (4 + r) + 2 * i1) = (uint16_t)(as_u32(as_h2(lo[r]) * four) >> 16);
+      }
+    }
+  }
+  wave_lds_fence();
+  const uint8_t* rd = (const uint8_t*)&S.qs[0][0] + x.qs_rd;
+  uint2 b01n = *(const uint2*)rd, b23n = *(const uint2*)(rd + 32);
+  uint4v zpn = *(const uint4v*)&S.kz_perm[x.kg * 4];
+  float4v Cz = float4v{0.f, 0.f, 0.f, 0.f};   // q . zero_k: an A tile whose 16 rows all hold the zero points
+#pragma unroll
+  for (int u = 0; u < 8; ++u) C[u] = float4v{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int kc = 0; kc < 4; ++kc) {
+    uint32_t bq[4], az[4], X[4], Y[4];
+    const uint4v zp = zpn;
+    const uint32_t b[4] = {b01n.x, b01n.y, b23n.x, b23n.y};
+#pragma unroll
+    for (int pi = 0; pi < 4; ++pi) X[pi] = Xn[pi];
+    if (kc < 3) {   // one chunk ahead, as in qk_packed
+      kb.x4_lo(x, kc + 1, Xn);
+      b01n = *(const uint2*)(rd + 64 * (kc + 1));
+      b23n = *(const uint2*)(rd + 64 * (kc + 1) + 32);
+      zpn = *(const uint4v*)&S.kz_perm[(kc + 1) * 16 + x.kg * 4];
+    } else if (BOOST) {
+      kb.x4_hi(x, Xn);
+      b01n = *(const uint2*)(bt + x.qb_rd);
+      b23n = *(const uint2*)(bt + x.qb_rd + 32);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int pi = 0; pi < 4; ++pi) {
+      bq[pi] = x.qpair[kc * 4 + pi];
+      az[pi] = zp[pi];
+      Y[pi] = X[pi] >> 10;
+    }
+    Cz = mfma16(az, bq, Cz);
+    unpack_mfma1(X, Y, b, C);
+  }
+  if (BOOST) {
+    uint32_t X[4], Y[4];
+    const uint32_t b[4] = {b01n.x, b01n.y, b23n.x, b23n.y};
+#pragma unroll
+    for (int pi = 0; pi < 4; ++pi) {
+      X[pi] = Xn[pi];
+      Y[pi] = X[pi] >> 10;
+    }
+    unpack_mfma1(X, Y, b, C);
   }
   cz = Cz[0];
 }
@@ -645,7 +770,7 @@ __device__ __forceinline__ void pv_quarter(LDS& S, const Ctx& x, float4v (&out)[
   S.vz_nat[(x.lane & 48) + 4 * (x.lane & 3) + ((x.lane >> 2) & 3)] = __builtin_amdgcn_perm(vm.y, vm.x, 0x07060302u);
   wave_lds_fence();
   const uint32_t* sq = &S.vs_q[x.pi_own][16 * x.kg];
-  const uint32_t* lz_rows = (x.n & 1) ? &S.vz_nat[16 * x.kg + 4 * ((x.n >> 1) & 3)] : &S.ones[0];
+  const uint32_t* lz_rows = (x.n & 1) ? &S.vz_nat[16 * x.kg + 4 * ((x.n >> 1) & 3)] : &S.ones4[0];
   uint32_t Xn[4];
   vb.x4(x, 0, Xn);
   uint4v spn = *(const uint4v*)&sq[0];
@@ -808,20 +933,35 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(kitty_kv_layer L, co
   for (int kc = 0; kc < 4; ++kc)
 #pragma unroll
     for (int pi = 0; pi < 4; ++pi) x.qpair[kc * 4 + pi] = *(const uint32_t*)(qrow + 32 * kc + krow(pi, x.kg));
-  if (x.n < G) {   // one copy per head
-    const uint4* src = (const uint4*)(qrow + 32 * x.kg);
-    uint4* dst = (uint4*)&S.q_nat[x.g][32 * x.kg];
+  // the tables of the generic QK / PV path: q in natural order for the slot gather, a zero entry
+  // for "no channel", a row of ones
+  auto stage_generic_tables = [&]() {
+    if (x.n < G) {   // one copy per head
+      const uint4* src = (const uint4*)(qrow + 32 * x.kg);
+      uint4* dst = (uint4*)&S.q_nat[x.g][32 * x.kg];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) dst[i] = src[i];
-    if (x.kg == 0) S.q_nat[x.g][128] = (_Float16)0.0f;
-  }
-  if (x.lane == 0) S.ks4_nat[128] = (_Float16)0.0f;
-  S.ones[x.lane] = 0x3C003C00u;
+      for (int i = 0; i < 4; ++i) dst[i] = src[i];
+      if (x.kg == 0) S.q_nat[x.g][128] = (_Float16)0.0f;
+    }
+    if (x.lane == 0) S.ks4_nat[128] = (_Float16)0.0f;
+    S.ones[x.lane] = 0x3C003C00u;
+    wave_lds_fence();
+  };
   if constexpr (QUARTER) {
+    // the generic tables share the V tile's space and are staged before the tail tiles instead
 #pragma unroll
     for (int t = 0; t < 4; ++t) S.vs_q[t][x.lane] = 0u;
+    if (x.lane < 4) S.ones4[x.lane] = 0x3C003C00u;
+#pragma unroll
+    for (int r = 0; r < 4; ++r)
+      x.q4[r] = *(const uint32_t*)(q + ((int64_t)x.b * H_Q + (int64_t)x.h * G + min(r, G - 1)) * kD + 2 * x.lane);
+    const int row = x.g + (x.lo_part ? 4 : 0);
+    x.qs_rd = row * (kQsPitch * 4) + 8 * x.kg;
+    x.qb_rd = row * 64 + 8 * x.kg;
+    wave_lds_fence();
+  } else {
+    stage_generic_tables();
   }
-  wave_lds_fence();
 
   Acc A;
 #pragma unroll
@@ -898,7 +1038,8 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(kitty_kv_layer L, co
           if (k1) wait_vmcnt<nK + 2 * kDmaV>(); else wait_vmcnt<2 * kDmaV>();
         }
         if (fav) __builtin_amdgcn_s_setprio(KITTY_PRIO_MFMA + 1); else __builtin_amdgcn_s_setprio(KITTY_PRIO_MFMA);
-        qk_packed<BOOST, SPLIT_COLS, !QUARTER>(S, x, KLds{S.kbuf[buf]}, C, cz);
+        if constexpr (QUARTER) qk_packed_tab<BOOST>(S, x, S.kbuf[buf], C, cz);
+        else qk_packed<BOOST, SPLIT_COLS>(S, x, KLds{S.kbuf[buf]}, C, cz);
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
         if (k2) dma_k<BOOST>(x, i + 2, buf ? lk1 : lk0);
         if (fav) __builtin_amdgcn_s_setprio(KITTY_PRIO_VALU + 1); else __builtin_amdgcn_s_setprio(KITTY_PRIO_VALU);
@@ -941,6 +1082,7 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(kitty_kv_layer L, co
     }
   }
   if (tail) {
+    if constexpr (QUARTER) stage_generic_tables();   // the V tile is idle from here on
     to_true_units(A);
     KRegs kb;
     VRegs vb;
