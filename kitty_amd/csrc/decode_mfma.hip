@@ -478,19 +478,19 @@ __device__ __forceinline__ void qk_packed_tab(LDS& S, const Ctx& x, uint8_t* kt,
     wave_lds_fence();
     const half2v four = {(_Float16)4.0f, (_Float16)4.0f};
     const uint32_t i0 = ib & 0xffu, i1 = ib >> 8;
+    uint32_t w4[8];   // the high plane's weight: 4 * scale
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      w4[r] = as_u32(as_h2(hi[r]) * four);
+      w4[4 + r] = as_u32(as_h2(lo[r]) * four);
+    }
     if (i0 < 32) {
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        *(uint16_t*)(bt + 64 * r + 2 * i0) = (uint16_t)(as_u32(as_h2(hi[r]) * four) & 0xffffu);
-        *(uint16_t*)(bt + 64 * (4 + r) + 2 * i0) = (uint16_t)(as_u32(as_h2(lo[r]) * four) & 0xffffu);
-      }
+      for (int r = 0; r < 8; ++r) *(uint16_t*)(bt + 64 * r + 2 * i0) = (uint16_t)(w4[r] & 0xffffu);
     }
     if (i1 < 32) {
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        *(uint16_t*)(bt + 64 * r + 2 * i1) = (uint16_t)(as_u32(as_h2(hi[r]) * four) >> 16);
-        *(uint16_t*)(bt + 64 * (4 + r) + 2 * i1) = (uint16_t)(as_u32(as_h2(lo[r]) * four) >> 16);
-      }
+      for (int r = 0; r < 8; ++r) *(uint16_t*)(bt + 64 * r + 2 * i1) = (uint16_t)(w4[r] >> 16);
     }
   }
   wave_lds_fence();
