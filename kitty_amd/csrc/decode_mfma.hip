@@ -16,6 +16,9 @@
 // sum_tok p*zero_v are one more small matrix product each.
 // With 1, 2 or 4 heads per kv head every head sits in at least four columns; each of the four then
 // does the softmax and feeds PV for a quarter of a page's tokens only (see combine_quarter).
+// In that case the q * scale operands of a page are not computed by every lane for itself but once
+// per page into an LDS table, and the high plane's operands are scattered to their slots (see
+// qk_packed_tab).
 //
 // Codes as operands.  A 32-bit word of a packed plane holds 16 two-bit codes of ONE row (K: one
 // channel, 16 tokens; V: one token, 16 channels) but an MFMA register must hold two consecutive k
@@ -356,8 +359,7 @@ __device__ __forceinline__ float ror4(float v) {   // value of column n - 4 (mod
 // same B operand - column n carries the rounded part of head n % 8, column n + 8 the remainder -
 // and the two partial sums are added across the columns afterwards: one matrix instruction per
 // tile of codes instead of two, none of them waiting for the one before it.
-// COMBINE = false leaves the two partial sums of split columns apart (combine_quarter adds them).
-template <bool BOOST, bool SPLIT_COLS, bool COMBINE = true, class LDS, class KSRC>
+template <bool BOOST, bool SPLIT_COLS, class LDS, class KSRC>
 __device__ __forceinline__ void qk_packed(LDS& S, const Ctx& x, const KSRC& kb, float4v (&C)[8], float& cz) {
   // One chunk of 32 plane rows ahead: the LDS reads of chunk kc + 1 are issued before the vector
   // and matrix work of chunk kc, so that their latency is covered by this wave's own work.
@@ -429,7 +431,7 @@ __device__ __forceinline__ void qk_packed(LDS& S, const Ctx& x, const KSRC& kb, 
     if (SPLIT_COLS) unpack_mfma1(X, Y, bh, C);
     else unpack_mfma2(X, Y, bh, bl, C);
   }
-  if (SPLIT_COLS && COMBINE) {
+  if (SPLIT_COLS) {
 #pragma unroll
     for (int u = 0; u < 8; ++u)
 #pragma unroll
