@@ -14,7 +14,7 @@
 // most 8 heads col n -> head (n % 8) % G, and columns 8..15 carry the low-order part of the QK
 // operand, see qk_packed).  The zero points never touch the codes: sum_ch q*zero_k and
 // sum_tok p*zero_v are one more small matrix product each.
-// With 1, 2 or 4 heads per kv head every head sits in at least four columns; each of the four then
+// With at most 4 heads per kv head every head sits in at least four columns; each of the four then
 // does the softmax and feeds PV for a quarter of a page's tokens only (see combine_quarter).
 // In that case the q * scale operands of a page are not computed by every lane for itself but once
 // per page into an LDS table, and the high plane's operands are scattered to their slots (see
@@ -72,7 +72,7 @@ struct Tables {
 };
 // LDS of one wave.  With tiles streamed through LDS (DMA) the budget is 160 KB / 8 waves per CU,
 // which leaves room for the q rows of 8 heads; larger groups use the register-fed variant.
-// QUARTER (1, 2 or 4 query heads per kv head, see softmax_quarter): four more V scale tables, q rows
+// QUARTER (at most 4 query heads per kv head, see softmax_quarter): four more V scale tables, q rows
 // of 4 heads.
 template <bool DMA, bool QUARTER>
 struct WaveLds;
@@ -542,7 +542,7 @@ __device__ __forceinline__ void qk_packed_tab(LDS& S, const Ctx& x, uint8_t* kt,
   cz = Cz[0];
 }
 
-// Quarter columns.  With 1, 2 or 4 query heads per kv head the 16 columns of a tile hold every
+// Quarter columns.  With at most 4 query heads per kv head the 16 columns of a tile hold every
 // head at least four times (columns n, n ^ 4, n ^ 8, n ^ 12; n and n ^ 8 carry the two parts of
 // q * scale), and the softmax of a page would be computed four times over.  Instead each of the four
 // columns keeps two of the eight 16-token tiles - tiles 2 pi_own + {0, 1}, i.e. operand register
@@ -890,7 +890,7 @@ __device__ __forceinline__ void wait_vmcnt() {
 }
 
 // DMA: packed tiles are streamed global -> LDS (G <= 8); otherwise they are loaded into registers.
-// QUARTER (needs DMA; 1, 2 or 4 query heads per kv head): body pages go through combine_quarter /
+// QUARTER (needs DMA; at most 4 query heads per kv head): body pages go through combine_quarter /
 // softmax_quarter / pv_quarter.
 template <bool BOOST, bool DMA, bool QUARTER>
 __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(kitty_kv_layer L, const __half* __restrict__ q, int H_Q,
@@ -912,7 +912,9 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(kitty_kv_layer L, co
   x.sc2 = scaling * kLog2e;
   const int G = H_Q / L.H_KV;
   constexpr bool SPLIT_COLS = DMA;   // both mean "at most 8 query heads per kv head"
-  x.g = SPLIT_COLS ? (x.n & 7) % G : x.n % G;
+  // quarter columns: column n carries head slot n % 4 (a slot past the last head repeats it; its
+  // columns are never written)
+  x.g = QUARTER ? min(x.n & 3, G - 1) : SPLIT_COLS ? (x.n & 7) % G : x.n % G;
   x.lo_part = SPLIT_COLS && (x.n & 8);
   x.pi_own = ((x.n >> 2) & 1) * 2 + (x.n >> 3);
   {
@@ -1173,7 +1175,7 @@ void launch_decode_mfma(const kitty_kv_layer& L, const void* q, int B, int H_Q, 
                         float* ws_acc, int num_splits, hipStream_t stream) {
   const dim3 grid(num_splits, L.H_KV, B), block(64);
   const int G = H_Q / L.H_KV;
-  const bool boost = L.D_BOOSTED == 32, dma = G <= 8, quarter = G == 1 || G == 2 || G == 4;
+  const bool boost = L.D_BOOSTED == 32, dma = G <= 8, quarter = G <= 4;
 #define KITTY_LAUNCH(BOOST, DMA, QUARTER)                                                                   \
   hipLaunchKernelGGL((decode_mfma_kernel<BOOST, DMA, QUARTER>), grid, block, 0, stream, L, (const __half*)q, H_Q, \
                      scaling, ws_ml, ws_acc, num_splits)

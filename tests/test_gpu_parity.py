@@ -315,7 +315,7 @@ def test_short_and_boundary_prompts(K, variant, T):
     _attend_both(K, cache, ol, H_KV, H_Q, q, variant=variant)
 
 
-@pytest.mark.parametrize("G", [1, 2, 4, 8, 16])
+@pytest.mark.parametrize("G", [1, 2, 3, 4, 5, 6, 8, 12, 16])
 def test_group_sizes(K, G):
     B, H_KV, T = 1, 2, 32 + 128 * 3 + 5
     H_Q = H_KV * G
@@ -325,7 +325,7 @@ def test_group_sizes(K, G):
         _attend_both(K, cache, ol, H_KV, H_Q, q, variant=variant)
 
 
-@pytest.mark.parametrize("G", [1, 4, 8, 16])
+@pytest.mark.parametrize("G", [1, 3, 4, 8, 16])
 def test_no_boosted_channels(K, G):
     """D_BOOSTED = 0 (no high plane): the other half of the kernel instantiations.  The reference's
     cache always boosts head_dim / 4 channels, so the layer is built by hand."""
@@ -349,7 +349,7 @@ def test_no_boosted_channels(K, G):
             _attend_both(K, cache, ol, H_KV, H_Q, q, variant=variant, num_splits=splits)
 
 
-@pytest.mark.parametrize("G", [2, 4, 8, 16])
+@pytest.mark.parametrize("G", [2, 3, 4, 8, 16])
 def test_slots_without_a_channel_contribute_nothing(K, G):
     """A slot map that claims fewer than D_BOOSTED slots (the quantizer never writes one, a caller
     that packs pages itself may): the rows of the high plane that no channel points to hold
