@@ -42,8 +42,9 @@ TRAFFIC_FILE = os.path.join(ROOT, "profiles", "decode_split_pmc_traffic.txt")
 
 def measured_traffic(workload, splits):
     """HBM bytes per launch of the split pass as measured with rocprofv3 --pmc FETCH_SIZE /
-    WRITE_SIZE on this workload (summary committed under profiles/); None when there is no
-    measurement for this workload."""
+    WRITE_SIZE on this workload in a run of its own (counters cannot be read from inside this
+    process): the figure of the summary committed under profiles/, not a measurement of this run.
+    None when there is no such summary for this workload."""
     try:
         with open(TRAFFIC_FILE) as f:
             rec = json.load(f).get(workload)
@@ -51,6 +52,31 @@ def measured_traffic(workload, splits):
     except (OSError, ValueError, KeyError):
         return None
 
+
+
+class HipEvents:
+    """hipEvent_t handles from the HIP runtime this process already has loaded (torch's)."""
+
+    def __init__(self):
+        import ctypes
+        self.ct = ctypes
+        self.hip = ctypes.CDLL("libamdhip64.so")
+        self.hip.hipEventCreate.argtypes = [ctypes.POINTER(ctypes.c_void_p)]
+        self.hip.hipEventElapsedTime.argtypes = [ctypes.POINTER(ctypes.c_float), ctypes.c_void_p, ctypes.c_void_p]
+
+    def create(self):
+        ev = self.ct.c_void_p()
+        rc = self.hip.hipEventCreate(self.ct.byref(ev))
+        if rc != 0:
+            raise RuntimeError(f"hipEventCreate failed ({rc})")
+        return ev
+
+    def elapsed_us(self, a, b) -> float:
+        ms = self.ct.c_float()
+        rc = self.hip.hipEventElapsedTime(self.ct.byref(ms), a, b)
+        if rc != 0:
+            raise RuntimeError(f"hipEventElapsedTime failed ({rc})")
+        return ms.value * 1e3
 
 
 def synth_kv(B, H, T, D, seed, device, student_t=False):
@@ -83,31 +109,34 @@ def algorithmic_bytes(B, H_Q, H_KV, layer):
     return B * (H_KV * (per_head_packed + per_head_fp16) + qo), B * H_KV * per_head_packed
 
 
-def cpu_baseline(K_row, V_row, q_row, H_Q, H_KV, B_full, budget_s=20.0):
-    """The reference's CPU path (fake-quant simulator + eager attention) on one sequence of the
-    workload, on the host cores; scaled by the batch size to the workload's step."""
+def cpu_baseline(K, V, q, H_Q, H_KV):
+    """The reference's CPU path (fake-quant simulator + eager attention) on the whole workload - every
+    sequence, full context - on the host cores; few repetitions rather than a smaller shape.  `value`
+    is the attention step (what the metric measures); the one-time fake quantization of the context is
+    reported beside it."""
     import torch
     from oracle import sim_baseline as S
     cores = os.cpu_count() or 1
     threads = min(cores, 16)
     torch.set_num_threads(threads)
-    K, V = K_row.clone(), V_row.clone()
+    K, V = K.clone(), V.clone()
     t0 = time.perf_counter()
     S.simulate_prefill(K, V)
     t_quant = time.perf_counter() - t0
-    S.eager_attention(q_row, K, V, 128 ** -0.5, H_Q // H_KV)          # warm-up
+    n_rep = H_Q // H_KV
+    S.eager_attention(q, K, V, 128 ** -0.5, n_rep)          # warm-up
     reps, t_att = 0, 0.0
-    while reps < 3 or (t_att < budget_s / 2 and reps < 20):
+    while reps < 2 or (t_att < 10.0 and reps < 10):
         t0 = time.perf_counter()
-        S.eager_attention(q_row, K, V, 128 ** -0.5, H_Q // H_KV)
+        S.eager_attention(q, K, V, 128 ** -0.5, n_rep)
         t_att += time.perf_counter() - t0
         reps += 1
-    us = t_att / reps * 1e6 * B_full
     return {
-        "value": us, "unit": "us/step", "cores": threads, "kind": "port",
-        "sample": (f"1 of {B_full} sequences of the workload (dense fake-quantized fp16 KV, eager GQA attention, "
-                   f"{reps} reps, torch {threads} threads), time x{B_full}; fake-quant of that sequence took "
-                   f"{t_quant:.2f} s once"),
+        "value": t_att / reps * 1e6, "unit": "us/step", "cores": threads, "kind": "port",
+        "sample": (f"the whole workload ({K.shape[0]} sequences x {K.shape[2]} tokens, dense fake-quantized fp16 KV, eager "
+                   f"GQA attention with fp32 softmax), 1 warm-up + {reps} timed steps, torch {threads} threads; the "
+                   f"fake quantization of the context took {t_quant:.2f} s once and is not part of the step"),
+        "fake_quant_s_once": t_quant,
     }
 
 
@@ -258,7 +287,79 @@ def bench_fake_quant(args):
     print(json.dumps(result))
 
 
+def bench_generate(args):
+    """End-to-end as the reference measures it (latency_benchmarking/benchmark_kitty.py:127-197): a stock
+    transformers model - random-init Llama-3.1-8B or Qwen3-8B shapes from a local config, nothing is
+    downloaded - with ``attn_implementation="kitty"`` and a fresh ``KittyHFCache`` per run, ``generate()``
+    greedy to ``max_length`` with early stopping disabled; warm-up runs, then a synchronised wall clock
+    over the repeat runs."""
+    import torch
+    import transformers
+    from kitty_amd import _lib, hf
+    _lib.lib()
+    hf.register()
+    dev = torch.device("cuda:0")
+    B, T0, max_len = args.e2e_batch, args.e2e_prompt, args.e2e_max_len
+    common = dict(hidden_size=4096, num_hidden_layers=32, num_attention_heads=32, num_key_value_heads=8, head_dim=128,
+                  max_position_embeddings=131072, attn_implementation="kitty")
+    if args.e2e_model == "qwen3":
+        cfg = transformers.Qwen3Config(vocab_size=151936, intermediate_size=12288, rope_theta=1000000.0, **common)
+        cls, name = transformers.Qwen3ForCausalLM, "Qwen3-8B"
+    else:
+        cfg = transformers.LlamaConfig(vocab_size=128256, intermediate_size=14336, rope_theta=500000.0, **common)
+        cls, name = transformers.LlamaForCausalLM, "Llama-3.1-8B"
+    torch.manual_seed(0)
+    old = torch.get_default_dtype()
+    torch.set_default_dtype(torch.float16)
+    try:
+        with torch.device(dev):
+            model = cls(cfg)
+    finally:
+        torch.set_default_dtype(old)
+    model.eval()
+    ids = torch.randint(0, cfg.vocab_size, (B, T0), generator=torch.Generator().manual_seed(1)).to(dev)
+
+    def run():
+        cache = hf.KittyHFCache(cfg, B, max_len, device=dev)
+        out = model.generate(input_ids=ids, max_length=max_len, max_new_tokens=None, return_dict_in_generate=False,
+                             do_sample=False, temperature=None, top_p=None, top_k=None, past_key_values=cache,
+                             eos_token_id=None, pad_token_id=0, disable_compile=True)
+        return out, cache
+
+    with torch.no_grad():
+        for _ in range(args.e2e_warmup_runs):
+            run()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.e2e_repeat_runs):
+            out, cache = run()
+        torch.cuda.synchronize()
+        dt = (time.perf_counter() - t0) / args.e2e_repeat_runs
+    assert tuple(out.shape) == (B, max_len) and cache.get_seq_length(0) == max_len - 1
+    cache.check_status()
+    new = max_len - T0
+    print(json.dumps({
+        "metric": "end_to_end_generate_tokens_per_s", "value": B * new / dt, "unit": "tokens/s", "n_gpus": 1,
+        "steps": args.e2e_repeat_runs, "warmup": args.e2e_warmup_runs, "ms_per_step": dt * 1e3 / new,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16 model, 2/4-bit packed KV",
+        "data": f"synthetic (random-init {name} shapes, random prompt tokens)",
+        "config": {"workload": f"stock transformers {cls.__name__} ({name} shapes, 32 layers) through the attention hook: "
+                               f"generate() of batch {B}, prompt {T0}, to max_length {max_len}, greedy, fresh cache per run",
+                   "batch": B, "prompt": T0, "max_length": max_len, "layers": 32, "mode": "generate",
+                   "transformers": transformers.__version__},
+        "generate_s_per_run": dt, "new_tokens_per_sequence": new,
+        "note": "one step = one decode iteration of generate(); the host-side launch sequence of the stock model's "
+                "dense layers is inside the timed region, as in the reference's benchmark",
+    }))
+
+
 def bench_end_to_end(args):
+    if args.e2e_mode == "generate":
+        return bench_generate(args)
+    return bench_decode_loop(args)
+
+
+def bench_decode_loop(args):
     """The side number of configs[4]: decode tokens/s of a full 32-layer Llama-3.1-8B-shaped model
     with random weights, every layer's KV in the packed cache.  The dense parts (projections, MLP,
     norms, RoPE, LM head) are plain torch; attention and the cache are this library, driven in the
@@ -298,9 +399,11 @@ def bench_end_to_end(args):
 
     inv_freq = 1.0 / (500000.0 ** (torch.arange(0, D, 2, device=dev, dtype=torch.float32) / D))
 
-    def rope(x, pos):                     # x [B, H, 1, D], rotate-half convention; pos: float or 0-d tensor
+    def rope_table(pos):                  # pos: float or 0-d tensor -> (cos, sin), fp16 [1, D]
         ang = pos * inv_freq
-        cos, sin = torch.cat([ang.cos(), ang.cos()]).half(), torch.cat([ang.sin(), ang.sin()]).half()
+        return (torch.cat([ang.cos(), ang.cos()]).half().view(1, D), torch.cat([ang.sin(), ang.sin()]).half().view(1, D))
+
+    def rope(x, cos, sin):                # x [B, H, 1, D], rotate-half convention
         x1, x2 = x[..., : D // 2], x[..., D // 2:]
         return x * cos + torch.cat([-x2, x1], dim=-1) * sin
 
@@ -311,12 +414,16 @@ def bench_end_to_end(args):
     @torch.no_grad()
     def step(cache, tok, pos):
         x = emb[tok]                      # [B, HID]: 2-D activations keep the GEMM launches cheap
+        cos, sin = rope_table(pos)
         for li, w in enumerate(layers):
             h = rms(x, w["n1"])
             qkv = F.linear(h, w["wqkv"]).view(B, 1, H_Q + 2 * H_KV, D).transpose(1, 2)
             q, k, v = qkv[:, :H_Q], qkv[:, H_Q:H_Q + H_KV], qkv[:, H_Q + H_KV:]
-            q, k = rope(q, pos).contiguous(), rope(k, pos)
-            cache.update(k, v, li)
+            q = rope(q, cos, sin).contiguous()
+            if mode == "host":
+                cache.update(rope(k, cos, sin), v, li)
+            else:                         # the append kernel rotates the key itself (same bits)
+                cache.update_with_rope(k, v, cos, sin, li)
             a, _ = kitty_attention_forward(mod, q, cache.kv_cache[li], D ** -0.5)
             cache.quantize_decode(li)
             x = x + F.linear(a.view(B, HID), w["wo"])
@@ -383,7 +490,8 @@ def bench_end_to_end(args):
     dt = (time.perf_counter() - t0) / args.steps
     notes = {"host": "dense layers are torch (hipBLASLt); one Python-driven launch sequence per layer, host counters "
                      "(the reference's mode), not graph-captured",
-             "device": "as host mode, but per-sequence counters on the device (fused append + flush launches)",
+             "device": "as host mode, but per-sequence counters on the device (append fused with the key's rotary "
+                       "embedding, flush launches)",
              "graph": "per-sequence counters on the device; the whole step captured once in a HIP graph and replayed"}
     print(json.dumps({
         "metric": "end_to_end_decode_tokens_per_s", "value": B / dt, "unit": "tokens/s", "n_gpus": 1,
@@ -406,9 +514,17 @@ def main():
     ap.add_argument("--workload", default="c1", choices=sorted(WORKLOADS) + ["c3", "e2e", "fq"])
     ap.add_argument("--e2e-batch", type=int, default=16)
     ap.add_argument("--e2e-context", type=int, default=32768)
-    ap.add_argument("--e2e-mode", default="host", choices=["host", "device", "graph"],
-                    help="host: the reference's shared host counters; device: per-sequence counters on the device; "
-                         "graph: device counters and the whole step replayed from one captured HIP graph")
+    ap.add_argument("--e2e-mode", default="generate", choices=["generate", "host", "device", "graph"],
+                    help="generate: a stock transformers model through the attention hook, generate() as the "
+                         "reference's benchmark runs it; the others drive hand-written dense layers around the cache "
+                         "over a long synthetic context - host: the reference's shared host counters; device: "
+                         "per-sequence counters on the device; graph: device counters and the whole step replayed "
+                         "from one captured HIP graph")
+    ap.add_argument("--e2e-model", default="llama", choices=["llama", "qwen3"])
+    ap.add_argument("--e2e-prompt", type=int, default=64)
+    ap.add_argument("--e2e-max-len", type=int, default=1024)
+    ap.add_argument("--e2e-warmup-runs", type=int, default=1)
+    ap.add_argument("--e2e-repeat-runs", type=int, default=2)
     ap.add_argument("--copies", type=int, default=0, help="independent cache copies to rotate over (0 = auto)")
     ap.add_argument("--splits", type=int, default=0)
     ap.add_argument("--variant", type=int, default=0)
@@ -500,9 +616,7 @@ def main():
                     dtype=torch.float32).half()
     out = torch.empty((B, 1, H_Q, D), dtype=torch.float16, device=dev)
     max_tiles = (2 + L0.MAX_PAGE) if seq_counts is not None else 1 + (T - L0.Sink_Count + 127) // 128
-    splits = args.splits or lib.kitty_decode_attn_default_splits(B, H_KV, max_tiles)
-    if not args.splits and seq_counts is not None and splits < 12:
-        splits = 12          # the library's rule for batches with per-sequence lengths
+    splits = args.splits or lib.kitty_decode_attn_default_splits(B, H_KV, max_tiles, int(seq_counts is not None))
     ws_bytes = lib.kitty_decode_attn_workspace_bytes(B, H_Q, D, splits)
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
     if seq_counts is not None:
@@ -512,38 +626,56 @@ def main():
     stream = torch.cuda.current_stream(dev).cuda_stream
     scaling = D ** -0.5
 
+    hip = HipEvents()
+
     def step(i, ev=None):
         d = descs[i % len(descs)]
-        if ev is not None:
-            ev[0].record()
+        if ev is not None:     # the events ride on the split kernel's own dispatch: its duration on the device
+            _lib.check(lib.kitty_profile_next_split(ev[0], ev[1]), "profile")
         rc = lib.kitty_decode_attn_split(d, q.data_ptr(), B, H_Q, scaling, ws.data_ptr(), ws_bytes, splits,
                                          args.variant, stream)
-        if ev is not None:
-            ev[1].record()
         _lib.check(rc, "split")
         _lib.check(lib.kitty_decode_attn_merge(ws.data_ptr(), ws_bytes, B, H_Q, D, splits, out.data_ptr(), stream),
                    "merge")
 
+    # Untimed, whatever --warmup says: after idle the clocks need some hundred launches to settle, and a
+    # short run would time the ramp.  Windows of 20 launches until the median kernel duration moves by
+    # less than 1 % three windows in a row (at most 150 windows).
+    n_done, settle = 0, {"windows": 0, "median_us": None, "settled": False}
+    win = [(hip.create(), hip.create()) for _ in range(20)]
+    prev, stable = None, 0
+    for w in range(150):
+        for e in win:
+            step(n_done, e)
+            n_done += 1
+        torch.cuda.synchronize()
+        med = sorted(hip.elapsed_us(a, b) for a, b in win)[len(win) // 2]
+        stable = stable + 1 if prev is not None and abs(med - prev) <= 0.01 * prev else 0
+        prev = med
+        settle.update(windows=w + 1, median_us=med)
+        if stable >= 3:
+            settle["settled"] = True
+            break
     for i in range(args.warmup):
-        step(i)
+        step(n_done + i)
+    n_done += args.warmup
     torch.cuda.synchronize()
-    events = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+    events = [(hip.create(), hip.create()) for _ in range(args.steps)]
     t0 = time.perf_counter()
     for i in range(args.steps):
-        step(i, events[i])
+        step(n_done + i, events[i])
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
     ms_per_step = wall / args.steps * 1e3
-    kern_us = sorted(a.elapsed_time(b) * 1e3 for a, b in events)
+    kern_us = sorted(hip.elapsed_us(a, b) for a, b in events)
     kern_avg_us = sum(kern_us) / len(kern_us)
     achieved = total_bytes / (kern_avg_us * 1e-6) / 1e9
 
     # cache-hot figure (same copy every step), reported separately
-    hot_ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(20)]
     for i in range(20):
-        step(0, hot_ev[i])
+        step(0, win[i])
     torch.cuda.synchronize()
-    hot_us = sorted(a.elapsed_time(b) * 1e3 for a, b in hot_ev)[len(hot_ev) // 2]
+    hot_us = sorted(hip.elapsed_us(a, b) for a, b in win)[len(win) // 2]
 
     if args.copy_calibration:
         src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).fill_(3)
@@ -577,12 +709,17 @@ def main():
             "packed_gbps": packed_bytes / (kern_avg_us * 1e-6) / 1e9,
             "packed_frac": packed_bytes / (kern_avg_us * 1e-6) / 1e9 / HBM_PEAK_GBPS,
             "cache_hot_kernel_us": hot_us,
+            "timing": "HIP events attached to the split kernel's dispatch on the launch stream (kernel begin to end), "
+                      "averaged over the timed steps",
+            "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE summary committed under profiles/ (a run of "
+                              "its own, calibrated by a 1 GiB copy), not measured in this run",
+            "clock_settling": settle,
         },
         "quantizer": {"gbps_in": quant_gbps, "ms": min(quant_ms), "input_bytes": quant_in_bytes,
                       "what": "quantize_prefill of the whole context (K select+quantize+pack, V quantize+pack)"},
     }
     if not args.no_cpu_baseline:
-        result["cpu_baseline"] = cpu_baseline(K[:1].cpu(), V[:1].cpu(), q[:1].cpu(), H_Q, H_KV, B)
+        result["cpu_baseline"] = cpu_baseline(K.cpu(), V.cpu(), q.cpu(), H_Q, H_KV)
     print(json.dumps(result))
 
 

@@ -21,7 +21,7 @@
 extern "C" {
 #endif
 
-#define KITTY_ABI_VERSION 1
+#define KITTY_ABI_VERSION 2
 
 enum {
   KITTY_OK = 0,
@@ -54,15 +54,39 @@ enum {
   KITTY_SEQ_COUNT_FIELDS = 8
 };
 /* Flag bits of a sequence's counter row.  INACTIVE: the slot holds no sequence (or a paused one):
- * kitty_append_token and kitty_flush_full leave it alone; attention still sees what its counters
+ * the append and flush entry points leave it alone; attention still sees what its counters
  * describe, nothing when they are zero. */
 enum { KITTY_SEQ_INACTIVE = 1 };
+
+/*
+ * Device-side status, one row of int32 per sequence (kitty_kv_layer.status, optional).  The
+ * reference stops with a Python assert before a buffer overflows (kitty.py:109,113,118) or a page
+ * is missing; kernels that take their occupancy from device memory cannot, so they skip the work
+ * that would go out of bounds, exit normally and leave a record here.  The words are sticky: the
+ * kernels only ever raise them, the host reads and clears them when it wants to know.
+ */
+enum {
+  KITTY_STATUS_TOKENS_DROPPED = 0,   /* count: tokens not appended because a Q-buffer was still full
+                                        (or, for a chunk, because it did not fit)                    */
+  KITTY_STATUS_FLUSH_SKIPPED = 1,    /* count: full Q-buffers left unflushed (no page assigned, or
+                                        the sequence is at MAX_PAGE)                                 */
+  KITTY_STATUS_BAD_PAGE_WRITE = 2,   /* flag: a quantize / flush kernel met a page id outside
+                                        [0, cache_pages) other than -1 and wrote nothing             */
+  KITTY_STATUS_BAD_PAGE_READ = 3,    /* flag: an attention kernel met a page id outside
+                                        [0, cache_pages); it read page 0 instead, the output of that
+                                        sequence is meaningless                                      */
+  KITTY_STATUS_FIELDS = 4
+};
 
 typedef struct kitty_kv_layer {
   int32_t H_KV, D, D_BOOSTED, PAGE_SIZE, S, MAX_PAGE;
   int32_t counts[KITTY_SEQ_COUNT_FIELDS];       /* used when seq_counts == NULL */
   const int32_t* seq_counts;                    /* optional, device, [B][8]; the two append
                                                    entry points below write it */
+
+  int32_t* status;                              /* optional, device, [B][KITTY_STATUS_FIELDS]  */
+  int64_t cache_pages_k, cache_pages_v;         /* pages the K / V arrays below hold: every page id
+                                                   read from a page table is checked against them */
 
   const uint8_t* key_cache;    int64_t key_cache_stride_page;     /* KeyCache            */
   const void*    key_meta;     int64_t key_meta_stride_page;      /* KeyCache_metadata   */
@@ -99,7 +123,8 @@ int kitty_select_boost_k(const void* key, int64_t stride_b, int64_t stride_h, in
  * slot_map NULL: the selection above is fused into the same kernel (one pass over K).
  * slot_map given: uint8 [B,H,pages,D], consumed exactly like the reference kernel consumes
  * dense_sparse_idx.  meta is fp16 [pages_total,H,D,2] (scale, zero).  page_table_stride_b counts
- * int64 entries; every other stride is in bytes.
+ * int64 entries; every other stride is in bytes.  A page id outside [0, cache_pages) is never
+ * written to; status (optional, device, [B][KITTY_STATUS_FIELDS]) records it.
  */
 int kitty_quant_pack_k(const void* key, int64_t stride_b, int64_t stride_h, int64_t stride_t,
                        int B, int H, int T, int D, int t_offset, int pages, int page_size, int d_boost,
@@ -107,7 +132,7 @@ int kitty_quant_pack_k(const void* key, int64_t stride_b, int64_t stride_h, int6
                        const int64_t* page_table, int64_t page_table_stride_b, int page_offset,
                        uint8_t* cache, int64_t cache_stride_page,
                        void* meta, int64_t meta_stride_page,
-                       int64_t cache_pages, void* stream);
+                       int64_t cache_pages, int32_t* status, void* stream);
 
 /*
  * Replaces quantize_pack_v_kernel and its launch (kernels/kitty_quant_pack.py:155-249, 339-356).
@@ -118,7 +143,7 @@ int kitty_quant_pack_v(const void* value, int64_t stride_b, int64_t stride_h, in
                        const int64_t* page_table, int64_t page_table_stride_b, int page_offset,
                        uint8_t* cache, int64_t cache_stride_page,
                        void* meta, int64_t meta_stride_page,
-                       int64_t cache_pages, void* stream);
+                       int64_t cache_pages, int32_t* status, void* stream);
 
 /*
  * Decode attention over the packed cache.  Replaces qk_kernel + torch softmax + sv_kernel as
@@ -126,11 +151,13 @@ int kitty_quant_pack_v(const void* value, int64_t stride_b, int64_t stride_h, in
  * split-K pass (QK^T, online softmax, PV per split of the sequence) and a merge pass.
  * q: fp16 [B,H_Q,1,D] contiguous.  out: fp16 [B,1,H_Q,D] contiguous.
  * workspace: at least kitty_decode_attn_workspace_bytes(B,H_Q,D,num_splits) bytes, 256-aligned.
- * num_splits <= 0 picks kitty_decode_attn_default_splits().  variant: 0 = default kernel,
- * 1 = the plain reference-order kernel (fp16 dequantization, no matrix cores).
+ * num_splits <= 0 picks kitty_decode_attn_default_splits() (max_tiles = 1 + the 128-token tiles
+ * after the sink of the longest sequence; per_sequence_counts = layer->seq_counts is set).
+ * variant: 0 = default kernel, 1 = the plain reference-order kernel (fp16 dequantization, no
+ * matrix cores).
  */
 size_t kitty_decode_attn_workspace_bytes(int B, int H_Q, int D, int num_splits);
-int kitty_decode_attn_default_splits(int B, int H_KV, int max_tiles);
+int kitty_decode_attn_default_splits(int B, int H_KV, int max_tiles, int per_sequence_counts);
 int kitty_decode_attn(const kitty_kv_layer* layer, const void* q, int B, int H_Q, float scaling,
                       void* out, void* workspace, size_t workspace_bytes, int num_splits,
                       int variant, void* stream);
@@ -151,6 +178,17 @@ int kitty_decode_attn_merge(const void* workspace, size_t workspace_bytes, int B
                             int num_splits, void* out, void* stream);
 
 /*
+ * Measurement aid, no counterpart in the reference (which times whole generate() calls,
+ * latency_benchmarking/benchmark_kitty.py:129-183): the next split pass that the calling thread
+ * launches (kitty_decode_attn_split, or inside kitty_decode_attn) attaches the two hipEvent_t to its
+ * kernel's own dispatch, so that hipEventElapsedTime between them is the kernel's duration on the
+ * device - the figure a kernel trace reports - without the host's enqueue gaps that an event pair
+ * recorded around the call includes.  The events must have timing enabled and outlive the launch.
+ * (NULL, NULL) cancels.  The plain variant records the events around its launch instead.
+ */
+int kitty_profile_next_split(void* start_event, void* stop_event);
+
+/*
  * Chunked-prefill attention: T_q new tokens attend to everything the layer already holds (sink
  * rows, packed pages, fp16 windows, in the token order of decode) and, causally, to the keys and
  * values of the chunk itself, which are still fp16 and not yet appended.  An extension: the
@@ -169,9 +207,9 @@ int kitty_prefill_attn(const kitty_kv_layer* layer,
 
 /*
  * Decode-time bookkeeping with per-sequence counters kept on the device (layer->seq_counts must be
- * set; it is read AND written).  The reference keeps one set of host ints for the whole batch and
+ * set; it is read AND written; layer->status, when set, is written).  The reference keeps one set of host ints for the whole batch and
  * drives slice copies from them (KittyCache.update, kitty.py:97-123; quantize_decode,
- * kitty.py:194-236); these two calls run the same state machine per sequence, with no host
+ * kitty.py:194-236); these calls run the same state machine per sequence, with no host
  * round trip, so that sequences of different lengths decode in one batch and the launch sequence
  * of a decode step never changes (a captured graph can replay it).  Call order per step, as in
  * modeling_qwen3.py:225-251: kitty_append_token, kitty_decode_attn, kitty_flush_full.
@@ -179,17 +217,38 @@ int kitty_prefill_attn(const kitty_kv_layer* layer,
  * kitty_append_token: one token per sequence.  k_new / v_new: fp16 [B,H_KV,1,D], D contiguous, byte
  * strides.  Per sequence: sink not full -> the sink row; else K -> Q_Buffer_K[Q_Buffer_Count_K],
  * V -> the local ring (a full ring first moves its oldest row to Q_Buffer_V).  A sequence whose
- * Q-buffer is full (a skipped kitty_flush_full) is left unchanged and the token dropped.
+ * Q-buffer is full (a skipped kitty_flush_full) is left unchanged, the token dropped and counted in
+ * status[KITTY_STATUS_TOKENS_DROPPED].
+ * rope_cos / rope_sin (optional, both or neither): fp16 [B,D] rows with byte stride rope_stride_b,
+ * the rotary embedding of each sequence's position.  When given, k_new holds the keys BEFORE the
+ * rotation and the kernel stores k * cos + rotate_half(k) * sin, each product and the sum rounded
+ * to fp16, which is what the caller's own fp16 tensor expression computes
+ * (modeling_qwen3.py:215-220 feeding kitty.py:102-123): one launch less and no rotated copy of K.
  *
  * kitty_flush_full: every sequence whose K (V) Q-buffer holds PAGE_SIZE rows gets it quantized,
  * with channel selection, into page page_table[b][PageCount] and its counters advanced; the
  * arithmetic is that of kitty_quant_pack_k / _v.  A sequence already at MAX_PAGE pages, or whose
- * page id is outside [0, cache_pages) (a page table entry of -1: no page assigned), is left as it
- * is, Q-buffer full, and drops the tokens appended until a later call finds a page there.
+ * page id is outside [0, layer->cache_pages_k / _v) (a page table entry of -1: no page assigned),
+ * is left as it is, Q-buffer full, counted in status[KITTY_STATUS_FLUSH_SKIPPED], and drops the
+ * tokens appended until a later call finds a page there.
+ *
+ * kitty_append_chunk: T >= 1 tokens per sequence in one call, k_new / v_new fp16 [B,H_KV,T,D].  The
+ * state afterwards is the one T rounds of kitty_append_token + kitty_flush_full leave: same
+ * counters, same packed pages bit for bit, same fp16 rows in the same slots of the sink, the
+ * Q-buffers and the ring (rows of a Q-buffer beyond its fill count are not part of the state).
+ * Pages that fill up inside the chunk are quantized straight from their sources (buffered rows
+ * and chunk rows) without a trip through the Q-buffer.  A sequence the chunk does not fit (it
+ * would pass MAX_PAGE, or needs a page whose table entry is not a valid page id) is left
+ * unchanged and its T tokens counted as dropped.  No counterpart in the reference, whose update()
+ * asserts one token per call once the cache holds anything (kitty.py:97-98).
  */
 int kitty_append_token(const kitty_kv_layer* layer, const void* k_new, const void* v_new,
-                       int64_t stride_b, int64_t stride_h, int B, void* stream);
-int kitty_flush_full(const kitty_kv_layer* layer, int B, int64_t cache_pages, void* stream);
+                       int64_t stride_b, int64_t stride_h,
+                       const void* rope_cos, const void* rope_sin, int64_t rope_stride_b,
+                       int B, void* stream);
+int kitty_flush_full(const kitty_kv_layer* layer, int B, void* stream);
+int kitty_append_chunk(const kitty_kv_layer* layer, const void* k_new, const void* v_new,
+                       int64_t stride_b, int64_t stride_h, int64_t stride_t, int B, int T, void* stream);
 
 /*
  * Fake quantization of dense fp16 keys or values in place: replaces fake_quant_groupwise_lastdim of

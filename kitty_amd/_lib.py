@@ -9,8 +9,11 @@ from ctypes import POINTER, c_char_p, c_float, c_int, c_int32, c_int64, c_size_t
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "libkitty_hip.so")
-ABI_VERSION = 1
+ABI_VERSION = 2
 SEQ_COUNT_FIELDS = 8
+STATUS_FIELDS = 4
+# order of a status row (KITTY_STATUS_*, include/kitty_hip.h)
+STATUS_NAMES = ("tokens_dropped", "flush_skipped", "bad_page_write", "bad_page_read")
 
 # order of kitty_kv_layer.counts / seq_counts rows (include/kitty_hip.h)
 CNT_SINK, CNT_PAGES_K, CNT_QBUF_K, CNT_PAGES_V, CNT_QBUF_V, CNT_LOCAL_V, CNT_LOCAL_OFF = range(7)
@@ -23,6 +26,8 @@ class KittyKVLayer(ctypes.Structure):
         ("S", c_int32), ("MAX_PAGE", c_int32),
         ("counts", c_int32 * SEQ_COUNT_FIELDS),
         ("seq_counts", c_void_p),
+        ("status", c_void_p),
+        ("cache_pages_k", c_int64), ("cache_pages_v", c_int64),
         ("key_cache", c_void_p), ("key_cache_stride_page", c_int64),
         ("key_meta", c_void_p), ("key_meta_stride_page", c_int64),
         ("value_cache", c_void_p), ("value_cache_stride_page", c_int64),
@@ -43,21 +48,25 @@ _SIGNATURES = {
                                      c_int, c_int, c_void_p, c_void_p]),
     "kitty_quant_pack_k": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_int, c_int, c_int, c_int, c_int, c_int,
                                    c_int, c_int, c_void_p, c_void_p, c_int64, c_int, c_void_p, c_int64, c_void_p,
-                                   c_int64, c_int64, c_void_p]),
+                                   c_int64, c_int64, c_void_p, c_void_p]),
     "kitty_quant_pack_v": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_int, c_int, c_int, c_int, c_int, c_int,
                                    c_int, c_void_p, c_int64, c_int, c_void_p, c_int64, c_void_p, c_int64, c_int64,
-                                   c_void_p]),
+                                   c_void_p, c_void_p]),
     "kitty_decode_attn_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int]),
-    "kitty_decode_attn_default_splits": (c_int, [c_int, c_int, c_int]),
+    "kitty_decode_attn_default_splits": (c_int, [c_int, c_int, c_int, c_int]),
     "kitty_decode_attn_split": (c_int, [POINTER(KittyKVLayer), c_void_p, c_int, c_int, c_float, c_void_p, c_size_t,
                                         c_int, c_int, c_void_p]),
     "kitty_decode_attn_merge": (c_int, [c_void_p, c_size_t, c_int, c_int, c_int, c_int, c_void_p, c_void_p]),
+    "kitty_profile_next_split": (c_int, [c_void_p, c_void_p]),
     "kitty_decode_attn": (c_int, [POINTER(KittyKVLayer), c_void_p, c_int, c_int, c_float, c_void_p, c_void_p,
                                   c_size_t, c_int, c_int, c_void_p]),
     "kitty_prefill_attn": (c_int, [POINTER(KittyKVLayer), c_void_p, c_int64, c_int64, c_int64, c_void_p, c_void_p,
                                    c_int64, c_int64, c_int64, c_int, c_int, c_int, c_float, c_void_p, c_void_p]),
-    "kitty_append_token": (c_int, [POINTER(KittyKVLayer), c_void_p, c_void_p, c_int64, c_int64, c_int, c_void_p]),
-    "kitty_flush_full": (c_int, [POINTER(KittyKVLayer), c_int, c_int64, c_void_p]),
+    "kitty_append_token": (c_int, [POINTER(KittyKVLayer), c_void_p, c_void_p, c_int64, c_int64, c_void_p, c_void_p,
+                                   c_int64, c_int, c_void_p]),
+    "kitty_flush_full": (c_int, [POINTER(KittyKVLayer), c_int, c_void_p]),
+    "kitty_append_chunk": (c_int, [POINTER(KittyKVLayer), c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int, c_int,
+                                   c_void_p]),
     "kitty_fake_quant": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_int, c_int, c_int, c_int, c_int, c_int,
                                  c_int, c_int, c_int, c_void_p, c_int64, c_int64, c_int64, c_int, c_void_p]),
 }

@@ -9,7 +9,8 @@ void launch_decode_merge(const float* ws_ml, const float* ws_acc, void* out, int
                          hipStream_t stream);
 bool decode_mfma_supported(const kitty_kv_layer& L, int H_Q);
 void launch_decode_mfma(const kitty_kv_layer& L, const void* q, int B, int H_Q, float scaling, float* ws_ml,
-                        float* ws_acc, int num_splits, hipStream_t stream);
+                        float* ws_acc, int num_splits, int n_simds, hipStream_t stream, hipEvent_t ev_start,
+                        hipEvent_t ev_stop);
 void launch_prefill_attn(const kitty_kv_layer& L, const void* q, int64_t q_stride_b, int64_t q_stride_h,
                          int64_t q_stride_t, const void* k_new, const void* v_new, int64_t new_stride_b,
                          int64_t new_stride_h, int64_t new_stride_t, int B, int H_Q, int Tq, float scaling,
@@ -23,24 +24,47 @@ extern "C" size_t kitty_decode_attn_workspace_bytes(int B, int H_Q, int D, int n
   return ws_total_bytes(B, H_Q, num_splits);
 }
 
-// Enough workgroups to cover every SIMD of the 256 CUs twice over, but no body split with fewer
+namespace kitty {
+// SIMDs of the current device (4 per compute unit), asked once per process; 1024 (a whole MI355X)
+// when there is no device to ask, so that the split rule can be evaluated without one.
+int device_simds() {
+  static const int n = [] {
+    int dev = 0, cus = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) {
+      (void)hipGetLastError();
+      cus = 256;
+    }
+    return 4 * cus;
+  }();
+  return n;
+}
+}  // namespace kitty
+
+// Enough single-wave workgroups to put two on every SIMD of the device, but no body split with fewer
 // than 4 tiles (a wave's fixed cost is about one tile's worth); three more for the sink and the
 // tiles with fp16 rows when the body splits are short.  When the splits are short (under 8 tiles)
 // the waves with the fp16 rows are the critical path, and a launch that fills the machine exactly
-// puts two of them on the same SIMD (workgroup i shares a SIMD with i + 1024): 15/16 of the
-// machine is faster then (B=1, 128k tokens: 32 us with 240 splits, 40 us with 256).
-extern "C" int kitty_decode_attn_default_splits(int B, int H_KV, int max_tiles) {
+// puts two of them on the same SIMD (workgroup i shares a SIMD with i + SIMDs): 15/16 of the
+// machine is faster then (B=1, 128k tokens: 32 us with 240 splits, 40 us with 256).  Sequences with
+// their own lengths (per_sequence_counts) get at least 12 splits when they can be long: more,
+// shorter splits even out the load.
+extern "C" int kitty_decode_attn_default_splits(int B, int H_KV, int max_tiles, int per_sequence_counts) {
   if (B <= 0 || H_KV <= 0 || max_tiles <= 0) return 1;
-  const int units = B * H_KV;
-  int s = (2048 + units - 1) / units;
-  if (max_tiles < 8 * s) s = (1920 + units - 1) / units;
+  const int units = B * H_KV, slots = 2 * device_simds();
+  int s = (slots + units - 1) / units;
+  if (max_tiles < 8 * s) s = (slots - slots / 16 + units - 1) / units;
   const int by_tiles = (max_tiles + 3) / 4 + 3;
   if (s > by_tiles) s = by_tiles;
+  if (per_sequence_counts && s < 12 && max_tiles >= 48) s = 12;
   if (s > 512) s = 512;
   return s < 1 ? 1 : s;
 }
 
 namespace {
+
+// events for the next split pass launched by this thread (kitty_profile_next_split)
+thread_local hipEvent_t g_ev_start = nullptr, g_ev_stop = nullptr;
 
 int check_layer(const kitty_kv_layer* layer, const void* q, int B, int H_Q, int* max_tiles) {
   KITTY_REQUIRE(layer && q, KITTY_E_NULL, "layer / q is NULL");
@@ -66,6 +90,9 @@ int check_layer(const kitty_kv_layer* layer, const void* q, int B, int H_Q, int*
                     ((uintptr_t)L.local_v % 16) == 0 && L.sink_stride_b % 16 == 0 && L.sink_stride_h % 16 == 0 &&
                     L.win_stride_b % 16 == 0 && L.win_stride_h % 16 == 0 && ((uintptr_t)q % 16) == 0,
                 KITTY_E_ALIGN, "cache tensors and q need 16-byte alignment");
+  KITTY_REQUIRE(L.cache_pages_k >= 0 && L.cache_pages_v >= 0 && ((uintptr_t)L.status % 4) == 0 &&
+                    ((uintptr_t)L.seq_counts % 4) == 0,
+                KITTY_E_RANGE, "negative cache_pages_k / cache_pages_v, or misaligned status / seq_counts");
   KITTY_REQUIRE(L.key_cache_stride_page >= (int64_t)L.H_KV * k_head_bytes(L.D_BOOSTED) &&
                     L.value_cache_stride_page >= (int64_t)L.H_KV * kVBytes &&
                     L.key_meta_stride_page >= (int64_t)L.H_KV * kD * 4 &&
@@ -85,6 +112,8 @@ int check_layer(const kitty_kv_layer* layer, const void* q, int B, int H_Q, int*
     const int nv = c[KITTY_CNT_PAGES_V] * kPage + c[KITTY_CNT_QBUF_V] + c[KITTY_CNT_LOCAL_V];
     KITTY_REQUIRE(nk == nv, KITTY_E_RANGE, "seqlen_K: %d, seqlen_V: %d", nk + c[KITTY_CNT_SINK],
                   nv + c[KITTY_CNT_SINK]);
+    KITTY_REQUIRE((c[KITTY_CNT_PAGES_K] == 0 || L.cache_pages_k > 0) && (c[KITTY_CNT_PAGES_V] == 0 || L.cache_pages_v > 0),
+                  KITTY_E_RANGE, "the counters name packed pages but cache_pages_k / cache_pages_v is 0");
     *max_tiles = 1 + (nk + kPage - 1) / kPage;
   }
   return 0;
@@ -112,11 +141,23 @@ extern "C" int kitty_decode_attn_split(const kitty_kv_layer* layer, const void* 
   const kitty_kv_layer& L = *layer;
   float* ws_ml = (float*)workspace;
   float* ws_acc = (float*)((uint8_t*)workspace + ws_ml_bytes(B, H_Q, num_splits));
-  if (variant == 0 && decode_mfma_supported(L, H_Q))
-    launch_decode_mfma(L, q, B, H_Q, scaling, ws_ml, ws_acc, num_splits, (hipStream_t)stream);
-  else
+  const hipEvent_t ev0 = g_ev_start, ev1 = g_ev_stop;
+  g_ev_start = g_ev_stop = nullptr;
+  if (variant == 0 && decode_mfma_supported(L, H_Q)) {
+    launch_decode_mfma(L, q, B, H_Q, scaling, ws_ml, ws_acc, num_splits, device_simds(), (hipStream_t)stream, ev0, ev1);
+  } else {
+    if (ev0) (void)hipEventRecord(ev0, (hipStream_t)stream);
     launch_decode_plain(L, q, B, H_Q, scaling, ws_ml, ws_acc, num_splits, (hipStream_t)stream);
+    if (ev1) (void)hipEventRecord(ev1, (hipStream_t)stream);
+  }
   return check_launch("kitty_decode_attn_split");
+}
+
+extern "C" int kitty_profile_next_split(void* start_event, void* stop_event) {
+  KITTY_REQUIRE((start_event == nullptr) == (stop_event == nullptr), KITTY_E_NULL, "two events, or none to cancel");
+  g_ev_start = (hipEvent_t)start_event;
+  g_ev_stop = (hipEvent_t)stop_event;
+  return 0;
 }
 
 extern "C" int kitty_decode_attn_merge(const void* workspace, size_t workspace_bytes, int B, int H_Q, int D,
@@ -136,11 +177,8 @@ extern "C" int kitty_decode_attn(const kitty_kv_layer* layer, const void* q, int
                                  void* stream) {
   int max_tiles = 0;
   if (int rc = check_layer(layer, q, B, H_Q, &max_tiles)) return rc;
-  if (num_splits <= 0) {
-    num_splits = kitty_decode_attn_default_splits(B, layer->H_KV, max_tiles);
-    // sequences of different lengths: more, shorter splits even out the load
-    if (layer->seq_counts && num_splits < 12 && max_tiles >= 48) num_splits = 12;
-  }
+  if (num_splits <= 0)
+    num_splits = kitty_decode_attn_default_splits(B, layer->H_KV, max_tiles, layer->seq_counts != nullptr);
   if (int rc = kitty_decode_attn_split(layer, q, B, H_Q, scaling, workspace, workspace_bytes, num_splits, variant,
                                        stream))
     return rc;

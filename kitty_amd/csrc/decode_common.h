@@ -35,9 +35,28 @@ __device__ inline SeqCounts load_counts(const kitty_kv_layer& L, int b) {
   s.rv = min(max(c[KITTY_CNT_QBUF_V], 0), kPage);
   s.lv = min(max(c[KITTY_CNT_LOCAL_V], 0), kPage);
   s.off = c[KITTY_CNT_LOCAL_OFF] & (kPage - 1);
+  if (L.cache_pages_k <= 0) s.pk = 0;   // no page to read, whatever the counters say
+  if (L.cache_pages_v <= 0) s.pv = 0;
   s.nbody = min(s.pk * kPage + s.rk, s.pv * kPage + s.rv + s.lv);
   s.ntiles = 1 + (s.nbody + kPage - 1) / kPage;
   return s;
+}
+
+// A page id as read from a page table, made safe to dereference.  The counters and tables of a
+// layer may be written by the caller on the device, so the host cannot vouch for them: an id outside
+// [0, cache_pages) (an entry of -1 = no page assigned, or garbage) reads page 0 instead and is noted
+// in `bad`; the output of that sequence is then meaningless, but nothing outside the page arrays is
+// touched.  The note reaches the sequence's status row once, when the kernel is done
+// (report_bad_page): a store next to the table reads would make the compiler treat every later
+// table read as possibly changed by it, and turn the scalar loads of the streaming loops into
+// vector loads with full waits.
+__device__ __forceinline__ int64_t checked_page(int64_t pg, int64_t cache_pages, int& bad) {
+  const bool ok = pg >= 0 && pg < cache_pages;
+  bad |= ok ? 0 : 1;
+  return ok ? pg : 0;
+}
+__device__ __forceinline__ void report_bad_page(const kitty_kv_layer& L, int b, int bad) {
+  if (bad && L.status) L.status[b * KITTY_STATUS_FIELDS + KITTY_STATUS_BAD_PAGE_READ] = 1;
 }
 
 // fp16 row of V for token u of the region that follows the V pages

@@ -40,6 +40,8 @@
 //   = rows 32kg + 8j .. +7, d-tile u = channels {8n + u}; O^T[u][j] = channel 32kg + 8j + u.
 #include <type_traits>
 
+#include <hip/hip_ext.h>
+
 #include "decode_common.h"
 
 // Wave priority while a phase is dominated by matrix instructions / by vector instructions: the
@@ -223,6 +225,7 @@ struct Ctx {
   uint32_t q4[4];       // q[head r][2 lane + {0,1}] of the four heads behind the table rows
   uint32_t qs_rd;       // byte offset of this lane's first read in the q * scale table: row, lane group
   uint32_t qb_rd;       // the same in the table of the high-plane slots
+  mutable int bad_page; // a page id outside the cache was met (checked_page); reported when the wave is done
 };
 
 // ---------------------------------------------------------------------------------------------
@@ -265,7 +268,7 @@ struct KLds {
 template <bool BOOST>
 __device__ __forceinline__ void k_load_regs(const Ctx& x, int page_index, KRegs& kb) {
   const kitty_kv_layer& L = *x.L;
-  const int64_t pg = L.page_table_k[(int64_t)x.b * L.page_table_k_stride_b + page_index];
+  const int64_t pg = checked_page(L.page_table_k[(int64_t)x.b * L.page_table_k_stride_b + page_index], L.cache_pages_k, x.bad_page);
   const uint8_t* page = L.key_cache + pg * L.key_cache_stride_page + (int64_t)x.h * k_head_bytes(BOOST ? 32 : 0);
   const uint8_t* meta = (const uint8_t*)L.key_meta + pg * L.key_meta_stride_page + (int64_t)x.h * kD * 4;
 #pragma unroll
@@ -290,7 +293,7 @@ constexpr int kDmaV = 6;
 template <bool BOOST>
 __device__ __forceinline__ void dma_k(const Ctx& x, int page_index, uint32_t lds) {
   const kitty_kv_layer& L = *x.L;
-  const int64_t pg = L.page_table_k[(int64_t)x.b * L.page_table_k_stride_b + page_index];
+  const int64_t pg = checked_page(L.page_table_k[(int64_t)x.b * L.page_table_k_stride_b + page_index], L.cache_pages_k, x.bad_page);
   const uint8_t* page = L.key_cache + pg * L.key_cache_stride_page + (int64_t)x.h * k_head_bytes(BOOST ? 32 : 0);
   const uint8_t* meta = (const uint8_t*)L.key_meta + pg * L.key_meta_stride_page + (int64_t)x.h * kD * 4;
   const uint32_t off16 = x.lane * 16, off4 = x.lane * 4, off4dup = (x.lane & 31) * 4;
@@ -685,7 +688,7 @@ struct VLds {
 
 __device__ __forceinline__ void v_load_regs(const Ctx& x, int page_index, VRegs& vb) {
   const kitty_kv_layer& L = *x.L;
-  const int64_t pg = L.page_table_v[(int64_t)x.b * L.page_table_v_stride_b + page_index];
+  const int64_t pg = checked_page(L.page_table_v[(int64_t)x.b * L.page_table_v_stride_b + page_index], L.cache_pages_v, x.bad_page);
   const uint8_t* page = L.value_cache + pg * L.value_cache_stride_page + (int64_t)x.h * kVBytes;
   const uint8_t* meta = (const uint8_t*)L.value_meta + pg * L.value_meta_stride_page + (int64_t)x.h * kPage * 4;
   const uint32_t v_off = (32 * x.kg + (x.n & 1)) * kRowBytes + (x.n >> 1) * 4;
@@ -697,7 +700,7 @@ __device__ __forceinline__ void v_load_regs(const Ctx& x, int page_index, VRegs&
 // Global -> LDS loads of one V page-head, byte for byte.
 __device__ __forceinline__ void dma_v(const Ctx& x, int page_index, uint32_t lds) {
   const kitty_kv_layer& L = *x.L;
-  const int64_t pg = L.page_table_v[(int64_t)x.b * L.page_table_v_stride_b + page_index];
+  const int64_t pg = checked_page(L.page_table_v[(int64_t)x.b * L.page_table_v_stride_b + page_index], L.cache_pages_v, x.bad_page);
   const uint8_t* page = L.value_cache + pg * L.value_cache_stride_page + (int64_t)x.h * kVBytes;
   const uint8_t* meta = (const uint8_t*)L.value_meta + pg * L.value_meta_stride_page + (int64_t)x.h * kPage * 4;
   const uint32_t off16 = x.lane * 16;
@@ -895,11 +898,13 @@ __device__ __forceinline__ void wait_vmcnt() {
 template <bool BOOST, bool DMA, bool QUARTER>
 __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(kitty_kv_layer L, const __half* __restrict__ q, int H_Q,
                                                             float scaling, float* __restrict__ ws_ml,
-                                                            float* __restrict__ ws_acc, int num_splits) {
+                                                            float* __restrict__ ws_acc, int num_splits,
+                                                            int n_simds) {
   static_assert(DMA || !QUARTER, "quarter columns are a variant of the LDS-streamed kernel");
   __shared__ WaveLds<DMA, QUARTER> S;
   Ctx x;
   x.L = &L;
+  x.bad_page = 0;
   x.b = blockIdx.z;
   x.h = blockIdx.y;
   const int split = blockIdx.x;
@@ -1019,11 +1024,11 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(kitty_kv_layer L, co
       if (t0 + 1 < t1) dma_k<BOOST>(x, t0 + 1, lk1);
       dma_v(x, t0, lv);
       // Of the two waves that share a SIMD the older one wins arbitration, and it is 8 % faster per
-      // tile.  When the launch is a single round (at most two workgroups per SIMD of the 256 CUs),
+      // tile.  When the launch is a single round (at most two workgroups per SIMD of the device),
       // the workgroups dispatched after every SIMD has one are the younger ones: they raise their
       // priority by one level after the first quarter of their range, which evens out the finishes.
       // (Two copies of the loop: the conditional priorities cost the other launches 1.5 %.)
-      constexpr uint32_t kSimds = 256 * 4;
+      const uint32_t kSimds = (uint32_t)n_simds;
       const uint32_t n_wg = gridDim.x * gridDim.y * gridDim.z;
       const uint32_t lin_id = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
       const bool young = n_wg <= 2 * kSimds && lin_id >= kSimds;
@@ -1129,6 +1134,7 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(kitty_kv_layer L, co
   }
   to_true_units(A);
 
+  report_bad_page(L, x.b, x.bad_page);
   // ---- partial of this split: columns n < G are the G heads -----------------------------------
   float l = A.lz[0], z = A.lz[1];
   if constexpr (QUARTER) {
@@ -1171,14 +1177,24 @@ bool decode_mfma_supported(const kitty_kv_layer& L, int H_Q) {
   return (L.D_BOOSTED == 32 || L.D_BOOSTED == 0) && L.D == kD && L.PAGE_SIZE == kPage && H_Q / L.H_KV <= 16;
 }
 
+// ev_start / ev_stop (both or neither): events attached to the kernel's own dispatch, which then hold
+// the moments the kernel began and ended on the device (what a kernel trace reports) rather than the
+// moments the host enqueued around it.
 void launch_decode_mfma(const kitty_kv_layer& L, const void* q, int B, int H_Q, float scaling, float* ws_ml,
-                        float* ws_acc, int num_splits, hipStream_t stream) {
+                        float* ws_acc, int num_splits, int n_simds, hipStream_t stream, hipEvent_t ev_start,
+                        hipEvent_t ev_stop) {
   const dim3 grid(num_splits, L.H_KV, B), block(64);
   const int G = H_Q / L.H_KV;
   const bool boost = L.D_BOOSTED == 32, dma = G <= 8, quarter = G <= 4;
-#define KITTY_LAUNCH(BOOST, DMA, QUARTER)                                                                   \
-  hipLaunchKernelGGL((decode_mfma_kernel<BOOST, DMA, QUARTER>), grid, block, 0, stream, L, (const __half*)q, H_Q, \
-                     scaling, ws_ml, ws_acc, num_splits)
+#define KITTY_LAUNCH(BOOST, DMA, QUARTER)                                                                        \
+  do {                                                                                                           \
+    if (ev_start)                                                                                                \
+      hipExtLaunchKernelGGL((decode_mfma_kernel<BOOST, DMA, QUARTER>), grid, block, 0, stream, ev_start, ev_stop, 0, \
+                            L, (const __half*)q, H_Q, scaling, ws_ml, ws_acc, num_splits, n_simds);              \
+    else                                                                                                         \
+      hipLaunchKernelGGL((decode_mfma_kernel<BOOST, DMA, QUARTER>), grid, block, 0, stream, L, (const __half*)q,  \
+                         H_Q, scaling, ws_ml, ws_acc, num_splits, n_simds);                                      \
+  } while (0)
   if (boost && quarter) KITTY_LAUNCH(true, true, true);
   else if (boost && dma) KITTY_LAUNCH(true, true, false);
   else if (boost) KITTY_LAUNCH(true, false, false);

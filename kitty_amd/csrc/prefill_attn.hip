@@ -132,6 +132,7 @@ struct Prefill {
   int n_body;        // body tiles
   int n_tiles;       // sink + body + chunk tiles actually walked
   int first_body, first_chunk;
+  mutable int bad_page = 0;   // a page id outside the cache was met (checked_page)
 
   __device__ TileSrc tile(int t) const {
     TileSrc s;
@@ -150,7 +151,7 @@ struct Prefill {
       const int i = t - first_body;
       s.ntok = min(kPage, c.nbody - i * kPage);
       if (i < c.pk) {
-        const int64_t pg = L.page_table_k[(int64_t)b * L.page_table_k_stride_b + i];
+        const int64_t pg = checked_page(L.page_table_k[(int64_t)b * L.page_table_k_stride_b + i], L.cache_pages_k, bad_page);
         s.k_kind = SRC_PACKED;
         s.k_ptr = L.key_cache + pg * L.key_cache_stride_page + (int64_t)h * k_head_bytes(L.D_BOOSTED);
         s.k_meta = (const uint8_t*)L.key_meta + pg * L.key_meta_stride_page + (int64_t)h * kD * 4;
@@ -160,7 +161,7 @@ struct Prefill {
         s.k_stride = kD * 2;
       }
       if (i < c.pv) {
-        const int64_t pg = L.page_table_v[(int64_t)b * L.page_table_v_stride_b + i];
+        const int64_t pg = checked_page(L.page_table_v[(int64_t)b * L.page_table_v_stride_b + i], L.cache_pages_v, bad_page);
         s.v_kind = SRC_PACKED;
         s.v_ptr = L.value_cache + pg * L.value_cache_stride_page + (int64_t)h * kVBytes;
         s.v_meta = (const uint8_t*)L.value_meta + pg * L.value_meta_stride_page + (int64_t)h * kPage * 4;
@@ -564,6 +565,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(kWaves
       *(__half2*)(orow + 16 * ct + 2 * kg + 8) = __floats2half2_rn(o[1], o[3]);
     }
   }
+  if (tid == 0) report_bad_page(L, b, P.bad_page);
 }
 
 }  // namespace

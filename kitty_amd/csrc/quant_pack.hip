@@ -120,11 +120,16 @@ __device__ __forceinline__ uint32_t gather_fields(uint32_t n) {
 }
 
 // One K page of one head.  MODE 0: slot map given.  MODE 1: selection fused, then quantize.
-// MODE 2: selection only.  src: the page's first token row of this head; slot_in / slot_out: 128
-// bytes (or NULL); dst: the page-head in the cache, meta_dst: its 128 (scale, zero) pairs.
-// Called by all 256 threads of a workgroup.
-template <int MODE>
-__device__ __forceinline__ void quant_k_page(const uint8_t* __restrict__ src_page, int64_t stride_t, int d_boost,
+// MODE 2: selection only.  row_of(t): the 256-byte row of token t (0..127) of this head; slot_in /
+// slot_out: 128 bytes (or NULL); dst: the page-head in the cache, meta_dst: its 128 (scale, zero)
+// pairs.  Called by all 256 threads of a workgroup.
+struct StridedRows {   // the rows of a page that lies in one tensor
+  const uint8_t* base;
+  int64_t stride_t;
+  __device__ __forceinline__ const uint8_t* operator()(int t) const { return base + (int64_t)t * stride_t; }
+};
+template <int MODE, class ROWS>
+__device__ __forceinline__ void quant_k_page(const ROWS row_of, int d_boost,
                                              const uint8_t* __restrict__ slot_in, uint8_t* __restrict__ slot_out,
                                              uint8_t* __restrict__ dst, uint8_t* __restrict__ meta_dst) {
   const int tid = threadIdx.x;
@@ -148,10 +153,9 @@ __device__ __forceinline__ void quant_k_page(const uint8_t* __restrict__ src_pag
   static_assert(sizeof(s_pmin) >= kD * 32, "the low plane reuses the minima");
   uint8_t* const s_lo = (uint8_t*)&s_pmin[0][0];
 
-  const uint8_t* src = src_page + (int64_t)(tg * 8) * stride_t + c8 * 16;
   uint4 rows[8];
 #pragma unroll
-  for (int r = 0; r < 8; ++r) rows[r] = nt_load16(src + (int64_t)r * stride_t);
+  for (int r = 0; r < 8; ++r) rows[r] = nt_load16(row_of(tg * 8 + r) + c8 * 16);
 
   // this thread's 8 tokens x 8 channels as floats, and per channel the partial min / max (/ sum
   // of |x|: exact in fp64, every term is a multiple of 2^-24 below 2^16)
@@ -269,7 +273,7 @@ __global__ __launch_bounds__(256) void quant_pack_k_kernel(
     const uint8_t* __restrict__ slot_map_in, uint8_t* __restrict__ slot_map_out, int pages,
     const int64_t* __restrict__ page_table, int64_t pt_stride_b, int page_offset,
     uint8_t* __restrict__ cache, int64_t cache_stride_page,
-    uint8_t* __restrict__ meta, int64_t meta_stride_page, int64_t cache_pages) {
+    uint8_t* __restrict__ meta, int64_t meta_stride_page, int64_t cache_pages, int32_t* __restrict__ status) {
   const int p = blockIdx.x, h = blockIdx.y, b = blockIdx.z, H = gridDim.y;
   const uint8_t* src = key + (int64_t)b * stride_b + (int64_t)h * stride_h + (int64_t)(t_offset + p * kPage) * stride_t;
   const int64_t slot_off = (((int64_t)b * H + h) * pages + p) * kD;
@@ -277,27 +281,29 @@ __global__ __launch_bounds__(256) void quant_pack_k_kernel(
   uint8_t* mdst = nullptr;
   if (MODE != 2) {
     const int64_t pg = page_table[(int64_t)b * pt_stride_b + page_offset + p];
-    if (pg < 0 || pg >= cache_pages) return;   // never write outside the cache
+    if (pg < 0 || pg >= cache_pages) {   // never write outside the cache; leave a record instead
+      if (status && threadIdx.x == 0) status[b * KITTY_STATUS_FIELDS + KITTY_STATUS_BAD_PAGE_WRITE] = 1;
+      return;
+    }
     dst = cache + pg * cache_stride_page + (int64_t)h * k_head_bytes(d_boost);
     mdst = meta + pg * meta_stride_page + (int64_t)h * kD * 4;
   }
-  quant_k_page<MODE>(src, stride_t, d_boost, slot_map_in ? slot_map_in + slot_off : nullptr,
+  quant_k_page<MODE>(StridedRows{src, stride_t}, d_boost, slot_map_in ? slot_map_in + slot_off : nullptr,
                      slot_map_out ? slot_map_out + slot_off : nullptr, dst, mdst);
 }
 
 // One V page of one head: 256 threads, 8 consecutive lanes share a token (16 channels each), 4
-// tokens per thread.  src: the page's first token row of this head.
-__device__ __forceinline__ void quant_v_page(const uint8_t* __restrict__ src_page, int64_t stride_t,
-                                             uint8_t* __restrict__ dst, uint8_t* __restrict__ mdst) {
+// tokens per thread.  row_of(t): the 256-byte row of token t of this head.
+template <class ROWS>
+__device__ __forceinline__ void quant_v_page(const ROWS row_of, uint8_t* __restrict__ dst, uint8_t* __restrict__ mdst) {
   const int tid = threadIdx.x;
   const int cg = tid & 7;
-  const uint8_t* src = src_page + cg * 32;
   uint4 la[4], lc[4];   // all eight loads of the thread are in flight before the first is used
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
-    const int t = (tid >> 3) + 32 * i;
-    la[i] = nt_load16(src + (int64_t)t * stride_t);
-    lc[i] = nt_load16(src + (int64_t)t * stride_t + 16);
+    const uint8_t* src = row_of((tid >> 3) + 32 * i) + cg * 32;
+    la[i] = nt_load16(src);
+    lc[i] = nt_load16(src + 16);
   }
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
@@ -341,12 +347,16 @@ __global__ __launch_bounds__(256) void quant_pack_v_kernel(
     int t_offset,
     const int64_t* __restrict__ page_table, int64_t pt_stride_b, int page_offset,
     uint8_t* __restrict__ cache, int64_t cache_stride_page,
-    uint8_t* __restrict__ meta, int64_t meta_stride_page, int64_t cache_pages) {
+    uint8_t* __restrict__ meta, int64_t meta_stride_page, int64_t cache_pages, int32_t* __restrict__ status) {
   const int p = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
   const int64_t pg = page_table[(int64_t)b * pt_stride_b + page_offset + p];
-  if (pg < 0 || pg >= cache_pages) return;
-  quant_v_page(value + (int64_t)b * stride_b + (int64_t)h * stride_h + (int64_t)(t_offset + p * kPage) * stride_t,
-               stride_t, cache + pg * cache_stride_page + (int64_t)h * kVBytes,
+  if (pg < 0 || pg >= cache_pages) {
+    if (status && threadIdx.x == 0) status[b * KITTY_STATUS_FIELDS + KITTY_STATUS_BAD_PAGE_WRITE] = 1;
+    return;
+  }
+  quant_v_page(StridedRows{value + (int64_t)b * stride_b + (int64_t)h * stride_h + (int64_t)(t_offset + p * kPage) * stride_t,
+                           stride_t},
+               cache + pg * cache_stride_page + (int64_t)h * kVBytes,
                meta + pg * meta_stride_page + (int64_t)h * kPage * 4);
 }
 
@@ -355,9 +365,40 @@ __global__ __launch_bounds__(256) void quant_pack_v_kernel(
 // KITTY_CNT_* fields).  The state machine is KittyCache.update's decode branch (kitty.py:97-123)
 // and quantize_decode (kitty.py:194-236), per sequence instead of per batch.
 // ---------------------------------------------------------------------------------------------
+__device__ __forceinline__ void bump_status(const kitty_kv_layer& L, int b, int field, int by) {
+  if (L.status) L.status[b * KITTY_STATUS_FIELDS + field] += by;   // one writer per sequence and launch
+}
+
+// k * cos + rotate_half(k) * sin for 4 channels starting at c, as fp16 tensor arithmetic evaluates it:
+// each product and the sum rounded to fp16 (the product of two fp16 numbers is exact in fp32, and so
+// is the sum of two, up to one rounding that rounding again to fp16 never alters).  Contraction is
+// switched off: left on, the compiler folds the second product and the sum into one fp16 FMA, which
+// skips a rounding the tensor expression has.
+__device__ __forceinline__ uint2 rope4(uint2 own, uint2 partner, uint2 cs, uint2 sn, bool upper) {
+#pragma clang fp contract(off)
+  const uint32_t o[2] = {own.x, own.y}, q[2] = {partner.x, partner.y}, c[2] = {cs.x, cs.y}, s[2] = {sn.x, sn.y};
+  uint32_t r[2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    uint16_t out[2];
+#pragma unroll
+    for (int k = 0; k < 2; ++k) {
+      const float x = h2f((uint16_t)(o[i] >> (16 * k))), y = h2f((uint16_t)(q[i] >> (16 * k)));
+      const float cc = h2f((uint16_t)(c[i] >> (16 * k))), ss = h2f((uint16_t)(s[i] >> (16 * k)));
+      const float a = __half2float(__float2half_rn(x * cc));
+      const float t = __half2float(__float2half_rn((upper ? y : -y) * ss));   // rotate_half: (-x2, x1)
+      out[k] = __half_as_ushort(__float2half_rn(a + t));
+    }
+    r[i] = (uint32_t)out[0] | ((uint32_t)out[1] << 16);
+  }
+  return uint2{r[0], r[1]};
+}
+
+template <bool ROPE>
 __global__ __launch_bounds__(256) void append_token_kernel(kitty_kv_layer L, const uint8_t* __restrict__ k_new,
                                                            const uint8_t* __restrict__ v_new, int64_t stride_b,
-                                                           int64_t stride_h) {
+                                                           int64_t stride_h, const uint8_t* __restrict__ rope_cos,
+                                                           const uint8_t* __restrict__ rope_sin, int64_t rope_stride_b) {
   const int b = blockIdx.x;
   int32_t* cnt = const_cast<int32_t*>(L.seq_counts) + b * KITTY_SEQ_COUNT_FIELDS;
   if (cnt[KITTY_CNT_FLAGS] & KITTY_SEQ_INACTIVE) return;   // the whole block: nobody reaches the barrier
@@ -367,45 +408,54 @@ __global__ __launch_bounds__(256) void append_token_kernel(kitty_kv_layer L, con
   // a full Q-buffer means the caller skipped a flush: drop the token rather than write out of bounds
   const bool ok = to_sink || (rk < kPage && (lv < kPage || rv < kPage));
   __syncthreads();   // every thread has read the counters before thread 0 rewrites them
-  if (ok) {
-    for (int i = threadIdx.x; i < L.H_KV * 32; i += blockDim.x) {
-      const int h = i >> 5, part = (i & 31) * 8;   // 8 bytes = 4 channels
-      const uint2 kk = *(const uint2*)(k_new + (int64_t)b * stride_b + (int64_t)h * stride_h + part);
-      const uint2 vv = *(const uint2*)(v_new + (int64_t)b * stride_b + (int64_t)h * stride_h + part);
-      if (to_sink) {
-        const int64_t o = (int64_t)b * L.sink_stride_b + (int64_t)h * L.sink_stride_h + (int64_t)sink * (kD * 2) + part;
-        *(uint2*)((uint8_t*)L.sink_k + o) = kk;
-        *(uint2*)((uint8_t*)L.sink_v + o) = vv;
-      } else {
-        const int64_t w = (int64_t)b * L.win_stride_b + (int64_t)h * L.win_stride_h + part;
-        *(uint2*)((uint8_t*)L.qbuf_k + w + (int64_t)rk * (kD * 2)) = kk;
-        if (lv < kPage) {
-          *(uint2*)((uint8_t*)L.local_v + w + (int64_t)lv * (kD * 2)) = vv;
-        } else {   // ring full: its oldest row moves to the V Q-buffer, the new one takes the slot
-          uint2* slot = (uint2*)((uint8_t*)L.local_v + w + (int64_t)off * (kD * 2));
-          *(uint2*)((uint8_t*)L.qbuf_v + w + (int64_t)rv * (kD * 2)) = *slot;
-          *slot = vv;
-        }
+  if (!ok) {
+    if (threadIdx.x == 0) bump_status(L, b, KITTY_STATUS_TOKENS_DROPPED, 1);
+    return;
+  }
+  for (int i = threadIdx.x; i < L.H_KV * 32; i += blockDim.x) {
+    const int h = i >> 5, part = (i & 31) * 8;   // 8 bytes = 4 channels
+    const uint8_t* krow = k_new + (int64_t)b * stride_b + (int64_t)h * stride_h;
+    uint2 kk = *(const uint2*)(krow + part);
+    if (ROPE) {
+      const uint2 partner = *(const uint2*)(krow + (part ^ (kD)));   // the channel 64 away: 128 bytes
+      const uint2 cs = *(const uint2*)(rope_cos + (int64_t)b * rope_stride_b + part);
+      const uint2 sn = *(const uint2*)(rope_sin + (int64_t)b * rope_stride_b + part);
+      kk = rope4(kk, partner, cs, sn, part >= kD);
+    }
+    const uint2 vv = *(const uint2*)(v_new + (int64_t)b * stride_b + (int64_t)h * stride_h + part);
+    if (to_sink) {
+      const int64_t o = (int64_t)b * L.sink_stride_b + (int64_t)h * L.sink_stride_h + (int64_t)sink * (kD * 2) + part;
+      *(uint2*)((uint8_t*)L.sink_k + o) = kk;
+      *(uint2*)((uint8_t*)L.sink_v + o) = vv;
+    } else {
+      const int64_t w = (int64_t)b * L.win_stride_b + (int64_t)h * L.win_stride_h + part;
+      *(uint2*)((uint8_t*)L.qbuf_k + w + (int64_t)rk * (kD * 2)) = kk;
+      if (lv < kPage) {
+        *(uint2*)((uint8_t*)L.local_v + w + (int64_t)lv * (kD * 2)) = vv;
+      } else {   // ring full: its oldest row moves to the V Q-buffer, the new one takes the slot
+        uint2* slot = (uint2*)((uint8_t*)L.local_v + w + (int64_t)off * (kD * 2));
+        *(uint2*)((uint8_t*)L.qbuf_v + w + (int64_t)rv * (kD * 2)) = *slot;
+        *slot = vv;
       }
     }
-    if (threadIdx.x == 0) {
-      if (to_sink) {
-        cnt[KITTY_CNT_SINK] = sink + 1;
+  }
+  if (threadIdx.x == 0) {
+    if (to_sink) {
+      cnt[KITTY_CNT_SINK] = sink + 1;
+    } else {
+      cnt[KITTY_CNT_QBUF_K] = rk + 1;
+      if (lv < kPage) {
+        cnt[KITTY_CNT_LOCAL_V] = lv + 1;
       } else {
-        cnt[KITTY_CNT_QBUF_K] = rk + 1;
-        if (lv < kPage) {
-          cnt[KITTY_CNT_LOCAL_V] = lv + 1;
-        } else {
-          cnt[KITTY_CNT_QBUF_V] = rv + 1;
-          cnt[KITTY_CNT_LOCAL_OFF] = (off + 1) & (kPage - 1);
-        }
+        cnt[KITTY_CNT_QBUF_V] = rv + 1;
+        cnt[KITTY_CNT_LOCAL_OFF] = (off + 1) & (kPage - 1);
       }
     }
   }
 }
 
 // blockIdx.z = 0: the K Q-buffer of (b, h) if it is full; 1: the V Q-buffer.
-__global__ __launch_bounds__(256) void flush_full_kernel(kitty_kv_layer L, int64_t cache_pages) {
+__global__ __launch_bounds__(256) void flush_full_kernel(kitty_kv_layer L) {
   const int h = blockIdx.x, b = blockIdx.y;
   const int32_t* cnt = L.seq_counts + b * KITTY_SEQ_COUNT_FIELDS;
   const int64_t w = (int64_t)b * L.win_stride_b + (int64_t)h * L.win_stride_h;
@@ -414,43 +464,236 @@ __global__ __launch_bounds__(256) void flush_full_kernel(kitty_kv_layer L, int64
     const int pk = cnt[KITTY_CNT_PAGES_K];
     if (cnt[KITTY_CNT_QBUF_K] != kPage || pk < 0 || pk >= L.MAX_PAGE) return;
     const int64_t pg = L.page_table_k[(int64_t)b * L.page_table_k_stride_b + pk];
-    if (pg < 0 || pg >= cache_pages) return;
-    quant_k_page<1>((const uint8_t*)L.qbuf_k + w, kD * 2, L.D_BOOSTED, nullptr, nullptr,
+    if (pg < 0 || pg >= L.cache_pages_k) return;
+    quant_k_page<1>(StridedRows{(const uint8_t*)L.qbuf_k + w, kD * 2}, L.D_BOOSTED, nullptr, nullptr,
                     const_cast<uint8_t*>(L.key_cache) + pg * L.key_cache_stride_page + (int64_t)h * k_head_bytes(L.D_BOOSTED),
                     (uint8_t*)L.key_meta + pg * L.key_meta_stride_page + (int64_t)h * kD * 4);
   } else {
     const int pv = cnt[KITTY_CNT_PAGES_V];
     if (cnt[KITTY_CNT_QBUF_V] != kPage || pv < 0 || pv >= L.MAX_PAGE) return;
     const int64_t pg = L.page_table_v[(int64_t)b * L.page_table_v_stride_b + pv];
-    if (pg < 0 || pg >= cache_pages) return;
-    quant_v_page((const uint8_t*)L.qbuf_v + w, kD * 2,
+    if (pg < 0 || pg >= L.cache_pages_v) return;
+    quant_v_page(StridedRows{(const uint8_t*)L.qbuf_v + w, kD * 2},
                  const_cast<uint8_t*>(L.value_cache) + pg * L.value_cache_stride_page + (int64_t)h * kVBytes,
                  (uint8_t*)L.value_meta + pg * L.value_meta_stride_page + (int64_t)h * kPage * 4);
   }
 }
 
 // after flush_full_kernel: the flushed Q-buffers are empty, their pages count.  The conditions are
-// those under which flush_full_kernel wrote the page.
-__global__ void advance_counts_kernel(kitty_kv_layer L, int B, int64_t cache_pages) {
+// those under which flush_full_kernel wrote the page; a full Q-buffer that stays is recorded.
+__global__ void advance_counts_kernel(kitty_kv_layer L, int B) {
   const int b = blockIdx.x * blockDim.x + threadIdx.x;
   if (b >= B) return;
   int32_t* cnt = const_cast<int32_t*>(L.seq_counts) + b * KITTY_SEQ_COUNT_FIELDS;
   if (cnt[KITTY_CNT_FLAGS] & KITTY_SEQ_INACTIVE) return;
   const int pk = cnt[KITTY_CNT_PAGES_K], pv = cnt[KITTY_CNT_PAGES_V];
-  if (cnt[KITTY_CNT_QBUF_K] == kPage && pk >= 0 && pk < L.MAX_PAGE) {
-    const int64_t pg = L.page_table_k[(int64_t)b * L.page_table_k_stride_b + pk];
-    if (pg >= 0 && pg < cache_pages) {
+  int skipped = 0;
+  bool bad = false;
+  if (cnt[KITTY_CNT_QBUF_K] == kPage) {
+    int64_t pg = -1;
+    if (pk >= 0 && pk < L.MAX_PAGE) pg = L.page_table_k[(int64_t)b * L.page_table_k_stride_b + pk];
+    if (pg >= 0 && pg < L.cache_pages_k) {
       cnt[KITTY_CNT_PAGES_K] = pk + 1;
       cnt[KITTY_CNT_QBUF_K] = 0;
+    } else {
+      ++skipped;
+      bad |= pg != -1;
     }
   }
-  if (cnt[KITTY_CNT_QBUF_V] == kPage && pv >= 0 && pv < L.MAX_PAGE) {
-    const int64_t pg = L.page_table_v[(int64_t)b * L.page_table_v_stride_b + pv];
-    if (pg >= 0 && pg < cache_pages) {
+  if (cnt[KITTY_CNT_QBUF_V] == kPage) {
+    int64_t pg = -1;
+    if (pv >= 0 && pv < L.MAX_PAGE) pg = L.page_table_v[(int64_t)b * L.page_table_v_stride_b + pv];
+    if (pg >= 0 && pg < L.cache_pages_v) {
       cnt[KITTY_CNT_PAGES_V] = pv + 1;
       cnt[KITTY_CNT_QBUF_V] = 0;
+    } else {
+      ++skipped;
+      bad |= pg != -1;
     }
   }
+  if (skipped) bump_status(L, b, KITTY_STATUS_FLUSH_SKIPPED, skipped);
+  if (bad && L.status) L.status[b * KITTY_STATUS_FIELDS + KITTY_STATUS_BAD_PAGE_WRITE] = 1;
+}
+
+// ---------------------------------------------------------------------------------------------
+// A chunk of T tokens per sequence in one go, with the state T single steps would leave.
+//
+// Per sequence the new rows (after those that still go to the sink) extend two streams of rows
+// waiting to be packed.  K: [ Q_Buffer_K rows | chunk rows ].  V: [ Q_Buffer_V rows | the rows the
+// ring gives up, oldest first | the chunk rows that pass through the ring and out again ]; the ring
+// keeps the newest 128 rows.  Every full group of 128 stream rows is a page, quantized straight from
+// wherever its rows lie; what is left of a stream is the new Q-buffer content.
+// ---------------------------------------------------------------------------------------------
+struct ChunkPlan {
+  bool active, ok;
+  int sink, pk, rk, pv, rv, lv, off;   // the sequence before the chunk
+  int a, n;          // chunk rows that go to the sink / past it
+  int npk, npv;      // new pages
+  int e, er;         // rows leaving the ring (e), of which rows that were in it before (er)
+  int rk2, rv2, lv2, off2;
+};
+
+// the counters part; `ok` still lacks the page ids (chunk_pages_ok)
+__device__ inline ChunkPlan chunk_plan(const kitty_kv_layer& L, int b, int T) {
+  const int32_t* cnt = L.seq_counts + b * KITTY_SEQ_COUNT_FIELDS;
+  ChunkPlan p;
+  p.active = !(cnt[KITTY_CNT_FLAGS] & KITTY_SEQ_INACTIVE);
+  p.sink = cnt[KITTY_CNT_SINK]; p.pk = cnt[KITTY_CNT_PAGES_K]; p.rk = cnt[KITTY_CNT_QBUF_K];
+  p.pv = cnt[KITTY_CNT_PAGES_V]; p.rv = cnt[KITTY_CNT_QBUF_V]; p.lv = cnt[KITTY_CNT_LOCAL_V];
+  p.off = cnt[KITTY_CNT_LOCAL_OFF] & (kPage - 1);
+  const bool sane = p.sink >= 0 && p.sink <= L.S && p.pk >= 0 && p.pv >= 0 && p.rk >= 0 && p.rv >= 0 && p.lv >= 0 &&
+                    p.lv <= kPage && p.rk <= kPage && p.rv <= kPage;
+  p.a = sane ? min(L.S - p.sink, T) : 0;
+  p.n = T - p.a;
+  p.npk = (p.rk + p.n) / kPage;
+  p.rk2 = (p.rk + p.n) % kPage;
+  p.lv2 = min(kPage, p.lv + p.n);
+  p.e = p.lv + p.n - p.lv2;
+  p.er = min(p.e, p.lv);
+  p.npv = (p.rv + p.e) / kPage;
+  p.rv2 = (p.rv + p.e) % kPage;
+  p.off2 = (p.off + p.e) & (kPage - 1);
+  // a Q-buffer that is still full (a flush found no page) takes nothing more, as in single steps
+  p.ok = sane && (p.n == 0 || (p.rk < kPage && p.rv < kPage)) && p.pk + p.npk <= L.MAX_PAGE &&
+         p.pv + p.npv <= L.MAX_PAGE;
+  return p;
+}
+// every page the plan wants to write has a valid id; called by all threads of a block
+__device__ inline bool chunk_pages_ok(const kitty_kv_layer& L, int b, const ChunkPlan& p) {
+  int bad = 0;
+  if (p.ok) {
+    for (int i = threadIdx.x; i < p.npk + p.npv; i += blockDim.x) {
+      const bool k = i < p.npk;
+      const int64_t pg = k ? L.page_table_k[(int64_t)b * L.page_table_k_stride_b + p.pk + i]
+                           : L.page_table_v[(int64_t)b * L.page_table_v_stride_b + p.pv + (i - p.npk)];
+      bad |= pg < 0 || pg >= (k ? L.cache_pages_k : L.cache_pages_v);
+    }
+  }
+  return p.ok && !__syncthreads_or(bad);
+}
+
+struct ChunkSrc {
+  const uint8_t* k;   // chunk rows of this (b, h): row t at k + t * stride_t
+  const uint8_t* v;
+  int64_t stride_t;
+};
+// row s of the K stream / of the V stream of one (b, h)
+struct KStreamRows {
+  const uint8_t* qbuf; const uint8_t* chunk; int64_t stride_t; int rk, first;
+  __device__ __forceinline__ const uint8_t* operator()(int t) const {
+    const int s = first + t;
+    return s < rk ? qbuf + (int64_t)s * (kD * 2) : chunk + (int64_t)(s - rk) * stride_t;
+  }
+};
+struct VStreamRows {
+  const uint8_t* qbuf; const uint8_t* ring; const uint8_t* chunk; int64_t stride_t; int rv, er, off, first;
+  __device__ __forceinline__ const uint8_t* operator()(int t) const {
+    const int s = first + t;
+    if (s < rv) return qbuf + (int64_t)s * (kD * 2);
+    if (s < rv + er) return ring + (int64_t)((off + s - rv) & (kPage - 1)) * (kD * 2);
+    return chunk + (int64_t)(s - rv - er) * stride_t;
+  }
+};
+
+// grid (2 * max_pages, H_KV, B): blockIdx.x < max_pages: new K page blockIdx.x, else new V page
+__global__ __launch_bounds__(256) void chunk_quant_kernel(kitty_kv_layer L, const uint8_t* __restrict__ k_new,
+                                                          const uint8_t* __restrict__ v_new, int64_t stride_b,
+                                                          int64_t stride_h, int64_t stride_t, int T, int max_pages) {
+  const int h = blockIdx.y, b = blockIdx.z;
+  const bool vside = (int)blockIdx.x >= max_pages;
+  const int p = vside ? blockIdx.x - max_pages : blockIdx.x;
+  const ChunkPlan c = chunk_plan(L, b, T);
+  if (!c.active || p >= (vside ? c.npv : c.npk)) return;        // uniform over the block
+  if (!chunk_pages_ok(L, b, c)) return;
+  const int64_t w = (int64_t)b * L.win_stride_b + (int64_t)h * L.win_stride_h;
+  const int64_t src = (int64_t)b * stride_b + (int64_t)h * stride_h + (int64_t)c.a * stride_t;
+  if (!vside) {
+    const int64_t pg = L.page_table_k[(int64_t)b * L.page_table_k_stride_b + c.pk + p];
+    quant_k_page<1>(KStreamRows{(const uint8_t*)L.qbuf_k + w, k_new + src, stride_t, c.rk, p * kPage}, L.D_BOOSTED,
+                    nullptr, nullptr,
+                    const_cast<uint8_t*>(L.key_cache) + pg * L.key_cache_stride_page + (int64_t)h * k_head_bytes(L.D_BOOSTED),
+                    (uint8_t*)L.key_meta + pg * L.key_meta_stride_page + (int64_t)h * kD * 4);
+  } else {
+    const int64_t pg = L.page_table_v[(int64_t)b * L.page_table_v_stride_b + c.pv + p];
+    quant_v_page(VStreamRows{(const uint8_t*)L.qbuf_v + w, (const uint8_t*)L.local_v + w, v_new + src, stride_t, c.rv,
+                             c.er, c.off, p * kPage},
+                 const_cast<uint8_t*>(L.value_cache) + pg * L.value_cache_stride_page + (int64_t)h * kVBytes,
+                 (uint8_t*)L.value_meta + pg * L.value_meta_stride_page + (int64_t)h * kPage * 4);
+  }
+}
+
+// grid (H_KV, B): the fp16 rows of one (b, h) after the chunk - sink rows, what is left of the two
+// streams (the new Q-buffer contents) and the ring.  Runs after chunk_quant_kernel, which reads the
+// old Q-buffers and ring.  Rows are moved by 16 lanes x 16 bytes.
+__global__ __launch_bounds__(256) void chunk_rows_kernel(kitty_kv_layer L, const uint8_t* __restrict__ k_new,
+                                                         const uint8_t* __restrict__ v_new, int64_t stride_b,
+                                                         int64_t stride_h, int64_t stride_t, int T) {
+  __shared__ uint4 s_stage[kPage][16];   // ring rows on their way to the V Q-buffer
+  const int h = blockIdx.x, b = blockIdx.y;
+  const ChunkPlan c = chunk_plan(L, b, T);
+  if (!c.active) return;
+  if (!chunk_pages_ok(L, b, c)) return;
+  const int piece = threadIdx.x & 15, r0 = threadIdx.x >> 4;
+  const int64_t w = (int64_t)b * L.win_stride_b + (int64_t)h * L.win_stride_h;
+  const uint8_t* ksrc = k_new + (int64_t)b * stride_b + (int64_t)h * stride_h;
+  const uint8_t* vsrc = v_new + (int64_t)b * stride_b + (int64_t)h * stride_h;
+  auto row16 = [&](const uint8_t* p) { return ((const uint4*)p)[piece]; };
+  // sink
+  {
+    const int64_t so = (int64_t)b * L.sink_stride_b + (int64_t)h * L.sink_stride_h;
+    for (int i = r0; i < c.a; i += 16) {
+      ((uint4*)((uint8_t*)L.sink_k + so + (int64_t)(c.sink + i) * (kD * 2)))[piece] = row16(ksrc + (int64_t)i * stride_t);
+      ((uint4*)((uint8_t*)L.sink_v + so + (int64_t)(c.sink + i) * (kD * 2)))[piece] = row16(vsrc + (int64_t)i * stride_t);
+    }
+  }
+  if (c.n == 0) return;
+  ksrc += (int64_t)c.a * stride_t;
+  vsrc += (int64_t)c.a * stride_t;
+  // K: stream rows 128 npk + i -> Q_Buffer_K[i]; rows that already sit there stay (no page was cut)
+  for (int i = (c.npk ? 0 : c.rk) + r0; i < c.rk2; i += 16)
+    ((uint4*)((uint8_t*)L.qbuf_k + w + (int64_t)i * (kD * 2)))[piece] =
+        row16(ksrc + (int64_t)(c.npk * kPage + i - c.rk) * stride_t);
+  // V: the same, but a stream row may lie in the ring, whose slots are about to be overwritten:
+  // those rows go through LDS
+  const int v_first = c.npv * kPage;
+  const int lo = c.npv ? 0 : c.rv;
+  for (int i = lo + r0; i < c.rv2; i += 16) {
+    const int s = v_first + i;
+    if (s >= c.rv && s < c.rv + c.er)
+      s_stage[i][piece] = row16((const uint8_t*)L.local_v + w + (int64_t)((c.off + s - c.rv) & (kPage - 1)) * (kD * 2));
+  }
+  __syncthreads();
+  for (int i = lo + r0; i < c.rv2; i += 16) {
+    const int s = v_first + i;
+    const uint4 v = (s < c.rv + c.er) ? s_stage[i][piece] : row16(vsrc + (int64_t)(s - c.rv - c.er) * stride_t);
+    ((uint4*)((uint8_t*)L.qbuf_v + w + (int64_t)i * (kD * 2)))[piece] = v;
+  }
+  // ring: the chunk rows that stay take the slots single steps would have given them
+  const int base = c.lv < kPage ? c.lv : c.off;
+  for (int j = c.e - c.er + r0; j < c.n; j += 16)
+    ((uint4*)((uint8_t*)L.local_v + w + (int64_t)((base + j) & (kPage - 1)) * (kD * 2)))[piece] =
+        row16(vsrc + (int64_t)j * stride_t);
+}
+
+// one block per sequence, after the two kernels above have read the old counters
+__global__ __launch_bounds__(64) void chunk_advance_kernel(kitty_kv_layer L, int T) {
+  const int b = blockIdx.x;
+  const ChunkPlan c = chunk_plan(L, b, T);
+  if (!c.active) return;
+  const bool ok = chunk_pages_ok(L, b, c);
+  if (threadIdx.x != 0) return;
+  int32_t* cnt = const_cast<int32_t*>(L.seq_counts) + b * KITTY_SEQ_COUNT_FIELDS;
+  if (!ok) {
+    bump_status(L, b, KITTY_STATUS_TOKENS_DROPPED, T);
+    return;
+  }
+  cnt[KITTY_CNT_SINK] = c.sink + c.a;
+  cnt[KITTY_CNT_PAGES_K] = c.pk + c.npk;
+  cnt[KITTY_CNT_QBUF_K] = c.rk2;
+  cnt[KITTY_CNT_PAGES_V] = c.pv + c.npv;
+  cnt[KITTY_CNT_QBUF_V] = c.rv2;
+  cnt[KITTY_CNT_LOCAL_V] = c.lv2;
+  cnt[KITTY_CNT_LOCAL_OFF] = c.off2;
 }
 
 int check_src(const void* p, int64_t sb, int64_t sh, int64_t st, int B, int H, int T, int D, int t_offset,
@@ -493,7 +736,7 @@ extern "C" int kitty_select_boost_k(const void* key, int64_t stride_b, int64_t s
   if (B == 0 || pages == 0) return 0;
   hipLaunchKernelGGL(quant_pack_k_kernel<2>, dim3(pages, H, B), dim3(256), 0, (hipStream_t)stream,
                      (const uint8_t*)key, stride_b, stride_h, stride_t, t_offset, d_boost, nullptr, slot_map,
-                     pages, nullptr, 0, 0, nullptr, 0, nullptr, 0, 0);
+                     pages, nullptr, 0, 0, nullptr, 0, nullptr, 0, 0, nullptr);
   return check_launch("kitty_select_boost_k");
 }
 
@@ -502,8 +745,10 @@ extern "C" int kitty_quant_pack_k(const void* key, int64_t stride_b, int64_t str
                                   const uint8_t* slot_map,
                                   const int64_t* page_table, int64_t page_table_stride_b, int page_offset,
                                   uint8_t* cache, int64_t cache_stride_page,
-                                  void* meta, int64_t meta_stride_page, int64_t cache_pages, void* stream) {
+                                  void* meta, int64_t meta_stride_page, int64_t cache_pages, int32_t* status,
+                                  void* stream) {
   if (int rc = check_src(key, stride_b, stride_h, stride_t, B, H, T, D, t_offset, pages, page_size)) return rc;
+  KITTY_REQUIRE(((uintptr_t)status % 4) == 0, KITTY_E_ALIGN, "status needs 4-byte alignment");
   // the slot map is a uint8 with d_boost as the "not boosted" marker, and the high plane has
   // d_boost rows: keep rows 4-byte friendly
   KITTY_REQUIRE(d_boost >= 0 && d_boost <= D, KITTY_E_SHAPE, "d_boost must be in [0, %d], got %d", D, d_boost);
@@ -518,12 +763,12 @@ extern "C" int kitty_quant_pack_k(const void* key, int64_t stride_b, int64_t str
     hipLaunchKernelGGL(quant_pack_k_kernel<0>, grid, block, 0, (hipStream_t)stream, (const uint8_t*)key, stride_b,
                        stride_h, stride_t, t_offset, d_boost, slot_map, nullptr, pages, page_table,
                        page_table_stride_b, page_offset, cache, cache_stride_page, (uint8_t*)meta,
-                       meta_stride_page, cache_pages);
+                       meta_stride_page, cache_pages, status);
   else
     hipLaunchKernelGGL(quant_pack_k_kernel<1>, grid, block, 0, (hipStream_t)stream, (const uint8_t*)key, stride_b,
                        stride_h, stride_t, t_offset, d_boost, nullptr, nullptr, pages, page_table,
                        page_table_stride_b, page_offset, cache, cache_stride_page, (uint8_t*)meta,
-                       meta_stride_page, cache_pages);
+                       meta_stride_page, cache_pages, status);
   return check_launch("kitty_quant_pack_k");
 }
 
@@ -531,8 +776,10 @@ extern "C" int kitty_quant_pack_v(const void* value, int64_t stride_b, int64_t s
                                   int B, int H, int T, int D, int t_offset, int pages, int page_size,
                                   const int64_t* page_table, int64_t page_table_stride_b, int page_offset,
                                   uint8_t* cache, int64_t cache_stride_page,
-                                  void* meta, int64_t meta_stride_page, int64_t cache_pages, void* stream) {
+                                  void* meta, int64_t meta_stride_page, int64_t cache_pages, int32_t* status,
+                                  void* stream) {
   if (int rc = check_src(value, stride_b, stride_h, stride_t, B, H, T, D, t_offset, pages, page_size)) return rc;
+  KITTY_REQUIRE(((uintptr_t)status % 4) == 0, KITTY_E_ALIGN, "status needs 4-byte alignment");
   if (int rc = check_dst(page_table, page_offset, cache, cache_stride_page, meta, meta_stride_page, cache_pages,
                          (int64_t)H * kVBytes, (int64_t)H * kPage * 4))
     return rc;
@@ -540,7 +787,7 @@ extern "C" int kitty_quant_pack_v(const void* value, int64_t stride_b, int64_t s
   hipLaunchKernelGGL(quant_pack_v_kernel, dim3(pages, H, B), dim3(256), 0, (hipStream_t)stream,
                      (const uint8_t*)value, stride_b, stride_h, stride_t, t_offset, page_table,
                      page_table_stride_b, page_offset, cache, cache_stride_page, (uint8_t*)meta, meta_stride_page,
-                     cache_pages);
+                     cache_pages, status);
   return check_launch("kitty_quant_pack_v");
 }
 
@@ -565,8 +812,10 @@ int check_append_layer(const kitty_kv_layer* layer, int B) {
                     ((uintptr_t)L.sink_k % 16) == 0 && ((uintptr_t)L.sink_v % 16) == 0 &&
                     ((uintptr_t)L.qbuf_k % 16) == 0 && ((uintptr_t)L.qbuf_v % 16) == 0 &&
                     ((uintptr_t)L.local_v % 16) == 0 && L.sink_stride_b % 16 == 0 && L.sink_stride_h % 16 == 0 &&
-                    L.win_stride_b % 16 == 0 && L.win_stride_h % 16 == 0 && ((uintptr_t)L.seq_counts % 4) == 0,
+                    L.win_stride_b % 16 == 0 && L.win_stride_h % 16 == 0 && ((uintptr_t)L.seq_counts % 4) == 0 &&
+                    ((uintptr_t)L.status % 4) == 0,
                 KITTY_E_ALIGN, "cache tensors need 16-byte alignment");
+  KITTY_REQUIRE(L.cache_pages_k >= 0 && L.cache_pages_v >= 0, KITTY_E_RANGE, "negative cache_pages_k / cache_pages_v");
   KITTY_REQUIRE(L.key_cache_stride_page >= (int64_t)L.H_KV * k_head_bytes(L.D_BOOSTED) &&
                     L.value_cache_stride_page >= (int64_t)L.H_KV * kVBytes &&
                     L.key_meta_stride_page >= (int64_t)L.H_KV * kD * 4 &&
@@ -577,21 +826,48 @@ int check_append_layer(const kitty_kv_layer* layer, int B) {
 }  // namespace
 
 extern "C" int kitty_append_token(const kitty_kv_layer* layer, const void* k_new, const void* v_new,
-                                  int64_t stride_b, int64_t stride_h, int B, void* stream) {
+                                  int64_t stride_b, int64_t stride_h, const void* rope_cos, const void* rope_sin,
+                                  int64_t rope_stride_b, int B, void* stream) {
   if (int rc = check_append_layer(layer, B)) return rc;
   KITTY_REQUIRE(k_new && v_new, KITTY_E_NULL, "k_new / v_new is NULL");
   KITTY_REQUIRE(((uintptr_t)k_new % 8) == 0 && ((uintptr_t)v_new % 8) == 0 && stride_b % 8 == 0 && stride_h % 8 == 0,
                 KITTY_E_ALIGN, "k_new / v_new need 8-byte aligned bases and strides");
-  hipLaunchKernelGGL(append_token_kernel, dim3(B), dim3(256), 0, (hipStream_t)stream, *layer, (const uint8_t*)k_new,
-                     (const uint8_t*)v_new, stride_b, stride_h);
+  KITTY_REQUIRE((rope_cos == nullptr) == (rope_sin == nullptr), KITTY_E_NULL, "rope_cos and rope_sin go together");
+  if (rope_cos) {
+    KITTY_REQUIRE(((uintptr_t)rope_cos % 8) == 0 && ((uintptr_t)rope_sin % 8) == 0 && rope_stride_b % 8 == 0 &&
+                      (rope_stride_b == 0 || rope_stride_b >= kD * 2),
+                  KITTY_E_ALIGN, "rope_cos / rope_sin need 8-byte aligned rows of D fp16 values");
+    hipLaunchKernelGGL(append_token_kernel<true>, dim3(B), dim3(256), 0, (hipStream_t)stream, *layer,
+                       (const uint8_t*)k_new, (const uint8_t*)v_new, stride_b, stride_h, (const uint8_t*)rope_cos,
+                       (const uint8_t*)rope_sin, rope_stride_b);
+  } else {
+    hipLaunchKernelGGL(append_token_kernel<false>, dim3(B), dim3(256), 0, (hipStream_t)stream, *layer,
+                       (const uint8_t*)k_new, (const uint8_t*)v_new, stride_b, stride_h, nullptr, nullptr, 0);
+  }
   return check_launch("kitty_append_token");
 }
 
-extern "C" int kitty_flush_full(const kitty_kv_layer* layer, int B, int64_t cache_pages, void* stream) {
+extern "C" int kitty_flush_full(const kitty_kv_layer* layer, int B, void* stream) {
   if (int rc = check_append_layer(layer, B)) return rc;
-  KITTY_REQUIRE(cache_pages >= 0, KITTY_E_RANGE, "bad cache_pages");
-  hipLaunchKernelGGL(flush_full_kernel, dim3(layer->H_KV, B, 2), dim3(256), 0, (hipStream_t)stream, *layer, cache_pages);
-  hipLaunchKernelGGL(advance_counts_kernel, dim3((B + 63) / 64), dim3(64), 0, (hipStream_t)stream, *layer, B,
-                     cache_pages);
+  hipLaunchKernelGGL(flush_full_kernel, dim3(layer->H_KV, B, 2), dim3(256), 0, (hipStream_t)stream, *layer);
+  hipLaunchKernelGGL(advance_counts_kernel, dim3((B + 63) / 64), dim3(64), 0, (hipStream_t)stream, *layer, B);
   return check_launch("kitty_flush_full");
+}
+
+extern "C" int kitty_append_chunk(const kitty_kv_layer* layer, const void* k_new, const void* v_new,
+                                  int64_t stride_b, int64_t stride_h, int64_t stride_t, int B, int T, void* stream) {
+  if (int rc = check_append_layer(layer, B)) return rc;
+  KITTY_REQUIRE(k_new && v_new, KITTY_E_NULL, "k_new / v_new is NULL");
+  KITTY_REQUIRE(T >= 1 && T <= (1 << 24), KITTY_E_RANGE, "T=%d out of range", T);
+  KITTY_REQUIRE(((uintptr_t)k_new % 16) == 0 && ((uintptr_t)v_new % 16) == 0 && stride_b % 16 == 0 &&
+                    stride_h % 16 == 0 && stride_t % 16 == 0 && stride_t >= kD * 2,
+                KITTY_E_ALIGN, "k_new / v_new need 16-byte aligned bases and strides with D contiguous");
+  const int max_pages = (T + kPage - 1) / kPage;   // a stream holds at most 127 rows before the chunk
+  const hipStream_t st = (hipStream_t)stream;
+  hipLaunchKernelGGL(chunk_quant_kernel, dim3(2 * max_pages, layer->H_KV, B), dim3(256), 0, st, *layer,
+                     (const uint8_t*)k_new, (const uint8_t*)v_new, stride_b, stride_h, stride_t, T, max_pages);
+  hipLaunchKernelGGL(chunk_rows_kernel, dim3(layer->H_KV, B), dim3(256), 0, st, *layer, (const uint8_t*)k_new,
+                     (const uint8_t*)v_new, stride_b, stride_h, stride_t, T);
+  hipLaunchKernelGGL(chunk_advance_kernel, dim3(B), dim3(64), 0, st, *layer, T);
+  return check_launch("kitty_append_chunk");
 }

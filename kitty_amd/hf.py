@@ -68,10 +68,13 @@ class PagedKittyHFCache(PagedKittyCache):
 
     def update(self, key_states: torch.Tensor, value_states: torch.Tensor, layer_idx: int,
                cache_kwargs: Optional[dict[str, Any]] = None):
-        if self._admit_slot is None and key_states.shape[-2] != 1:
-            raise ValueError("several new tokens per sequence: admit a prompt inside `with cache.admitting(slot):`")
         _current.cache = self
-        _current.phase = "prefill" if super().update(key_states, value_states, layer_idx, cache_kwargs) else "decode"
+        if self._admit_slot is None and key_states.shape[-2] != 1:
+            # several new tokens for every slot over what the slots hold: attention needs the cache
+            # as it was, the attention function appends afterwards
+            _current.phase = "chunk"
+        else:
+            _current.phase = "prefill" if super().update(key_states, value_states, layer_idx, cache_kwargs) else "decode"
         return key_states, value_states
 
     def get_seq_length(self, layer_idx: int = 0) -> int:
@@ -83,9 +86,10 @@ class PagedKittyHFCache(PagedKittyCache):
         n = query_length if isinstance(query_length, int) else int(query_length.shape[0])
         return n, 0
 
-    def position_ids(self) -> torch.Tensor:
-        """[slots, 1] int64 on the cache's device: the position of each slot's next token."""
-        return torch.from_numpy(self.seq_lengths().astype("int64")).view(-1, 1).to(self.seq_counts.device)
+    def position_ids(self, n_tokens: int = 1) -> torch.Tensor:
+        """[slots, n_tokens] int64 on the cache's device: the positions of each slot's next tokens."""
+        first = torch.from_numpy(self.seq_lengths().astype("int64")).view(-1, 1)
+        return (first + torch.arange(n_tokens, dtype=torch.int64).view(1, -1)).to(self.seq_counts.device)
 
 
 def kitty_attention(module, query: torch.Tensor, key: torch.Tensor, value: torch.Tensor,

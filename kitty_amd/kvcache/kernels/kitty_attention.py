@@ -46,9 +46,7 @@ def kitty_attention_forward(
     else:
         max_tiles = 2 + kv_cache.MAX_PAGE
     if not num_splits or num_splits <= 0:
-        num_splits = lib.kitty_decode_attn_default_splits(B, H_KV, max_tiles)
-        if kv_cache.seq_counts is not None and num_splits < 12 and max_tiles >= 48:
-            num_splits = 12      # sequences of different lengths: more, shorter splits even out the load
+        num_splits = lib.kitty_decode_attn_default_splits(B, H_KV, max_tiles, int(kv_cache.seq_counts is not None))
     ws_bytes = lib.kitty_decode_attn_workspace_bytes(B, H_Q, D, num_splits)
     ws = kv_cache.workspace(ws_bytes)
     # [B, T=1, H_Q, D], the layout HF attention modules expect (kitty_attention.py:475-481)

@@ -11,6 +11,9 @@ K kernel.  Keyword-only additions:
                     kernel consumes it (tie order is then whatever ``torch.topk`` does there).
 ``slot_map=``       a caller-supplied uint8 ``[B, H, pages, D]`` map (the kernel boundary of the
                     reference's ``quantize_pack_k_kernel``).
+``status=``         int32 ``[B, 4]`` device tensor: a page id outside the cache is never written
+                    to, and row b's "bad page" word is raised instead (the reference would write
+                    out of bounds).
 """
 from typing import Optional
 
@@ -28,6 +31,16 @@ def _src_args(x: torch.Tensor, name: str):
         x = x.contiguous()
     B, H, T, D = x.shape
     return x, (x.data_ptr(), x.stride(0) * 2, x.stride(1) * 2, x.stride(2) * 2, B, H, T, D)
+
+
+def _status_ptr(status, B: int, device):
+    if status is None:
+        return None
+    _lib.require_hip(status, "status")
+    if status.dtype != torch.int32 or status.dim() != 2 or status.shape[0] < B or status.shape[1] != _lib.STATUS_FIELDS \
+            or not status.is_contiguous():
+        raise ValueError(f"status must be a contiguous int32 [>= {B}, {_lib.STATUS_FIELDS}] tensor")
+    return status.data_ptr()
 
 
 def _check_dst(page_table, cache, cache_metadata):
@@ -79,6 +92,7 @@ def quantize_pack_k(
     *,
     select: str = "hip",
     slot_map: Optional[torch.Tensor] = None,
+    status: Optional[torch.Tensor] = None,
 ) -> None:
     """Quantize and pack the key states into the paged key cache."""
     assert key_states.dim() == 4
@@ -101,7 +115,8 @@ def quantize_pack_k(
         None if slot_map is None else slot_map.data_ptr(),
         page_table_k.data_ptr(), page_table_k.stride(0), page_offset_k,
         cache.data_ptr(), cache.stride(0), cache_metadata.data_ptr(), cache_metadata.stride(0) * 2,
-        cache.shape[0], _lib.current_stream_ptr(key_states.device))
+        cache.shape[0], _status_ptr(status, key_states.shape[0], key_states.device),
+        _lib.current_stream_ptr(key_states.device))
     _lib.check(rc, "quantize_pack_k")
 
 
@@ -114,6 +129,8 @@ def quantize_pack_v(
     cache: torch.Tensor,                        # (MAX_BS * MAX_PAGE, bytes_per_page_V) uint8
     cache_metadata: torch.Tensor,               # (MAX_BS * MAX_PAGE, H_KV, PAGE_SIZE, 2) float16
     page_size: int,
+    *,
+    status: Optional[torch.Tensor] = None,
 ) -> None:
     """Quantize and pack the value states into the paged value cache."""
     assert value_states.dim() == 4
@@ -123,5 +140,6 @@ def quantize_pack_v(
         *src, value_states_t_offset, value_states_page_count, page_size,
         page_table_v.data_ptr(), page_table_v.stride(0), page_offset_v,
         cache.data_ptr(), cache.stride(0), cache_metadata.data_ptr(), cache_metadata.stride(0) * 2,
-        cache.shape[0], _lib.current_stream_ptr(value_states.device))
+        cache.shape[0], _status_ptr(status, value_states.shape[0], value_states.device),
+        _lib.current_stream_ptr(value_states.device))
     _lib.check(rc, "quantize_pack_v")

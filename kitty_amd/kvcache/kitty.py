@@ -132,7 +132,8 @@ class KittyCache(_HFCache):
             kvcache.Q_Buffer_K[rows, :, :len_qbuf_k, :].copy_(K[:, :, len_prefill - len_qbuf_k:, :])
         if pages_k > 0:
             quantize_pack_k(K, len_sink, pages_k, kvcache.PageTable_K[rows], 0, kvcache.KeyCache,
-                            kvcache.KeyCache_metadata, P, kvcache.D_BOOSTED, select=self.select)
+                            kvcache.KeyCache_metadata, P, kvcache.D_BOOSTED, select=self.select,
+                            status=kvcache.status[rows])
         kvcache.Sink_Buffer_V[rows, :, :len_sink, :].copy_(V[:, :, :len_sink, :])
         if len_local_v > 0:
             kvcache.Local_Buffer_V[rows, :, :len_local_v, :].copy_(V[:, :, len_prefill - len_local_v:, :])
@@ -143,7 +144,7 @@ class KittyCache(_HFCache):
         if pages_v > 0:
             assert len_prefill - len_sink - len_local_v - len_qbuf_v == pages_v * P
             quantize_pack_v(V, len_sink, pages_v, kvcache.PageTable_V[rows], 0, kvcache.ValueCache,
-                            kvcache.ValueCache_metadata, P)
+                            kvcache.ValueCache_metadata, P, status=kvcache.status[rows])
         return n
 
     def quantize_decode(self, layer_idx: int = 0) -> None:
@@ -157,16 +158,43 @@ class KittyCache(_HFCache):
             if kvcache.PageCount_K >= kvcache.MAX_PAGE:
                 raise ValueError(f"key cache is full (max_length={kvcache.MAX_LEN})")
             quantize_pack_k(kvcache.Q_Buffer_K, 0, 1, kvcache.PageTable_K, kvcache.PageCount_K, kvcache.KeyCache,
-                            kvcache.KeyCache_metadata, kvcache.PAGE_SIZE, kvcache.D_BOOSTED, select=self.select)
+                            kvcache.KeyCache_metadata, kvcache.PAGE_SIZE, kvcache.D_BOOSTED, select=self.select,
+                            status=kvcache.status)
             kvcache.PageCount_K += 1
             kvcache.Q_Buffer_Count_K = 0
         if kvcache.Q_Buffer_Count_V == kvcache.PAGE_SIZE:
             if kvcache.PageCount_V >= kvcache.MAX_PAGE:
                 raise ValueError(f"value cache is full (max_length={kvcache.MAX_LEN})")
             quantize_pack_v(kvcache.Q_Buffer_V, 0, 1, kvcache.PageTable_V, kvcache.PageCount_V, kvcache.ValueCache,
-                            kvcache.ValueCache_metadata, kvcache.PAGE_SIZE)
+                            kvcache.ValueCache_metadata, kvcache.PAGE_SIZE, status=kvcache.status)
             kvcache.PageCount_V += 1
             kvcache.Q_Buffer_Count_V = 0
+
+    # ---- what the device could not do --------------------------------------------------------------
+    def check_status(self, raise_on_error: bool = True, clear: bool = False) -> dict:
+        """Read the layers' device-side status words (one synchronising copy per call).
+
+        The reference stops with an assert before a buffer overflows (kitty.py:109,113,118).  With
+        per-sequence counters on the device the host cannot know, so the kernels skip such work,
+        exit normally and leave a record per sequence: tokens dropped because a Q-buffer was still
+        full, flushes skipped for want of a page, page ids outside the cache met by a writer or by
+        attention.  Returns ``{name: int32 array [layers, MAX_BS]}`` and raises ``RuntimeError``
+        when anything is set (unless ``raise_on_error=False``); ``clear=True`` zeroes the words."""
+        import numpy as np
+        st = torch.stack([L.status for L in self.kv_cache]).cpu().numpy()
+        out = {name: st[:, :, i].copy() for i, name in enumerate(_lib.STATUS_NAMES)}
+        if clear:
+            for L in self.kv_cache:
+                L.status.zero_()
+        if raise_on_error and st.any():
+            parts = []
+            for name, a in out.items():
+                if a.any():
+                    layers, seqs = np.nonzero(a)
+                    parts.append(f"{name}: layer {int(layers[0])} sequence {int(seqs[0])} = {int(a[layers[0], seqs[0]])}"
+                                 f" ({len(seqs)} (layer, sequence) pairs)")
+            raise RuntimeError("the device skipped work it could not do: " + "; ".join(parts))
+        return out
 
     # ---- per-sequence counters on the device ---------------------------------------------------
     def enable_device_counters(self, seq_counts: Optional[torch.Tensor] = None) -> None:
@@ -210,13 +238,37 @@ class KittyCache(_HFCache):
             for f, v in zip(L.COUNT_FIELDS, row):
                 setattr(L, f, int(v))
 
-    def _append_token_device(self, L: KVCache_Layer, key_states: torch.Tensor, value_states: torch.Tensor) -> None:
+    def _append_token_device(self, L: KVCache_Layer, key_states: torch.Tensor, value_states: torch.Tensor,
+                             rope=None) -> None:
         if L.Sink_Count >= L.S and L.Q_Buffer_Count_K >= L.PAGE_SIZE:
             raise ValueError("Q-buffer is full: call quantize_decode() after every decode step")
-        self._launch_append(L, key_states, value_states)
+        self._launch_append(L, key_states, value_states, rope)
         L.step_host_counters()
 
-    def _launch_append(self, L: KVCache_Layer, key_states: torch.Tensor, value_states: torch.Tensor) -> None:
+    def update_with_rope(self, key_states: torch.Tensor, value_states: torch.Tensor, cos: torch.Tensor,
+                         sin: torch.Tensor, layer_idx: int) -> bool:
+        """Decode-step ``update`` that also applies the rotary embedding to the new key:
+        ``key_states`` are the keys BEFORE the rotation, ``cos`` / ``sin`` fp16 ``[B, 1, D]`` (or
+        ``[B, D]``, or one row for all) as the model's rotary module returns them.  The append kernel
+        stores ``k * cos + rotate_half(k) * sin`` with fp16 tensor arithmetic's roundings, i.e. the
+        bits the caller's own ``apply_rotary_pos_emb`` would have produced
+        (modeling_qwen3.py:215-220), without materialising the rotated key.  Needs device counters."""
+        L = self.kv_cache[layer_idx]
+        if not L.device_counters:
+            raise ValueError("the fused rotary append is part of the device-counter path: call enable_device_counters()")
+        assert key_states.shape[-2] == 1 and value_states.shape[-2] == 1, \
+            "Decode: key_states and value_states should have sequence length of 1."
+        B, D = key_states.shape[0], L.D
+        rope = []
+        for name, t in (("cos", cos), ("sin", sin)):
+            _lib.require_hip(t, name)
+            if t.dtype != torch.float16 or t.shape[-1] != D or t.numel() not in (D, B * D):
+                raise ValueError(f"{name} must be float16 with {D} or {B} x {D} elements, got {tuple(t.shape)} {t.dtype}")
+            rope.append(t.reshape(-1, D).contiguous())
+        self._append_token_device(L, key_states, value_states, rope)
+        return False
+
+    def _launch_append(self, L: KVCache_Layer, key_states: torch.Tensor, value_states: torch.Tensor, rope=None) -> None:
         B = key_states.shape[0]
         for name, t in (("key_states", key_states), ("value_states", value_states)):
             _lib.require_hip(t, name)
@@ -228,9 +280,15 @@ class KittyCache(_HFCache):
             key_states = key_states.contiguous()
         if value_states.stride() != key_states.stride():
             key_states, value_states = key_states.contiguous(), value_states.contiguous()
+        cos_p = sin_p = None
+        rope_stride = 0
+        if rope is not None:
+            cos, sin = rope
+            cos_p, sin_p = cos.data_ptr(), sin.data_ptr()
+            rope_stride = 0 if cos.shape[0] == 1 else cos.stride(0) * 2
         rc = _lib.lib().kitty_append_token(L.descriptor(), key_states.data_ptr(), value_states.data_ptr(),
-                                           key_states.stride(0) * 2, key_states.stride(1) * 2, B,
-                                           _lib.current_stream_ptr(key_states.device))
+                                           key_states.stride(0) * 2, key_states.stride(1) * 2, cos_p, sin_p, rope_stride,
+                                           B, _lib.current_stream_ptr(key_states.device))
         _lib.check(rc, "KittyCache.update")
         L.active_batch = B
 
@@ -248,8 +306,7 @@ class KittyCache(_HFCache):
             L.Q_Buffer_Count_V = 0
 
     def _launch_flush(self, L: KVCache_Layer) -> None:
-        rc = _lib.lib().kitty_flush_full(L.descriptor(), L.active_batch, L.KeyCache.size(0),
-                                         _lib.current_stream_ptr(L.device))
+        rc = _lib.lib().kitty_flush_full(L.descriptor(), L.active_batch, _lib.current_stream_ptr(L.device))
         _lib.check(rc, "KittyCache.quantize_decode")
 
     def append(self, key_states: torch.Tensor, value_states: torch.Tensor, layer_idx: int = 0) -> None:
@@ -264,11 +321,11 @@ class KittyCache(_HFCache):
         ``update`` + ``quantize_prefill``.
         """
         L = self.kv_cache[layer_idx]
-        if L.device_counters:
-            raise NotImplementedError("chunk append works on the shared host counters; with device "
-                                      "counters append token by token (update + quantize_decode)")
         if key_states.shape != value_states.shape or key_states.dim() != 4:
             raise ValueError("key_states and value_states must both be [B, H_KV, T, D]")
+        if L.device_counters:
+            self._append_chunk_device(L, key_states, value_states)
+            return
         if L.get_total_length() == 0:
             self.update(key_states, value_states, layer_idx)
             self.quantize_prefill(layer_idx)
@@ -312,6 +369,45 @@ class KittyCache(_HFCache):
                 j += run
             L.Local_Count_V = lv_after
             L.Write_Offset_Local_V = (off + evicted) % P
+
+    @staticmethod
+    def chunk_counts(c: dict, T: int, S: int, P: int) -> dict:
+        """The counters after a chunk of ``T`` tokens (what T single steps leave; the device's
+        chunk kernels use the same closed form).  ``c``: sink, pk, rk, pv, rv, lv, off."""
+        a = min(S - c["sink"], T)
+        n = T - a
+        lv2 = min(P, c["lv"] + n)
+        e = c["lv"] + n - lv2
+        return dict(sink=c["sink"] + a, pk=c["pk"] + (c["rk"] + n) // P, rk=(c["rk"] + n) % P,
+                    pv=c["pv"] + (c["rv"] + e) // P, rv=(c["rv"] + e) % P, lv=lv2, off=(c["off"] + e) % P)
+
+    def _append_chunk_device(self, L: KVCache_Layer, key_states: torch.Tensor, value_states: torch.Tensor) -> None:
+        """``append`` with per-sequence counters on the device: three launches (new pages straight
+        from their sources, fp16 rows, counters), every sequence from its own state.  The host ints
+        follow the longest sequence by the same closed form."""
+        B, H, T, D = key_states.shape
+        for name, t in (("key_states", key_states), ("value_states", value_states)):
+            _lib.require_hip(t, name)
+            if t.dtype != torch.float16:
+                raise ValueError(f"{name} must be float16, got {t.dtype}")
+        if (H, D) != (L.H_KV, L.D) or B > L.MAX_BS or T < 1:
+            raise ValueError(f"key_states / value_states must be [B <= {L.MAX_BS}, {L.H_KV}, T >= 1, {L.D}]")
+        if key_states.stride(-1) != 1 or any(s % 8 for s in key_states.stride()[:3]) or key_states.data_ptr() % 16:
+            key_states = key_states.contiguous()
+        if value_states.stride() != key_states.stride() or value_states.data_ptr() % 16:
+            key_states, value_states = key_states.contiguous(), value_states.contiguous()
+        names = ("sink", "pk", "rk", "pv", "rv", "lv", "off")
+        before = dict(zip(names, L.counts()[:7]))
+        after = self.chunk_counts(before, T, L.S, L.PAGE_SIZE)
+        if after["pk"] > L.MAX_PAGE or after["pv"] > L.MAX_PAGE:
+            raise ValueError(f"appending {T} tokens exceeds max_length={L.MAX_LEN}")
+        ks = [x * 2 for x in key_states.stride()]
+        rc = _lib.lib().kitty_append_chunk(L.descriptor(), key_states.data_ptr(), value_states.data_ptr(),
+                                           ks[0], ks[1], ks[2], B, T, _lib.current_stream_ptr(key_states.device))
+        _lib.check(rc, "KittyCache.append")
+        L.active_batch = B
+        for f, name in zip(L.COUNT_FIELDS, names):
+            setattr(L, f, int(after[name]))
 
     def _push_k(self, L: KVCache_Layer, src: torch.Tensor, lo: int, hi: int, B: int) -> None:
         """Rows ``src[:, :, lo:hi]`` enter the K quantize stream: whole pages straight from ``src``

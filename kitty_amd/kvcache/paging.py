@@ -279,6 +279,9 @@ class PagedKittyCache(KittyCache):
             return True
         assert key_states.shape[-2] == 1 and value_states.shape[-2] == 1, \
             "Decode: key_states and value_states should have sequence length of 1."
+        if key_states.shape[0] != self.n_slots:
+            # the host shadow steps every active slot; a smaller batch would leave the slots past it behind
+            raise ValueError(f"a decode batch of a paged cache is all {self.n_slots} slots, got {key_states.shape[0]} rows")
         self._launch_append(L, key_states, value_states)     # the host ints follow at the end of the step
         return False
 
@@ -319,9 +322,65 @@ class PagedKittyCache(KittyCache):
         """After the replay of a captured decode step (all layers): advance the host side."""
         self._end_of_step()
 
-    def append(self, key_states, value_states, layer_idx: int = 0) -> None:
-        raise NotImplementedError("chunk append works on the shared host counters; admit a prompt in one "
-                                  "piece and decode token by token")
+    def append(self, key_states: torch.Tensor, value_states: torch.Tensor, layer_idx: int = 0) -> None:
+        """``T`` new tokens for every slot at once, ``[n_slots, H_KV, T, D]`` (rows of free slots are
+        ignored): the state afterwards is the one ``T`` decode steps leave.  Call it for every layer,
+        layer 0 first, the last layer last, like the decode step's calls.  The pages the chunk fills
+        (and the page of the flush after it) are taken from the pools before the first layer's
+        launch; if they cannot be had, ``OutOfPages`` is raised and nothing has changed."""
+        if self._admit_slot is not None:
+            raise ValueError("a prompt under admission goes through update() + quantize_prefill()")
+        if key_states.dim() != 4 or key_states.shape != value_states.shape or key_states.shape[0] != self.n_slots:
+            raise ValueError(f"key_states / value_states must both be [{self.n_slots}, H_KV, T, D]")
+        T = key_states.shape[-2]
+        if layer_idx == 0 and not self._capturing:
+            self._reserve_for_chunk(T)
+        L = self.kv_cache[layer_idx]
+        saved = L.counts()
+        self._append_chunk_device(L, key_states, value_states)
+        for f, v in zip(L.COUNT_FIELDS, saved):          # the host ints are set for all layers at the end
+            setattr(L, f, int(v))
+        if layer_idx == len(self.kv_cache) - 1 and not self._capturing:
+            self._end_of_chunk(T)
+
+    def _chunk_after(self, T: int) -> np.ndarray:
+        """The shadow counters of every slot after a chunk of T tokens (active slots only change)."""
+        L = self.kv_cache[0]
+        c = self._shadow.copy()
+        for slot in np.flatnonzero(self._active):
+            r = c[slot]
+            after = self.chunk_counts(dict(sink=r[_F_SINK], pk=r[_F_PK], rk=r[_F_RK], pv=r[_F_PV], rv=r[_F_RV],
+                                           lv=r[_F_LV], off=r[_F_OFF]), T, L.S, L.PAGE_SIZE)
+            c[slot, :7] = [after[k] for k in ("sink", "pk", "rk", "pv", "rv", "lv", "off")]
+        return c
+
+    def _reserve_for_chunk(self, T: int) -> None:
+        L = self.kv_cache[0]
+        c = self._shadow
+        if (self._active & (c[:, _F_SINK] >= L.S) & ((c[:, _F_RK] >= L.PAGE_SIZE) | (c[:, _F_RV] >= L.PAGE_SIZE))).any():
+            raise OutOfPages("a sequence still waits for the page of a flush: release pages (ensure_pages) first")
+        after = self._chunk_after(T)
+        if (after[:, _F_PK] > self.max_page).any() or (after[:, _F_PV] > self.max_page).any():
+            raise ValueError(f"appending {T} tokens exceeds max_length={L.MAX_LEN}")
+        plan = []
+        for kind, pool, host, f in (("k", self.pool_k, self._table_k, _F_PK), ("v", self.pool_v, self._table_v, _F_PV)):
+            slots, entries = [], []
+            for slot in np.flatnonzero(self._active):
+                have = int((host[slot] >= 0).sum())                       # assigned entries are a prefix of the row
+                want = min(int(after[slot, f]) + 1, self.max_page)       # the pages filled, and the next flush's
+                slots += [int(slot)] * max(0, want - have)
+                entries += list(range(have, want))
+            if len(slots) > pool.free:
+                raise OutOfPages(f"a chunk of {T} tokens needs {len(slots)} more {kind.upper()} pages, {pool.free} are free")
+            plan.append((kind, pool, slots, entries))
+        for kind, pool, slots, entries in plan:
+            if slots:
+                self._write_tables(kind, slots, entries, pool.take(len(slots)))
+            self._starved = {(k, s) for k, s in self._starved if k != kind}
+
+    def _end_of_chunk(self, T: int) -> None:
+        self._shadow = self._chunk_after(T)
+        self._sync_longest()
 
     def enable_device_counters(self, seq_counts=None) -> None:
         raise ValueError("a paged cache keeps its counters on the device from the start")

@@ -12,6 +12,9 @@ against the reference keeps working.  Differences, all additive:
   79-80).  When it is ``None`` the shared counters are used, exactly like the reference;
 * ``enable_device_counters()`` - from then on decode steps advance ``seq_counts`` on the device
   (one fused append kernel, one flush launch) and the host ints only shadow the longest sequence;
+* ``status`` - int32 ``[MAX_BS, 4]`` on the device: what the kernels could not do (tokens dropped,
+  flushes skipped, page ids out of range); the reference asserts on the host instead
+  (kitty.py:109,113,118), which kernels that take their counters from device memory cannot;
 * ``n_pages=`` / ``page_tables=`` - a page pool smaller (or larger) than the reference's static
   ``MAX_BS * MAX_PAGE`` pages, with page tables handed in by the owner of the pool (entries of -1:
   no page assigned); see ``paging.PagedKittyCache``.
@@ -86,6 +89,7 @@ class KVCache_Layer:
         self.value_states: Optional[torch.Tensor] = None
         # extensions
         self.seq_counts: Optional[torch.Tensor] = None
+        self.status = torch.zeros((MAX_BS, _lib.STATUS_FIELDS), dtype=torch.int32, device=dev)
         self.device_counters = False
         self.active_batch = MAX_BS
         self._workspace: Optional[torch.Tensor] = None
@@ -169,6 +173,8 @@ class KVCache_Layer:
             d.qbuf_k, d.qbuf_v = self.Q_Buffer_K.data_ptr(), self.Q_Buffer_V.data_ptr()
             d.local_v = self.Local_Buffer_V.data_ptr()
             d.win_stride_b, d.win_stride_h = self.Q_Buffer_K.stride(0) * 2, self.Q_Buffer_K.stride(1) * 2
+            d.cache_pages_k, d.cache_pages_v = self.KeyCache.shape[0], self.ValueCache.shape[0]
+            d.status = self.status.data_ptr()
             self._desc = d
         for i, v in enumerate(self.counts()):
             d.counts[i] = int(v)

@@ -158,7 +158,10 @@ class KittyKVCache(_HFCache):
     implementation take it as ``past_key_values``."""
     is_compileable = False
 
-    def __init__(self, cache_config: KittyKVCacheConfig, max_length: int):
+    def __init__(self, cache_config: KittyKVCacheConfig, max_length: Optional[int] = None):
+        """``KittyKVCache(cache_config)`` as in the reference (kitty_simulate.py:151).  ``max_length``
+        (optional) sizes a layer's buffers once for good; without it they start at twice the prompt
+        and double when full (the reference re-allocates on every step through ``torch.cat``)."""
         if _HFCache is not object:
             try:
                 super().__init__(layers=[])          # transformers >= 4.54
@@ -217,10 +220,11 @@ class KittyKVCache(_HFCache):
             if key_states.dtype != torch.float16 or D != 128 or value_states.shape != key_states.shape:
                 raise ValueError("key_states / value_states must be float16 [B, nh, T, 128]")
             assert L > c.sink_length, "Kitty-KV: sequence length must be greater than sink_length, currently."
-            if L > self.max_length:
+            if self.max_length is not None and L > self.max_length:
                 raise ValueError(f"prompt of {L} tokens exceeds max_length={self.max_length}")
+            cap = self.max_length if self.max_length is not None else max(2 * L, L + 1024)
             for store, x in ((self.key_cache, key_states), (self.value_cache, value_states)):
-                buf = torch.empty((B, nh, self.max_length, D), dtype=torch.float16, device=key_states.device)
+                buf = torch.empty((B, nh, cap, D), dtype=torch.float16, device=key_states.device)
                 buf[:, :, :L].copy_(x)
                 store.append(buf)
             self._len.append(L)
@@ -239,8 +243,15 @@ class KittyKVCache(_HFCache):
         L = self._len[layer_idx]
         T_new = key_states.shape[-2]
         assert T_new == 1, "decode appends one token per step"
-        if L + 1 > self.max_length:
+        if self.max_length is not None and L + 1 > self.max_length:
             raise ValueError(f"cache is full (max_length={self.max_length})")
+        if L + 1 > self.key_cache[layer_idx].shape[2]:                         # no max_length given: double
+            for store in (self.key_cache, self.value_cache):
+                old = store[layer_idx]
+                buf = torch.empty((old.shape[0], old.shape[1], 2 * old.shape[2], old.shape[3]), dtype=old.dtype,
+                                  device=old.device)
+                buf[:, :, :L].copy_(old[:, :, :L])
+                store[layer_idx] = buf
         K, V = self.key_cache[layer_idx], self.value_cache[layer_idx]
         K[:, :, L:L + 1].copy_(key_states)
         V[:, :, L:L + 1].copy_(value_states)

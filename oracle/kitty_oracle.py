@@ -472,6 +472,19 @@ def attend_dense(q: np.ndarray, K: np.ndarray, V: np.ndarray, scaling: float,
     return out.astype(F16) if reference_rounding else out
 
 
+def rope_fp16(x: np.ndarray, cos: np.ndarray, sin: np.ndarray) -> np.ndarray:
+    """The caller-side rotation of the keys (modeling_qwen3.py:98-102, 125-128, applied at :215-220
+    before ``update``): ``x * cos + rotate_half(x) * sin`` on fp16 tensors, i.e. both products and
+    the sum rounded to fp16.  x fp16 [B, H, T, D]; cos / sin fp16 [B, T, D] (unsqueezed over the
+    heads as the reference does).  numpy's float16 operators round each result once, like torch's.
+    Pinned by torch's own fp16 operators on the same inputs (tests/test_oracle_attention.py)."""
+    x = x.astype(F16)
+    cos, sin = cos.astype(F16)[:, None], sin.astype(F16)[:, None]
+    half = x.shape[-1] // 2
+    rot = np.concatenate([-x[..., half:], x[..., :half]], axis=-1)
+    return ((x * cos).astype(F16) + (rot * sin).astype(F16)).astype(F16)
+
+
 def decode_attention(layer: OracleLayer, query: np.ndarray, scaling: float,
                      seq_counts: Optional[list] = None, reference_rounding: bool = True,
                      dequant: str = "two") -> np.ndarray:

@@ -15,6 +15,7 @@ import os
 import sys
 
 os.environ.setdefault("TRITON_INTERPRET", "1")
+sys.dont_write_bytecode = True      # the reference checkout is read-only: leave no __pycache__ beside its file
 
 import numpy as np
 import torch

@@ -34,7 +34,7 @@ def test_header_and_binding_agree(lib):
     assert sorted(_lib.EXPORTS) == names
     for n in names:
         assert hasattr(lib, n), f"{n} declared in kitty_hip.h but not exported"
-    assert lib.kitty_abi_version() == _lib.ABI_VERSION == 1
+    assert lib.kitty_abi_version() == _lib.ABI_VERSION == 2
 
 
 def test_struct_layout_matches_c(tmp_path):
@@ -56,14 +56,14 @@ def test_host_side_rejection_without_gpu(lib):
     """Negative return codes come from host checks that run before any HIP call."""
     from kitty_amd import _lib
     E_NULL, E_SHAPE, E_RANGE, E_ALIGN, E_WORKSPACE = -1, -2, -3, -4, -5
-    assert lib.kitty_quant_pack_v(None, 0, 0, 0, 1, 1, 128, 128, 0, 1, 128, None, 0, 0, None, 0, None, 0, 0, None) == E_NULL
+    assert lib.kitty_quant_pack_v(None, 0, 0, 0, 1, 1, 128, 128, 0, 1, 128, None, 0, 0, None, 0, None, 0, 0, None, None) == E_NULL
     assert b"NULL" in lib.kitty_last_error()
     fake = ctypes.c_void_p(4096)
-    rc = lib.kitty_quant_pack_k(fake, 256, 256, 256, 1, 1, 128, 64, 0, 1, 128, 32, None, fake, 1, 0, fake, 5248, fake, 512, 1, None)
+    rc = lib.kitty_quant_pack_k(fake, 256, 256, 256, 1, 1, 128, 64, 0, 1, 128, 32, None, fake, 1, 0, fake, 5248, fake, 512, 1, None, None)
     assert rc == E_SHAPE and b"head_dim 128" in lib.kitty_last_error()
-    rc = lib.kitty_quant_pack_k(fake, 32768, 32768, 256, 1, 1, 128, 128, 64, 1, 128, 32, None, fake, 1, 0, fake, 5248, fake, 512, 1, None)
+    rc = lib.kitty_quant_pack_k(fake, 32768, 32768, 256, 1, 1, 128, 128, 64, 1, 128, 32, None, fake, 1, 0, fake, 5248, fake, 512, 1, None, None)
     assert rc == E_RANGE and b"exceed" in lib.kitty_last_error()
-    rc = lib.kitty_quant_pack_k(ctypes.c_void_p(4098), 32768, 32768, 256, 1, 1, 128, 128, 0, 1, 128, 32, None, fake, 1, 0, fake, 5248, fake, 512, 1, None)
+    rc = lib.kitty_quant_pack_k(ctypes.c_void_p(4098), 32768, 32768, 256, 1, 1, 128, 128, 0, 1, 128, 32, None, fake, 1, 0, fake, 5248, fake, 512, 1, None, None)
     assert rc == E_ALIGN
     rc = lib.kitty_select_boost_k(fake, 32768, 32768, 256, 1, 1, 128, 128, 0, 1, 128, 129, fake, None)
     assert rc == E_SHAPE
@@ -89,26 +89,44 @@ def test_host_side_rejection_without_gpu(lib):
     L.D = 64
     assert lib.kitty_decode_attn(*args(4, fake, 1 << 20, 4)) == E_SHAPE
     L.D = 128
-    assert lib.kitty_append_token(ctypes.byref(L), fake, fake, 256, 256, 1, None) == E_NULL    # no seq_counts
+    L.cache_pages_k = -1                                                           # a negative page count
+    assert lib.kitty_decode_attn(*args(4, fake, 1 << 20, 4)) == E_RANGE
+    L.cache_pages_k, L.counts[1], L.counts[2] = 0, 1, 0                            # a packed page but no page array
+    L.counts[5] = 128
+    assert lib.kitty_decode_attn(*args(4, fake, 1 << 20, 4)) == E_RANGE and b"cache_pages" in lib.kitty_last_error()
+    L.counts[1] = L.counts[5] = 0
+    L.cache_pages_k = L.cache_pages_v = 4
+    tok = lambda k, v, sb, sh, B, cos=None, sin=None, rs=0: lib.kitty_append_token(ctypes.byref(L), k, v, sb, sh, cos, sin, rs, B, None)
+    assert tok(fake, fake, 256, 256, 1) == E_NULL    # no seq_counts
     assert b"seq_counts" in lib.kitty_last_error()
-    assert lib.kitty_flush_full(ctypes.byref(L), 1, 4, None) == E_NULL
+    assert lib.kitty_flush_full(ctypes.byref(L), 1, None) == E_NULL
+    assert lib.kitty_append_chunk(ctypes.byref(L), fake, fake, 32768, 32768, 256, 1, 8, None) == E_NULL
     L.seq_counts = 4096
-    assert lib.kitty_append_token(ctypes.byref(L), None, fake, 256, 256, 1, None) == E_NULL
-    assert lib.kitty_append_token(ctypes.byref(L), fake, fake, 250, 256, 1, None) == E_ALIGN
-    assert lib.kitty_append_token(ctypes.byref(L), fake, fake, 256, 256, 0, None) == E_RANGE
-    assert lib.kitty_flush_full(ctypes.byref(L), 1, -1, None) == E_RANGE
+    assert tok(None, fake, 256, 256, 1) == E_NULL
+    assert tok(fake, fake, 250, 256, 1) == E_ALIGN
+    assert tok(fake, fake, 256, 256, 0) == E_RANGE
+    assert tok(fake, fake, 256, 256, 1, cos=fake) == E_NULL and b"rope" in lib.kitty_last_error()   # cos without sin
+    assert tok(fake, fake, 256, 256, 1, cos=fake, sin=fake, rs=100) == E_ALIGN
+    assert lib.kitty_append_chunk(ctypes.byref(L), fake, fake, 32768, 32768, 256, 1, 0, None) == E_RANGE
+    assert lib.kitty_append_chunk(ctypes.byref(L), fake, fake, 32768, 32768, 250, 1, 8, None) == E_ALIGN
+    L.cache_pages_v = -3
+    assert lib.kitty_flush_full(ctypes.byref(L), 1, None) == E_RANGE
+    L.cache_pages_v = 4
     L.PAGE_SIZE = 256
-    assert lib.kitty_flush_full(ctypes.byref(L), 1, 4, None) == E_SHAPE
+    assert lib.kitty_flush_full(ctypes.byref(L), 1, None) == E_SHAPE
     assert lib.kitty_decode_attn_workspace_bytes(16, 32, 128, 16) == 16 * 32 * 16 * 2 * 4 + 16 * 32 * 16 * 128 * 4
     assert lib.kitty_decode_attn_workspace_bytes(16, 32, 64, 16) == 0
-    assert 1 <= lib.kitty_decode_attn_default_splits(16, 8, 257) <= 257
-    assert lib.kitty_decode_attn_default_splits(1, 8, 1025) > lib.kitty_decode_attn_default_splits(16, 8, 1025)
-    # long splits: two waves per SIMD of the 256 CUs; short splits (under 8 tiles): 15/16 of that;
-    # never fewer than 4 tiles per body split
-    assert lib.kitty_decode_attn_default_splits(16, 8, 257) == 16
-    assert lib.kitty_decode_attn_default_splits(1, 8, 1025) == 240
-    assert lib.kitty_decode_attn_default_splits(1, 8, 33) == 33 // 4 + 1 + 3
-    assert lib.kitty_decode_attn_default_splits(0, 8, 33) == 1
+    ds = lib.kitty_decode_attn_default_splits
+    assert 1 <= ds(16, 8, 257, 0) <= 257
+    assert ds(1, 8, 1025, 0) > ds(16, 8, 1025, 0)
+    # long splits: two waves per SIMD of the device (256 compute units when there is none to ask); short
+    # splits (under 8 tiles): 15/16 of that; never fewer than 4 tiles per body split; at least 12
+    # for long sequences with their own lengths
+    assert ds(16, 8, 257, 0) == 16
+    assert ds(1, 8, 1025, 0) == 240
+    assert ds(1, 8, 33, 0) == 33 // 4 + 1 + 3
+    assert ds(0, 8, 33, 0) == 1
+    assert ds(64, 8, 131, 0) == 4 and ds(64, 8, 131, 1) == 12 and ds(64, 8, 40, 1) == 4
 
 
 def test_missing_library_fails_loudly(monkeypatch, tmp_path):

@@ -164,8 +164,8 @@ def test_skipped_flush_drops_the_token_instead_of_overrunning(K):
     L.enable_device_counters(torch.tensor([[32, 0, 128, 0, 0, 128, 0, 0], [32, 0, 127, 0, 0, 127, 0, 0]], dtype=torch.int32))
     k = torch.ones(B, H_KV, 1, 128, dtype=torch.float16, device="cuda")
     snapshot = [t.clone() for t in (L.Q_Buffer_K, L.Q_Buffer_V, L.Local_Buffer_V, L.Sink_Buffer_K)]
-    rc = K.lib.lib().kitty_append_token(L.descriptor(), k.data_ptr(), k.data_ptr(), k.stride(0) * 2, k.stride(1) * 2, B,
-                                        K.lib.current_stream_ptr(k.device))
+    rc = K.lib.lib().kitty_append_token(L.descriptor(), k.data_ptr(), k.data_ptr(), k.stride(0) * 2, k.stride(1) * 2,
+                                        None, None, 0, B, K.lib.current_stream_ptr(k.device))
     assert rc == 0
     torch.cuda.synchronize()
     assert L.seq_counts.cpu().tolist() == [[32, 0, 128, 0, 0, 128, 0, 0], [32, 0, 128, 0, 0, 128, 0, 0]]
@@ -179,18 +179,17 @@ def test_device_counter_calls_reject_bad_arguments(K):
     k = torch.zeros(2, 1, 1, 128, dtype=torch.float16, device="cuda")
     lib = K.lib.lib()
     st = K.lib.current_stream_ptr(k.device)
-    assert lib.kitty_append_token(L.descriptor(), k.data_ptr(), k.data_ptr(), 256, 256, 2, st) == -1   # no seq_counts
+    assert lib.kitty_append_token(L.descriptor(), k.data_ptr(), k.data_ptr(), 256, 256, None, None, 0, 2, st) == -1   # no seq_counts
     assert b"seq_counts" in lib.kitty_last_error()
-    assert lib.kitty_flush_full(L.descriptor(), 2, L.KeyCache.size(0), st) == -1
+    assert lib.kitty_flush_full(L.descriptor(), 2, st) == -1
     with pytest.raises(ValueError):
         L.enable_device_counters(torch.zeros(3, 8, dtype=torch.int32))
     with pytest.raises(ValueError):
         L.enable_device_counters(torch.tensor([[32, 0, 5, 0, 0, 4, 0, 0]] * 2, dtype=torch.int32))   # K != V length
     L.enable_device_counters()
-    assert lib.kitty_append_token(L.descriptor(), None, k.data_ptr(), 256, 256, 2, st) == -1
-    assert lib.kitty_append_token(L.descriptor(), k.data_ptr() + 2, k.data_ptr(), 256, 256, 2, st) == -4
-    with pytest.raises(NotImplementedError):
-        c.append(k, k, 0)
+    assert lib.kitty_append_token(L.descriptor(), None, k.data_ptr(), 256, 256, None, None, 0, 2, st) == -1
+    assert lib.kitty_append_token(L.descriptor(), k.data_ptr() + 2, k.data_ptr(), 256, 256, None, None, 0, 2, st) == -4
+    assert lib.kitty_append_chunk(L.descriptor(), k.data_ptr() + 2, k.data_ptr(), 256, 256, 256, 2, 1, st) == -4
 
 
 def test_decode_step_replays_from_one_captured_graph(K):

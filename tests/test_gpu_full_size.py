@@ -8,7 +8,7 @@ import pytest
 import torch
 
 from oracle import kitty_oracle as O
-from tests.test_gpu_parity import ATOL, _check_attn
+from tests.test_gpu_parity import _check_attn
 
 pytestmark = pytest.mark.gpu
 SC = 128 ** -0.5
@@ -28,16 +28,48 @@ def K():
                                synth=staticmethod(bench.synth_kv)))
 
 
-def _sampled_check(K, L, out, q, units, max_len, counts=None, variant=0):
+# Fixed bounds of the matrix-core kernel against the reference's two fp16 readings of the
+# dequantization at the full shapes (tests/test_gpu_parity.py::_check_attn), per config:
+# (bound against "two", bound against "fma"); measured on the sampled units 6.1e-3 / 7.2e-4 (config 1),
+# 1.0e-2 / 3.1e-3 (config 2: peaked softmaxes, where "two" and "fma" themselves sit 1.3e-2 apart),
+# 2.9e-3 / 1.6e-3 (config 4), each with a quarter on top.  Against the affine value: 2e-3 everywhere.
+TOLS = {"c1": (7.5e-3, 1.0e-3), "c2": (1.3e-2, 4.0e-3), "c4": (3.7e-3, 2.0e-3)}
+
+
+def _sampled_check(K, L, out, q, units, max_len, config, counts=None, variant=0):
     G = q.shape[1] // L.H_KV
     for b, h in units:
         ol = K.u.oracle_head_view(L, b, h, max_len, None if counts is None else counts[b][:7])
         qs = q[b:b + 1, h * G:(h + 1) * G].cpu().numpy()
         got = out[b:b + 1, :, h * G:(h + 1) * G].cpu().numpy().astype(np.float64)
-        _check_attn(got, ol, qs, what=f"b={b} h={h}", variant=variant)
+        _check_attn(got, ol, qs, what=f"b={b} h={h}", variant=variant, tol_two=TOLS[config][0], tol_fma=TOLS[config][1])
 
 
-def _properties(K, mod, q, L, out0, max_len, counts=None):
+def _sampled_quantizer_check(L, k, v, units):
+    """Sampled (sequence, kv head, page) units of a prefilled full-size cache against the oracle's
+    quantizer on the same source rows: packed K bytes (both planes and the slot map), packed V bytes
+    and both sets of (scale, zero) pairs, bit for bit.  K page p holds tokens 32 + 128 p ..; so does V
+    page p (the V side lags by the 128 rows of the ring, but starts at the same token)."""
+    lay = O.Layout(H_KV=L.H_KV)
+    for b, h, page in units:
+        assert page < L.PageCount_V <= L.PageCount_K
+        pg = b * L.MAX_PAGE + page
+        lo = L.S + page * 128
+        xk = k[b:b + 1, h:h + 1, lo:lo + 128].cpu().numpy()
+        xv = v[b:b + 1, h:h + 1, lo:lo + 128].cpu().numpy()
+        oc, om = np.zeros((1, lay.k_stride_h), np.uint8), np.zeros((1, 1, 128, 2), np.float16)
+        O.quantize_pack_k(xk, 0, 1, np.zeros((1, 1), np.int64), 0, oc, om, 128, 32)
+        got = L.KeyCache[pg, h * lay.k_stride_h:(h + 1) * lay.k_stride_h].cpu().numpy()
+        assert np.array_equal(got, oc[0]), ("K bytes", b, h, page)
+        assert np.array_equal(L.KeyCache_metadata[pg, h].cpu().numpy().view(np.uint16), om[0, 0].view(np.uint16)), (b, h, page)
+        oc, om = np.zeros((1, lay.v_stride_h), np.uint8), np.zeros((1, 1, 128, 2), np.float16)
+        O.quantize_pack_v(xv, 0, 1, np.zeros((1, 1), np.int64), 0, oc, om, 128)
+        got = L.ValueCache[pg, h * lay.v_stride_h:(h + 1) * lay.v_stride_h].cpu().numpy()
+        assert np.array_equal(got, oc[0]), ("V bytes", b, h, page)
+        assert np.array_equal(L.ValueCache_metadata[pg, h].cpu().numpy().view(np.uint16), om[0, 0].view(np.uint16)), (b, h, page)
+
+
+def _properties(K, mod, q, L, out0, max_len, config, counts=None):
     a = out0.float()
     for splits in (1, 5):
         o, _ = K.attn(mod, q, L, SC, num_splits=splits)
@@ -51,8 +83,8 @@ def _properties(K, mod, q, L, out0, max_len, counts=None):
     d = (o1.float() - a).abs()
     b, _, hq, _ = np.unravel_index(d.flatten().argmax().item(), tuple(d.shape))
     unit = [(int(b), int(hq) // (q.shape[1] // L.H_KV))]
-    _sampled_check(K, L, out0, q, unit, max_len, counts=counts, variant=0)
-    _sampled_check(K, L, o1, q, unit, max_len, counts=counts, variant=1)
+    _sampled_check(K, L, out0, q, unit, max_len, config, counts=counts, variant=0)
+    _sampled_check(K, L, o1, q, unit, max_len, config, counts=counts, variant=1)
 
 
 def test_config1_full_size(K):
@@ -63,12 +95,13 @@ def test_config1_full_size(K):
     cache.quantize_prefill(0)
     L = cache.kv_cache[0]
     assert (L.PageCount_K, L.PageCount_V, L.Q_Buffer_Count_K, L.Q_Buffer_Count_V, L.Local_Count_V) == (255, 254, 96, 96, 128)
+    _sampled_quantizer_check(L, k, v, [(0, 0, 0), (3, 5, 17), (9, 2, 128), (15, 7, 253)])
     q = torch.randn(B, H_Q, 1, 128, device="cuda", generator=torch.Generator(device="cuda").manual_seed(1)).half()
     mod = K.u.module(H_KV, H_Q)
     out, _ = K.attn(mod, q, L, SC)
     assert torch.isfinite(out.float()).all()
-    _sampled_check(K, L, out, q, [(0, 0), (7, 3), (15, 7)], T + 256)
-    _properties(K, mod, q, L, out, T + 256)
+    _sampled_check(K, L, out, q, [(0, 0), (7, 3), (15, 7)], T + 256, "c1")
+    _properties(K, mod, q, L, out, T + 256, "c1")
 
 
 def test_config4_full_size(K):
@@ -79,12 +112,13 @@ def test_config4_full_size(K):
     cache.quantize_prefill(0)
     L = cache.kv_cache[0]
     assert (L.PageCount_K, L.PageCount_V, L.Q_Buffer_Count_K) == (1023, 1022, 96)
+    _sampled_quantizer_check(L, k, v, [(0, 0, 0), (0, 3, 511), (0, 7, 1021)])
     q = torch.randn(B, H_Q, 1, 128, device="cuda", generator=torch.Generator(device="cuda").manual_seed(4)).half()
     mod = K.u.module(H_KV, H_Q)
     out, _ = K.attn(mod, q, L, SC)
     assert torch.isfinite(out.float()).all()
-    _sampled_check(K, L, out, q, [(0, 2), (0, 7)], T + 256)
-    _properties(K, mod, q, L, out, T + 256)
+    _sampled_check(K, L, out, q, [(0, 2), (0, 7)], T + 256, "c4")
+    _properties(K, mod, q, L, out, T + 256, "c4")
 
 
 def test_config2_full_size_ragged(K):
@@ -96,6 +130,7 @@ def test_config2_full_size_ragged(K):
     cache.update(k, v, 0)
     cache.quantize_prefill(0)
     L = cache.kv_cache[0]
+    _sampled_quantizer_check(L, k, v, [(0, 1, 3), (31, 6, 64), (63, 7, L.PageCount_V - 1)])
     rng = np.random.default_rng(1002)
     counts = []
     for b in range(B):
@@ -109,5 +144,5 @@ def test_config2_full_size_ragged(K):
     mod = K.u.module(H_KV, H_Q)
     out, _ = K.attn(mod, q, L, SC)
     assert torch.isfinite(out.float()).all()
-    _sampled_check(K, L, out, q, [(0, 0), (31, 5), (63, 7)], Tmax + 256, counts=counts)
-    _properties(K, mod, q, L, out, Tmax + 256, counts=counts)
+    _sampled_check(K, L, out, q, [(0, 0), (31, 5), (63, 7)], Tmax + 256, "c2", counts=counts)
+    _properties(K, mod, q, L, out, Tmax + 256, "c2", counts=counts)

@@ -242,20 +242,30 @@ def _build(K, B, H_KV, H_Q, T, max_len, seed, student_t=False):
     return cache, ol
 
 
-def _check_attn(got, ol, q, seq_counts=None, what="", variant=0, elementwise=True):
-    """Tolerance: max-abs 2e-3 (fp16 outputs) against dequantize-then-attend in float64 over the
-    same packed cache.
+# Fixed bounds of the matrix-core kernel (variant 0) against the two fp16 readings of the reference's
+# dequantization, for inputs of the tests' small shapes; the full-size configs pass their own (see
+# tests/test_gpu_full_size.py).  Measured worst cases over this file: 7.8e-3 against "two", 3.2e-3
+# against "fma", 9.8e-4 against "affine"; the bounds leave a quarter on top.
+TOL_TWO, TOL_FMA = 1.0e-2, 4.0e-3
 
-    How a page is dequantized is itself ambiguous at that level on outlier-heavy keys: the
-    reference's expression fp16(code)*scale+zero rounds twice when evaluated eagerly or by the
-    Triton interpreter ("two") and once when a compiler contracts it ("fma"); both approximate the
-    unrounded affine value ("affine"), and the modes sit 1-2e-3 apart from each other on the
-    BASELINE data.  The plain kernel (variant 1) implements "two" and must meet 2e-3 against it.
-    The matrix-core kernel (variant 0) evaluates the affine value: it is held to 2e-3 against
-    "affine" overall and, element by element, to 7.5e-4 plus one fp16 ulp of the value (the output
-    is fp16, and the probabilities enter the PV product as fp16(fp16(p) * scale_v): weights off by
-    up to 2^-10 relative, which shows when a few tokens dominate); against "two" to 2e-3 + d, d being the measured distance between those two oracles
-    on the same inputs."""
+
+def _check_attn(got, ol, q, seq_counts=None, what="", variant=0, elementwise=True, tol_two=TOL_TWO, tol_fma=TOL_FMA):
+    """The tolerance contract of decode attention: max-abs error of the fp16 outputs against
+    dequantize-then-attend in float64 over the same packed cache, with constants only.
+
+    How a page is dequantized is itself ambiguous at the 2e-3 level on outlier-heavy keys: the
+    reference's expression fp16(code)*scale+zero (kitty_attention.py:162-165, 317-320) rounds twice
+    when evaluated eagerly or by the Triton interpreter ("two") and once when a compiler contracts
+    it into an FMA ("fma"); both approximate the unrounded affine value ("affine"), and the two
+    fp16 readings sit up to 1.3e-2 apart from EACH OTHER on the BASELINE data (config 2).
+
+    * The plain kernel (variant 1) implements "two": 2e-3 against it.
+    * The matrix-core kernel (variant 0) evaluates the affine value: 2e-3 against "affine" overall and,
+      element by element, 7.5e-4 plus one fp16 ulp of the value (the output is fp16, and the
+      probabilities enter the PV product as fp16(fp16(p) * scale_v)).  Against the reference's two
+      fp16 readings it is held to the fixed bounds ``tol_two`` / ``tol_fma``: what was measured on the
+      case, plus a quarter, so that a regression shows.
+    Returns the error against the kernel's own reading."""
     kw = dict(seq_counts=seq_counts, reference_rounding=False)
     two = O.decode_attention(ol, q, 128 ** -0.5, dequant="two", **kw)
     err_two = np.abs(got - two).max()
@@ -263,12 +273,13 @@ def _check_attn(got, ol, q, seq_counts=None, what="", variant=0, elementwise=Tru
         assert err_two <= ATOL, f"{what}: {err_two:.3e} vs float64 attention over fp16-dequantized KV"
         return err_two
     affine = O.decode_attention(ol, q, 128 ** -0.5, dequant="affine", **kw)
-    d = np.abs(two - affine).max()
     err_affine = np.abs(got - affine).max()
     assert err_affine <= ATOL, f"{what}: {err_affine:.3e} vs float64 attention over affine-dequantized KV"
     excess = (np.abs(got - affine) - (7.5e-4 + 2.0 ** -10 * np.abs(affine))).max() if elementwise else 0.0
     assert excess <= 0, f"{what}: {excess:.3e} beyond 7.5e-4 + one fp16 ulp of the affine value"
-    assert err_two <= ATOL + d, f"{what}: {err_two:.3e} vs fp16-dequantized KV (modes differ by {d:.3e})"
+    assert err_two <= tol_two, f"{what}: {err_two:.3e} vs twice-rounded fp16 dequantization (bound {tol_two:.1e})"
+    err_fma = np.abs(got - O.decode_attention(ol, q, 128 ** -0.5, dequant="fma", **kw)).max()
+    assert err_fma <= tol_fma, f"{what}: {err_fma:.3e} vs once-rounded fp16 dequantization (bound {tol_fma:.1e})"
     return err_affine
 
 

@@ -15,6 +15,47 @@ def _tiny_llama(attn):
     return LlamaForCausalLM(cfg)
 
 
+def _tiny_qwen3(attn):
+    from transformers import Qwen3Config, Qwen3ForCausalLM
+    cfg = Qwen3Config(vocab_size=256, hidden_size=256, intermediate_size=512, num_hidden_layers=2,
+                      num_attention_heads=4, num_key_value_heads=1, head_dim=128, max_position_embeddings=4096,
+                      attn_implementation=attn)
+    torch.manual_seed(0)
+    return Qwen3ForCausalLM(cfg)
+
+
+class _DecodeCapture:
+    """Stands in for the decode-attention call of the hook and checks every call it sees against the
+    CPU oracle: the layer's bytes at that moment (after update, before quantize_decode) are copied
+    into an oracle layer, and the kernel's output for the query the model really produced is held to
+    the contract of tests/test_gpu_parity.py (max-abs 2e-3 against dequantize-then-attend)."""
+
+    def __init__(self, hf, max_len, every=1):
+        self.hf, self.max_len, self.every, self.calls, self.worst = hf, max_len, every, 0, 0.0
+
+    def __enter__(self):
+        from tests import gpu_util
+        from tests.test_gpu_parity import _check_attn
+        self.orig = self.hf.kitty_attention_forward
+
+        def checked(module, query, layer, scaling, **kw):
+            out, w = self.orig(module, query, layer, scaling, **kw)
+            self.calls += 1
+            if self.calls % self.every == 0:
+                assert abs(scaling - 128 ** -0.5) < 1e-9
+                ol = gpu_util.oracle_from_layer(layer, self.max_len)
+                got = out.detach().cpu().numpy().astype(np.float64)
+                self.worst = max(self.worst, _check_attn(got, ol, query.detach().cpu().numpy(), what=f"call {self.calls}"))
+            return out, w
+
+        self.hf.kitty_attention_forward = checked
+        return self
+
+    def __exit__(self, *exc):
+        self.hf.kitty_attention_forward = self.orig
+        return False
+
+
 def test_register_and_cache_adapter_on_cpu():
     from kitty_amd import hf
     hf.register()
@@ -88,7 +129,8 @@ def test_stock_llama_long_prompt_decode_and_chunk():
     c_ref, c_mod = DynamicCache(), hf.KittyHFCache(mod.config, B, 1024, device=dev)
     ol = O.OracleLayer(B, 1024, 1)                                  # counters only: the state machine
     zeros = lambda n: np.zeros((B, 1, n, 128), np.float16)
-    with torch.no_grad():
+    # every 7th decode-attention call of the model (both layers, across the flushes) against the oracle
+    with torch.no_grad(), _DecodeCapture(hf, 1024, every=7) as cap:
         cur, cos = ids, []
         for s in range(steps + 1):
             a = ref(input_ids=cur, past_key_values=c_ref, use_cache=True).logits[:, -1].float()
@@ -114,6 +156,90 @@ def test_stock_llama_long_prompt_decode_and_chunk():
     # dense attention's (random weights leave the argmax itself nearly tied, so it is not compared)
     print("cosine similarity of the logits: min %.4f mean %.4f" % (min(cos), sum(cos) / len(cos)))
     assert min(cos) >= 0.97, min(cos)
+    assert cap.calls == 2 * steps and cap.worst <= 2e-3
+    print("decode attention inside the model vs oracle: worst max-abs error %.2e over %d checked calls"
+          % (cap.worst, cap.calls // 7))
+
+
+@pytest.mark.gpu
+def test_stock_qwen3_on_the_hook():
+    """The reference's own model family (per-head q/k RMS norm before the rotation,
+    modeling_qwen3.py:214-215) as the stock transformers module: dense agreement while everything is
+    fp16, then a packed prompt with decode steps whose attention calls are checked against the oracle
+    on the queries and caches the model really produced, and generate() as the reference's benchmark
+    drives it (fresh cache, greedy, no early stop: benchmark_kitty.py:131-149)."""
+    if not torch.cuda.is_available():
+        pytest.skip("needs a GPU")
+    from transformers import DynamicCache
+    from kitty_amd import hf
+    hf.register()
+    dev = torch.device("cuda")
+    ref = _tiny_qwen3("sdpa").to(dev).half().eval()
+    mod = _tiny_qwen3("kitty").to(dev).half().eval()
+    mod.load_state_dict(ref.state_dict())
+    g = torch.Generator().manual_seed(5)
+    with torch.no_grad():
+        # (i) 20 + 40 tokens: nothing is quantized
+        B = 2
+        ids = torch.randint(0, 256, (B, 20), generator=g).to(dev)
+        c_ref, c_mod = DynamicCache(), hf.KittyHFCache(mod.config, B, 512, device=dev)
+        cur = ids
+        for s in range(41):
+            a = ref(input_ids=cur, past_key_values=c_ref, use_cache=True).logits[:, -1].float()
+            b = mod(input_ids=cur, past_key_values=c_mod, use_cache=True).logits[:, -1].float()
+            assert torch.isfinite(b).all() and (a - b).abs().max().item() <= 3e-2, (s, (a - b).abs().max().item())
+            cur = a.argmax(-1, keepdim=True)
+        # (ii) a packed prompt, decode across a K flush, every 5th attention call against the oracle
+        ids = torch.randint(0, 256, (B, 32 + 128 * 2 + 100), generator=g).to(dev)
+        cache = hf.KittyHFCache(mod.config, B, 1024, device=dev)
+        with _DecodeCapture(hf, 1024, every=5) as cap:
+            cur = mod(input_ids=ids, past_key_values=cache, use_cache=True).logits[:, -1].float().argmax(-1, keepdim=True)
+            for s in range(60):
+                out = mod(input_ids=cur, past_key_values=cache, use_cache=True).logits[:, -1].float()
+                assert torch.isfinite(out).all()
+                cur = out.argmax(-1, keepdim=True)
+        L = cache.kv_cache[1]
+        assert cap.calls == 2 * 60 and cap.worst <= 2e-3
+        assert (L.PageCount_K, L.Q_Buffer_Count_K, L.PageCount_V) == (3, 32, 2)
+        # (iii) generate() with a fresh cache, as the reference's benchmark calls it
+        gen_cache = hf.KittyHFCache(mod.config, B, 1024, device=dev)
+        got = mod.generate(input_ids=ids, max_length=ids.shape[1] + 40, max_new_tokens=None, do_sample=False,
+                           temperature=None, top_p=None, top_k=None, past_key_values=gen_cache, eos_token_id=None,
+                           pad_token_id=0, disable_compile=True)
+        assert tuple(got.shape) == (B, ids.shape[1] + 40) and torch.equal(got[:, :ids.shape[1]], ids)
+        assert gen_cache.get_seq_length(0) == ids.shape[1] + 39
+        gen_cache.check_status()
+
+
+@pytest.mark.gpu
+def test_chunk_through_the_hook_with_device_counters():
+    """Several new tokens per sequence over a packed cache with the counters on the device: chunk
+    attention, then the device-side chunk append; the logits are those of the host-counter cache."""
+    if not torch.cuda.is_available():
+        pytest.skip("needs a GPU")
+    from kitty_amd import hf
+    hf.register()
+    dev = torch.device("cuda")
+    mod = _tiny_llama("kitty").to(dev).half().eval()
+    B, T0 = 2, 32 + 128 + 90
+    g = torch.Generator().manual_seed(6)
+    ids = torch.randint(0, 256, (B, T0), generator=g).to(dev)
+    host, devc = (hf.KittyHFCache(mod.config, B, 1024, device=dev) for _ in range(2))
+    with torch.no_grad():
+        mod(input_ids=ids, past_key_values=host, use_cache=True)
+        mod(input_ids=ids, past_key_values=devc, use_cache=True)
+        devc.enable_device_counters()
+        for n in (50, 1, 200):
+            more = torch.randint(0, 256, (B, n), generator=g).to(dev)
+            a = mod(input_ids=more, past_key_values=host, use_cache=True).logits
+            b = mod(input_ids=more, past_key_values=devc, use_cache=True).logits
+            assert torch.equal(a, b), n
+    torch.cuda.synchronize()
+    assert devc.get_seq_length(0) == host.get_seq_length(0) == T0 + 251
+    for lh, ld in zip(host.kv_cache, devc.kv_cache):
+        assert ld.seq_counts.cpu().tolist() == [lh.counts()] * B
+        assert torch.equal(lh.KeyCache, ld.KeyCache) and torch.equal(lh.ValueCache, ld.ValueCache)
+    devc.check_status()
 
 
 @pytest.mark.gpu

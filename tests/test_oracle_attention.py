@@ -115,3 +115,28 @@ def test_sim_baseline_shapes_and_levels():
     assert len(torch.unique(V[0, 0, 40].float())) <= 4
     out = S.eager_attention(torch.randn(1, 8, 1, 128).half(), K, V, 128 ** -0.5, 4)
     assert tuple(out.shape) == (1, 1, 8, 128)
+
+
+def test_rope_restatement_equals_torch_fp16_operators():
+    """oracle.rope_fp16 against the caller's expression evaluated by torch's own fp16 operators
+    (modeling_qwen3.py:98-102, 125-128: q * cos + rotate_half(q) * sin on fp16 tensors), bit for bit,
+    and the two closed forms a rotation has: angle 0 is the identity, angle pi/2 swaps the halves."""
+    import torch
+    rng = np.random.default_rng(5)
+    B, H, T, D = 3, 2, 4, 128
+    x = (rng.standard_normal((B, H, T, D)) * 4).astype(np.float16)
+    pos = rng.integers(0, 100000, size=(B, T)).astype(np.float64)
+    inv = 1.0 / (500000.0 ** (np.arange(0, D, 2) / D))
+    ang = pos[..., None] * inv
+    cos = np.concatenate([np.cos(ang), np.cos(ang)], -1).astype(np.float16)       # [B, T, D]
+    sin = np.concatenate([np.sin(ang), np.sin(ang)], -1).astype(np.float16)
+    got = O.rope_fp16(x, cos, sin)
+    xt, ct, st = torch.from_numpy(x), torch.from_numpy(cos).unsqueeze(1), torch.from_numpy(sin).unsqueeze(1)
+    rot = torch.cat((-xt[..., D // 2:], xt[..., : D // 2]), dim=-1)
+    want = (xt * ct) + (rot * st)
+    assert want.dtype == torch.float16
+    assert np.array_equal(got.view(np.uint16), want.numpy().view(np.uint16))
+    one, zero = np.ones((B, T, D), np.float16), np.zeros((B, T, D), np.float16)
+    assert np.array_equal(O.rope_fp16(x, one, zero), x)
+    quarter = O.rope_fp16(x, zero, one)
+    assert np.array_equal(quarter[..., : D // 2], -x[..., D // 2:]) and np.array_equal(quarter[..., D // 2:], x[..., : D // 2])

@@ -125,3 +125,62 @@ def test_paged_cache_bookkeeping_before_any_launch():
     with pytest.raises(ValueError):                        # a pool needs its owner's page tables
         from kitty_amd.kvcache.utils_kv_per_layer import KVCache_Layer
         KVCache_Layer(2, 1024, 1, 128, 32, 2, 4, 128, 32, device="cpu", n_pages=4)
+
+
+def test_chunk_counts_closed_form_equals_single_steps():
+    """KittyCache.chunk_counts (the host's copy of what the device's chunk kernels compute) against
+    the oracle stepping token by token, from every phase of the state machine."""
+    from kitty_amd.kvcache.kitty import KittyCache
+    names = ("sink", "pk", "rk", "pv", "rv", "lv", "off")
+    for T0 in (1, 31, 32, 33, 32 + 127, 32 + 128, 32 + 129, 32 + 128 * 2 + 5):
+        for warm in (0, 140):
+            for T in (1, 2, 31, 96, 127, 128, 129, 300):
+                k, v = make_kv(1, 1, T0 + warm + T, seed=T0 + T)
+                ol = O.OracleLayer(1, 2048, 1)
+                ol.update(k[:, :, :T0], v[:, :, :T0])
+                ol.quantize_prefill()
+                for s in range(warm + T):
+                    if s == warm:
+                        before = dict(zip(names, [getattr(ol, f) for f in FIELDS]))
+                    ol.update(k[:, :, T0 + s:T0 + s + 1], v[:, :, T0 + s:T0 + s + 1])
+                    ol.quantize_decode()
+                after = KittyCache.chunk_counts(before, T, 32, 128)
+                assert [after[n] for n in names] == [getattr(ol, f) for f in FIELDS], (T0, warm, T)
+
+
+def test_paged_decode_batch_must_be_all_slots():
+    import torch
+    cache = PagedKittyCache(_cfg(), 4, 1024, pool_pages=8, device="cpu")
+    k = torch.zeros(2, 2, 1, 128, dtype=torch.float16)
+    with pytest.raises(ValueError, match="all 4 slots"):   # before anything is launched
+        cache.update(k, k, 0)
+
+
+def test_paged_chunk_reserves_its_pages_before_the_first_launch():
+    cache = PagedKittyCache(_cfg(), 3, 32 + 128 * 6, pool_pages=9, device="cpu")
+    # two sequences as an admission leaves them: counters in the shadow, pages up to the next flush's
+    for slot, T0 in ((0, 32 + 128 + 100), (2, 10)):
+        cache._take_for_admission(slot, T0)
+        n = __import__("kitty_amd.kvcache.kitty", fromlist=["prefill_split"]).prefill_split(T0, 32, 128)
+        cache._shadow[slot] = [n["sink"], n["pages_k"], n["qbuf_k"], n["pages_v"], n["qbuf_v"], n["local_v"], 0, 0]
+        cache._active[slot] = True
+    cache.check_tables()
+    assert cache.pages_in_use() == (3, 2)                  # slot 0: 1 + 1 and 0 + 1; slot 2: 0 + 1 each
+    cache._reserve_for_chunk(200)                          # slot 0: rk 100 + 200 -> 2 more K pages; V 100 + 200 -> 2
+    after = cache._chunk_after(200)
+    assert after[0, :7].tolist() == [32, 3, 44, 2, 44, 128, 200 % 128] and after[2, :7].tolist() == [32, 1, 50, 0, 50, 128, 50]
+    assert after[1].tolist() == cache._shadow[1].tolist()  # the free slot
+    # pages up to and including the one of the flush after the chunk
+    assert (cache._table_k[0] >= 0).sum() == 4 and (cache._table_v[0] >= 0).sum() == 3
+    assert (cache._table_k[2] >= 0).sum() == 2 and (cache._table_v[2] >= 0).sum() == 1
+    cache._end_of_chunk(200)
+    cache.check_tables()
+    assert cache.seq_lengths().tolist() == [32 + 128 + 100 + 200, 0, 210]
+    assert cache.kv_cache[1].get_total_length() == 460
+    used = cache.pages_in_use()
+    with pytest.raises(OutOfPages):                        # 4 more K pages for slot 0 alone, 3 are free
+        cache._reserve_for_chunk(128 * 4)
+    assert cache.pages_in_use() == used
+    cache.check_tables()
+    with pytest.raises(ValueError):                        # beyond max_length
+        cache._reserve_for_chunk(128 * 7)

@@ -122,7 +122,7 @@ def cpu_cache(monkeypatch):
     def rec_k(key_states, t_offset, pages, page_table, page_offset, cache, meta, page_size, d_boost, **kw):
         calls.append(("k", tuple(key_states.shape), t_offset, pages, page_offset, page_size, d_boost))
 
-    def rec_v(value_states, t_offset, pages, page_table, page_offset, cache, meta, page_size):
+    def rec_v(value_states, t_offset, pages, page_table, page_offset, cache, meta, page_size, **kw):
         calls.append(("v", tuple(value_states.shape), t_offset, pages, page_offset, page_size))
 
     monkeypatch.setattr(kmod, "quantize_pack_k", rec_k)
@@ -225,7 +225,7 @@ def cpu_cache_oracle_quant(monkeypatch):
         O.quantize_pack_k(key_states.numpy(), t_offset, pages, page_table.numpy(), page_offset, cache.numpy(),
                           meta.numpy(), page_size, d_boost)
 
-    def qv(value_states, t_offset, pages, page_table, page_offset, cache, meta, page_size):
+    def qv(value_states, t_offset, pages, page_table, page_offset, cache, meta, page_size, **kw):
         O.quantize_pack_v(value_states.numpy(), t_offset, pages, page_table.numpy(), page_offset, cache.numpy(),
                           meta.numpy(), page_size)
 
