@@ -3,7 +3,7 @@
  *
  * Every entry point is asynchronous and ordered on the HIP stream passed in (NULL = the default
  * stream), allocates nothing, frees nothing and keeps no state between calls except a thread-local
- * error string.  All data pointers are device pointers owned by the caller.  Return value: 0 on
+ * error string (kitty_decode_attn_static also remembers where its array lies on each device).  All data pointers are device pointers owned by the caller.  Return value: 0 on
  * success, a negative KITTY_E_* code when an argument is rejected on the host before anything is
  * launched, a positive hipError_t when a launch fails.  kitty_last_error() describes the last
  * failure on the calling thread.
@@ -187,6 +187,22 @@ int kitty_decode_attn_merge(const void* workspace, size_t workspace_bytes, int B
  * (NULL, NULL) cancels.  The plain variant records the events around its launch instead.
  */
 int kitty_profile_next_split(void* start_event, void* stop_event);
+
+/*
+ * kitty_decode_attn without a workspace argument and without any allocation: the split-K partials
+ * go to an array of KITTY_STATIC_WORKSPACE_BYTES that is part of the library's device image (one copy
+ * per device, held until the process ends).  No counterpart in the reference; it is for callers that
+ * cannot allocate: code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.
+ * Same kernels, same results as kitty_decode_attn with the same num_splits.  num_splits <= 0 picks
+ * kitty_decode_attn's default, cut back to what the array holds; an explicit num_splits whose
+ * partials ((2 + D) floats per batch row, query head and split) exceed the array is rejected with
+ * KITTY_E_WORKSPACE.  The device that owns the tensors must be the current device.  All calls on one
+ * device share the array: calls that overlap there (different streams or threads) race; calls
+ * ordered on one stream do not, and nothing in the array needs clearing between them.
+ */
+#define KITTY_STATIC_WORKSPACE_BYTES (16u << 20)
+int kitty_decode_attn_static(const kitty_kv_layer* layer, const void* q, int B, int H_Q, float scaling,
+                             void* out, int num_splits, int variant, void* stream);
 
 /*
  * Chunked-prefill attention: T_q new tokens attend to everything the layer already holds (sink

@@ -60,6 +60,8 @@ _SIGNATURES = {
     "kitty_profile_next_split": (c_int, [c_void_p, c_void_p]),
     "kitty_decode_attn": (c_int, [POINTER(KittyKVLayer), c_void_p, c_int, c_int, c_float, c_void_p, c_void_p,
                                   c_size_t, c_int, c_int, c_void_p]),
+    "kitty_decode_attn_static": (c_int, [POINTER(KittyKVLayer), c_void_p, c_int, c_int, c_float, c_void_p, c_int, c_int,
+                                         c_void_p]),
     "kitty_prefill_attn": (c_int, [POINTER(KittyKVLayer), c_void_p, c_int64, c_int64, c_int64, c_void_p, c_void_p,
                                    c_int64, c_int64, c_int64, c_int, c_int, c_int, c_float, c_void_p, c_void_p]),
     "kitty_append_token": (c_int, [POINTER(KittyKVLayer), c_void_p, c_void_p, c_int64, c_int64, c_void_p, c_void_p,

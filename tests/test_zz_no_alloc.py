@@ -1,0 +1,101 @@
+"""kitty_decode_attn_static (decode attention whose split-K partials live in the library's own
+device array, for callers that cannot allocate) against kitty_decode_attn with a caller-owned
+workspace: same kernels, so the outputs must be bit-identical.  Two calls in a row, the second on a
+smaller input, then the first again: whatever a call leaves in the shared array must not leak into
+the next."""
+import numpy as np
+import pytest
+import torch
+
+from tests.helpers import make_kv, make_q
+
+pytestmark = pytest.mark.gpu
+SC = 128 ** -0.5
+STATIC_BYTES = 16 << 20
+
+
+@pytest.fixture(scope="module")
+def K():
+    if not torch.cuda.is_available():
+        pytest.skip("needs a GPU")
+    import kitty_amd
+    from kitty_amd import _lib
+    _lib.lib()
+    from tests import gpu_util
+    return type("NS", (), dict(KittyCache=kitty_amd.KittyCache, u=gpu_util, lib=_lib))
+
+
+def _cache(K, B, H_KV, H_Q, T, seed):
+    k, v = make_kv(B, H_KV, T, seed=seed)
+    c = K.KittyCache(K.u.cfg(H_KV, H_Q), B, T + 256)
+    c.update(K.u.to_dev(k), K.u.to_dev(v), 0)
+    c.quantize_prefill(0)
+    return c
+
+
+def _both(K, cache, q, splits, variant=0):
+    """(output through the caller-owned workspace, output through the library's array, return code)"""
+    lib = K.lib.lib()
+    L = cache.kv_cache[0]
+    B, H_Q = q.shape[0], q.shape[1]
+    st = K.lib.current_stream_ptr(q.device)
+    n = splits if splits > 0 else lib.kitty_decode_attn_default_splits(
+        B, L.H_KV, 1 + (L.get_total_length() - L.Sink_Count + 127) // 128, int(L.seq_counts is not None))
+    ws = torch.empty(lib.kitty_decode_attn_workspace_bytes(B, H_Q, 128, n), dtype=torch.uint8, device=q.device)
+    want = torch.full((B, 1, H_Q, 128), 7.0, dtype=torch.float16, device=q.device)
+    got = torch.full_like(want, -7.0)
+    K.lib.check(lib.kitty_decode_attn(L.descriptor(), q.data_ptr(), B, H_Q, SC, want.data_ptr(), ws.data_ptr(),
+                                      ws.numel(), n, variant, st), "kitty_decode_attn")
+    rc = lib.kitty_decode_attn_static(L.descriptor(), q.data_ptr(), B, H_Q, SC, got.data_ptr(), splits, variant, st)
+    torch.cuda.synchronize()
+    return want, got, rc
+
+
+def test_static_entry_point_matches_the_workspace_one_on_calls_in_a_row(K):
+    big = _cache(K, 4, 2, 8, 32 + 128 * 9 + 70, seed=61)
+    small = _cache(K, 2, 2, 8, 32 + 128 * 2 + 5, seed=62)
+    qb = K.u.to_dev(make_q(4, 8, seed=61))
+    qs = K.u.to_dev(make_q(2, 8, seed=62))
+    for cache, q, splits in ((big, qb, 5), (small, qs, 2), (big, qb, 0), (small, qs, 0), (big, qb, 5)):
+        for variant in (0, 1):
+            want, got, rc = _both(K, cache, q, splits, variant)
+            assert rc == 0, K.lib.lib().kitty_last_error()
+            assert torch.equal(want, got), (splits, variant)
+            assert torch.isfinite(got.float()).all()
+
+
+def test_static_entry_point_allocates_nothing(K):
+    """Device memory in use by the process does not move across calls (the first call on a device
+    only asks the runtime where the array lies)."""
+    cache = _cache(K, 2, 2, 8, 32 + 128 * 3, seed=63)
+    q = K.u.to_dev(make_q(2, 8, seed=63))
+    lib = K.lib.lib()
+    L = cache.kv_cache[0]
+    out = torch.empty((2, 1, 8, 128), dtype=torch.float16, device="cuda")
+    st = K.lib.current_stream_ptr(q.device)
+    desc = L.descriptor()
+    assert lib.kitty_decode_attn_static(desc, q.data_ptr(), 2, 8, SC, out.data_ptr(), 3, 0, st) == 0
+    torch.cuda.synchronize()
+    free0, _ = torch.cuda.mem_get_info()
+    for _ in range(20):
+        assert lib.kitty_decode_attn_static(desc, q.data_ptr(), 2, 8, SC, out.data_ptr(), 3, 0, st) == 0
+    torch.cuda.synchronize()
+    free1, _ = torch.cuda.mem_get_info()
+    assert free1 == free0
+
+
+def test_static_entry_point_rejects_what_does_not_fit(K):
+    cache = _cache(K, 2, 2, 8, 32 + 128 * 3, seed=64)
+    q = K.u.to_dev(make_q(2, 8, seed=64))
+    lib = K.lib.lib()
+    L = cache.kv_cache[0]
+    out = torch.zeros((2, 1, 8, 128), dtype=torch.float16, device="cuda")
+    st = K.lib.current_stream_ptr(q.device)
+    per_split = 2 * 8 * (2 + 128) * 4
+    too_many = STATIC_BYTES // per_split + 1
+    assert lib.kitty_decode_attn_static(L.descriptor(), q.data_ptr(), 2, 8, SC, out.data_ptr(), too_many, 0, st) == -5
+    assert b"array holds" in lib.kitty_last_error()
+    assert lib.kitty_decode_attn_static(L.descriptor(), None, 2, 8, SC, out.data_ptr(), 2, 0, st) == -1
+    assert lib.kitty_decode_attn_static(L.descriptor(), q.data_ptr(), 2, 7, SC, out.data_ptr(), 2, 0, st) == -2
+    torch.cuda.synchronize()
+    assert not out.any()
