@@ -42,6 +42,15 @@ __device__ inline SeqCounts load_counts(const kitty_kv_layer& L, int b) {
   return s;
 }
 
+// One entry of a page table.  The tables are not written while an attention kernel runs, and the
+// compiler cannot know that (the global -> LDS loads are memory writes to it, so every later table
+// read counts as possibly changed): read through the constant address space, the entry of a
+// wave-uniform index is a scalar load, which neither occupies the vector memory queue nor makes
+// the wave wait for the tile loads in flight.
+__device__ __forceinline__ int64_t page_id(const int64_t* table, int64_t index) {
+  typedef const int64_t __attribute__((address_space(4)))* const_ptr;
+  return *(const_ptr)(uintptr_t)(table + index);
+}
 // A page id as read from a page table, made safe to dereference.  The counters and tables of a
 // layer may be written by the caller on the device, so the host cannot vouch for them: an id outside
 // [0, cache_pages) (an entry of -1 = no page assigned, or garbage) reads page 0 instead and is noted

@@ -268,7 +268,7 @@ struct KLds {
 template <bool BOOST>
 __device__ __forceinline__ void k_load_regs(const Ctx& x, int page_index, KRegs& kb) {
   const kitty_kv_layer& L = *x.L;
-  const int64_t pg = checked_page(L.page_table_k[(int64_t)x.b * L.page_table_k_stride_b + page_index], L.cache_pages_k, x.bad_page);
+  const int64_t pg = checked_page(page_id(L.page_table_k, (int64_t)x.b * L.page_table_k_stride_b + page_index), L.cache_pages_k, x.bad_page);
   const uint8_t* page = L.key_cache + pg * L.key_cache_stride_page + (int64_t)x.h * k_head_bytes(BOOST ? 32 : 0);
   const uint8_t* meta = (const uint8_t*)L.key_meta + pg * L.key_meta_stride_page + (int64_t)x.h * kD * 4;
 #pragma unroll
@@ -293,7 +293,7 @@ constexpr int kDmaV = 6;
 template <bool BOOST>
 __device__ __forceinline__ void dma_k(const Ctx& x, int page_index, uint32_t lds) {
   const kitty_kv_layer& L = *x.L;
-  const int64_t pg = checked_page(L.page_table_k[(int64_t)x.b * L.page_table_k_stride_b + page_index], L.cache_pages_k, x.bad_page);
+  const int64_t pg = checked_page(page_id(L.page_table_k, (int64_t)x.b * L.page_table_k_stride_b + page_index), L.cache_pages_k, x.bad_page);
   const uint8_t* page = L.key_cache + pg * L.key_cache_stride_page + (int64_t)x.h * k_head_bytes(BOOST ? 32 : 0);
   const uint8_t* meta = (const uint8_t*)L.key_meta + pg * L.key_meta_stride_page + (int64_t)x.h * kD * 4;
   const uint32_t off16 = x.lane * 16, off4 = x.lane * 4, off4dup = (x.lane & 31) * 4;
@@ -571,22 +571,34 @@ __device__ __forceinline__ void combine_quarter(const Ctx& x, const float4v (&C)
     for (int j = 0; j < 4; ++j) own[i][j] = odd ? T[2 + i][j] : T[i][j];
 }
 
-// logits of up to 128 fp16 rows (sink or K Q-buffer): A = the rows themselves, B = q
-__device__ __forceinline__ void qk_fp16(const Ctx& x, const uint8_t* rows, int nrows_alloc, float4v (&C)[8]) {
+// logits of up to 128 fp16 rows (sink or K Q-buffer): A = the rows themselves, B = q.  Here the k-slots
+// are in natural order - slot (kg, 2pi + h) = channel 32kc + 8kg + 2pi + h - so that an operand is one
+// 16-byte load of the row, and q comes from its natural-order copy in LDS (q_nat).  The loads of
+// four tiles (16 per lane) are issued together: the rows come straight from HBM and a wave has
+// nothing else to do while it waits, so the depth of the queue is what the phase costs.
+template <class LDS>
+__device__ __forceinline__ void qk_fp16(const LDS& S, const Ctx& x, const uint8_t* rows, int nrows_alloc, float4v (&C)[8]) {
+  uint4v bq[4];
 #pragma unroll
-  for (int u = 0; u < 8; ++u) {
-    C[u] = float4v{0.f, 0.f, 0.f, 0.f};
-    const int row = min(8 * x.n + u, nrows_alloc - 1);     // A row of this lane; clamped rows are masked later
-    const uint8_t* rp = rows + (int64_t)row * (kD * 2);
+  for (int kc = 0; kc < 4; ++kc) bq[kc] = *(const uint4v*)&S.q_nat[x.g][32 * kc + 8 * x.kg];
 #pragma unroll
-    for (int kc = 0; kc < 4; ++kc) {
-      uint32_t a[4], bq[4];
+  for (int half = 0; half < 2; ++half) {
+    uint4v a[4][4];
 #pragma unroll
-      for (int pi = 0; pi < 4; ++pi) {
-        a[pi] = *(const uint32_t*)(rp + (32 * kc + krow(pi, x.kg)) * 2);   // channels 32kc + krow + {0,1}
-        bq[pi] = x.qpair[kc * 4 + pi];
-      }
-      C[u] = mfma16(a, bq, C[u]);
+    for (int i = 0; i < 4; ++i) {
+      const int row = min(8 * x.n + 4 * half + i, nrows_alloc - 1);   // A row of this lane; clamped rows are masked later
+      const uint8_t* rp = rows + (int64_t)row * (kD * 2) + 16 * x.kg;
+#pragma unroll
+      for (int kc = 0; kc < 4; ++kc) a[i][kc] = *(const uint4v*)(rp + 64 * kc);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      float4v acc = float4v{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int kc = 0; kc < 4; ++kc)
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, a[i][kc]),
+                                                     __builtin_bit_cast(half8, bq[kc]), acc, 0, 0, 0);
+      C[4 * half + i] = acc;
     }
   }
 }
@@ -688,7 +700,7 @@ struct VLds {
 
 __device__ __forceinline__ void v_load_regs(const Ctx& x, int page_index, VRegs& vb) {
   const kitty_kv_layer& L = *x.L;
-  const int64_t pg = checked_page(L.page_table_v[(int64_t)x.b * L.page_table_v_stride_b + page_index], L.cache_pages_v, x.bad_page);
+  const int64_t pg = checked_page(page_id(L.page_table_v, (int64_t)x.b * L.page_table_v_stride_b + page_index), L.cache_pages_v, x.bad_page);
   const uint8_t* page = L.value_cache + pg * L.value_cache_stride_page + (int64_t)x.h * kVBytes;
   const uint8_t* meta = (const uint8_t*)L.value_meta + pg * L.value_meta_stride_page + (int64_t)x.h * kPage * 4;
   const uint32_t v_off = (32 * x.kg + (x.n & 1)) * kRowBytes + (x.n >> 1) * 4;
@@ -700,7 +712,7 @@ __device__ __forceinline__ void v_load_regs(const Ctx& x, int page_index, VRegs&
 // Global -> LDS loads of one V page-head, byte for byte.
 __device__ __forceinline__ void dma_v(const Ctx& x, int page_index, uint32_t lds) {
   const kitty_kv_layer& L = *x.L;
-  const int64_t pg = checked_page(L.page_table_v[(int64_t)x.b * L.page_table_v_stride_b + page_index], L.cache_pages_v, x.bad_page);
+  const int64_t pg = checked_page(page_id(L.page_table_v, (int64_t)x.b * L.page_table_v_stride_b + page_index), L.cache_pages_v, x.bad_page);
   const uint8_t* page = L.value_cache + pg * L.value_cache_stride_page + (int64_t)x.h * kVBytes;
   const uint8_t* meta = (const uint8_t*)L.value_meta + pg * L.value_meta_stride_page + (int64_t)x.h * kPage * 4;
   const uint32_t off16 = x.lane * 16;
@@ -811,9 +823,12 @@ __device__ __forceinline__ void pv_quarter(LDS& S, const Ctx& x, float4v (&out)[
 }
 
 // fp16 V rows (sink, V Q-buffer, local ring), accumulators in true units.  The matrix core wants
-// A[row = channel][k = token], i.e. the rows transposed: 32 tokens at a time (the tokens of one
-// lane group) are copied into LDS as [channel][token] with 16-bit stores, after which the eight
-// k-slots of a lane are one 128-bit read.  The other three lane groups multiply by zero meanwhile.
+// A[row = channel][k = token], i.e. the rows transposed: 32 tokens at a time are copied into LDS as
+// [channel][token] with 16-bit stores, after which the eight k-slots of a lane are one 128-bit read.
+// Which 32 tokens: k-chunk s of every lane group - tokens 32kg + 8s + {0..7}, kg = 0..3, the tokens
+// behind accumulator register s of the logits - so that one staging feeds ONE full-depth matrix
+// instruction per channel tile.  A tile of at most 32 tokens (the sink) has them all in lane group 0:
+// there tokens 0..31 are staged once and multiplied in four steps, the other lane groups feeding zeros.
 constexpr int kVtPitch = 80;                 // bytes per channel row: 32 tokens + padding
 constexpr int kVtBytes = kD * kVtPitch;      // 10240
 static_assert(kVtBytes <= 2 * kKTile && kVtBytes <= 10240, "the staging area reuses the K tile buffers");
@@ -823,10 +838,13 @@ __device__ __forceinline__ void pv_fp16(uint8_t* vt, const Ctx& x, Acc& A, int t
                                         const float4v (&P)[8]) {
   const kitty_kv_layer& L = *x.L;
   const uint32_t one_or_zero = (x.n & 1) ? 0u : 0x3C003C00u;    // even rows sum p, odd rows stay 0
-  const int tt = x.lane >> 1, c0 = (x.lane & 1) * 8;            // staging: token of the quarter, first piece
-  // the rows of quarter qt + 1 are fetched while quarter qt is multiplied
-  auto fetch = [&](int qt, uint4 (&piece)[8]) {
-    const int t = 32 * qt + tt;
+  const int tt = x.lane >> 1, c0 = (x.lane & 1) * 8;            // staging: position among the 32 tokens, first piece
+  const bool by_chunk = ntok > 32;
+  const int t_base = by_chunk ? 32 * (tt >> 3) + (tt & 7) : tt, t_step = by_chunk ? 8 : 32;
+  const bool col_on = !QUARTER || x.pi_own == 0;
+  // the rows of staging s + 1 are fetched while staging s is multiplied
+  auto fetch = [&](int s, uint4 (&piece)[8]) {
+    const int t = t_base + t_step * s;
     const bool ok = t < ntok;   // rows past the tile's end carry p = 0; zeros keep 0 * value at 0
     const __half* row = nullptr;
     if (ok) {
@@ -839,11 +857,7 @@ __device__ __forceinline__ void pv_fp16(uint8_t* vt, const Ctx& x, Acc& A, int t
 #pragma unroll
     for (int k = 0; k < 8; ++k) piece[k] = ok ? ((const uint4*)row)[c0 + k] : uint4{0u, 0u, 0u, 0u};
   };
-  uint4 piece[8];
-  fetch(0, piece);
-#pragma unroll 1
-  for (int qt = 0; qt < 4; ++qt) {
-    if (32 * qt >= ntok) break;
+  auto stage = [&](const uint4 (&piece)[8]) {
     wave_lds_fence();
 #pragma unroll
     for (int k = 0; k < 8; ++k) {
@@ -855,26 +869,39 @@ __device__ __forceinline__ void pv_fp16(uint8_t* vt, const Ctx& x, Acc& A, int t
         *(uint16_t*)(dst + (2 * i + 1) * kVtPitch) = (uint16_t)(w4[i] >> 16);
       }
     }
-    if (32 * (qt + 1) < ntok) fetch(qt + 1, piece);
-    wave_lds_fence();
-    const bool mine = x.kg == qt && (!QUARTER || x.pi_own == 0);
+  };
+  // one matrix instruction per channel tile: k-slots = 8 staged tokens at byte `at` of every channel row
+  auto multiply = [&](int j, int at, bool on) {
+    uint32_t bp[4], alz[4];
+#pragma unroll
+    for (int pi = 0; pi < 4; ++pi) {
+      const half2v p2 = {(_Float16)P[2 * pi][j], (_Float16)P[2 * pi + 1][j]};   // tokens 32kg + 8j + 2pi + {0,1}
+      bp[pi] = on ? as_u32(p2) : 0u;
+      alz[pi] = one_or_zero;
+    }
+    A.lz = mfma16(alz, bp, A.lz);
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const uint4v a4 = *(const uint4v*)(vt + (8 * x.n + u) * kVtPitch + at);
+      const uint32_t a[4] = {a4[0], a4[1], a4[2], a4[3]};
+      A.out[u] = mfma16(a, bp, A.out[u]);
+    }
+  };
+  uint4 piece[8];
+  fetch(0, piece);
+  if (by_chunk) {
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      uint32_t bp[4], alz[4];
-#pragma unroll
-      for (int pi = 0; pi < 4; ++pi) {
-        const half2v p2 = {(_Float16)P[2 * pi][j], (_Float16)P[2 * pi + 1][j]};   // tokens 32kg + 8j + 2pi + {0,1}
-        bp[pi] = mine ? as_u32(p2) : 0u;
-        alz[pi] = one_or_zero;
-      }
-      A.lz = mfma16(alz, bp, A.lz);
-#pragma unroll
-      for (int u = 0; u < 8; ++u) {
-        const uint4v a4 = *(const uint4v*)(vt + (8 * x.n + u) * kVtPitch + 16 * j);   // tokens 8j .. 8j+7 of the quarter
-        const uint32_t a[4] = {a4[0], a4[1], a4[2], a4[3]};
-        A.out[u] = mfma16(a, bp, A.out[u]);
-      }
+      stage(piece);
+      if (j < 3) fetch(j + 1, piece);
+      wave_lds_fence();
+      multiply(j, 16 * x.kg, col_on);
     }
+  } else {
+    stage(piece);
+    wave_lds_fence();
+#pragma unroll
+    for (int j = 0; j < 4; ++j) multiply(j, 16 * j, col_on && x.kg == 0);
   }
   wave_lds_fence();
 }
@@ -890,6 +917,15 @@ __device__ __forceinline__ void to_true_units(Acc& A) {
 template <int N>
 __device__ __forceinline__ void wait_vmcnt() {
   asm volatile("s_waitcnt vmcnt(%0)" :: "n"(N) : "memory");
+}
+
+// Every vector load of the kernel's prologue (q, counters) has landed.  The compiler does not see the
+// tile loads of the streaming loops (inline assembly); what it does see is its own prologue loads,
+// and it would wait for the registers they fill where they are first used - inside the loop, with
+// s_waitcnt vmcnt(0), which there also waits for every tile load in flight, in every iteration.
+// An explicit wait before the loop, one that the compiler's bookkeeping understands, settles them.
+__device__ __forceinline__ void settle_prologue_loads() {
+  __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0); expcnt, lgkmcnt: no wait
 }
 
 // DMA: packed tiles are streamed global -> LDS (G <= 8); otherwise they are loaded into registers.
@@ -986,6 +1022,10 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(kitty_kv_layer L, co
   // split when a body split is long enough to hide it (12 tiles or more), else three (sink / first
   // tail tile / the others).  The remaining splits share the body evenly (tile counts differ by at
   // most one).  1 split: everything.
+  // (Measured and dropped: no wave of its own for the tail but three splits that take one tail unit
+  // each after a body share shortened by the unit's cost.  With all 16 splits of a 32k context
+  // streaming, the body alone takes 4 us longer than with 15 streaming and one idle, and the gain
+  // from hiding the tail is spent.)
   const int nbt = c_div_up(x.c.nbody, kPage);
   const int npp = min(min(x.c.pv, x.c.pk), nbt);
   const int n_tail = num_splits >= 4 && npp < 12 * (num_splits - 3) ? 3 : (num_splits >= 2 ? 1 : 0);
@@ -1017,6 +1057,7 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(kitty_kv_layer L, co
     // count the instructions issued AFTER the tile that is needed; nothing is loaded past the end
     // of the range (the last two iterations wait on shorter queues).
     if (t0 < t1) {
+      settle_prologue_loads();
       constexpr int nK = kDmaK<BOOST>;
       const uint32_t lk0 = (uint32_t)(uintptr_t)&S.kbuf[0][0], lk1 = (uint32_t)(uintptr_t)&S.kbuf[1][0];
       const uint32_t lv = (uint32_t)(uintptr_t)&S.vbuf[0];
@@ -1104,7 +1145,7 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(kitty_kv_layer L, co
         qk_packed<BOOST, SPLIT_COLS>(S, x, kb, C, cz);
         softmax_tile<true>(x, A, C, cz, ntok);
       } else {
-        qk_fp16(x, qbuf_k, kPage, C);
+        qk_fp16(S, x, qbuf_k, kPage, C);
         softmax_tile<false>(x, A, C, 0.f, ntok);
       }
       if (i < x.c.pv) {
@@ -1127,7 +1168,7 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(kitty_kv_layer L, co
     }
     if (do_sink && x.c.sink > 0) {
       const uint8_t* sink_k = (const uint8_t*)L.sink_k + (int64_t)x.b * L.sink_stride_b + (int64_t)x.h * L.sink_stride_h;
-      qk_fp16(x, sink_k, L.S, C);
+      qk_fp16(S, x, sink_k, L.S, C);
       softmax_tile<false>(x, A, C, 0.f, x.c.sink);
       pv_fp16<true, QUARTER>(&S.kbuf[0][0], x, A, 0, x.c.sink, C);
     }

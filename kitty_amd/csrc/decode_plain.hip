@@ -68,7 +68,7 @@ __global__ __launch_bounds__(256) void decode_plain_kernel(kitty_kv_layer L, con
 #pragma unroll
     for (int g = 0; g < kMaxGroup; ++g) acc[g] = 0.f;
     if (k_packed) {
-      const int64_t pg = checked_page(L.page_table_k[(int64_t)b * L.page_table_k_stride_b + body], L.cache_pages_k, bad_page);
+      const int64_t pg = checked_page(page_id(L.page_table_k, (int64_t)b * L.page_table_k_stride_b + body), L.cache_pages_k, bad_page);
       const uint8_t* src = L.key_cache + pg * L.key_cache_stride_page + (int64_t)h * k_head_bytes(DB);
       for (int i = tid; i < k_head_bytes(DB) / 16; i += 256) ((uint4*)s_codes)[i] = ((const uint4*)src)[i];
       if (tid < kD)
@@ -124,7 +124,7 @@ __global__ __launch_bounds__(256) void decode_plain_kernel(kitty_kv_layer L, con
     }
     // ---- stage V ---------------------------------------------------------------------------
     if (v_packed) {
-      const int64_t pg = checked_page(L.page_table_v[(int64_t)b * L.page_table_v_stride_b + body], L.cache_pages_v, bad_page);
+      const int64_t pg = checked_page(page_id(L.page_table_v, (int64_t)b * L.page_table_v_stride_b + body), L.cache_pages_v, bad_page);
       const uint8_t* src = L.value_cache + pg * L.value_cache_stride_page + (int64_t)h * kVBytes;
       ((uint4*)s_codes)[tid] = ((const uint4*)src)[tid];
       if (tid < kPage)

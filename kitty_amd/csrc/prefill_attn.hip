@@ -151,7 +151,7 @@ struct Prefill {
       const int i = t - first_body;
       s.ntok = min(kPage, c.nbody - i * kPage);
       if (i < c.pk) {
-        const int64_t pg = checked_page(L.page_table_k[(int64_t)b * L.page_table_k_stride_b + i], L.cache_pages_k, bad_page);
+        const int64_t pg = checked_page(page_id(L.page_table_k, (int64_t)b * L.page_table_k_stride_b + i), L.cache_pages_k, bad_page);
         s.k_kind = SRC_PACKED;
         s.k_ptr = L.key_cache + pg * L.key_cache_stride_page + (int64_t)h * k_head_bytes(L.D_BOOSTED);
         s.k_meta = (const uint8_t*)L.key_meta + pg * L.key_meta_stride_page + (int64_t)h * kD * 4;
@@ -161,7 +161,7 @@ struct Prefill {
         s.k_stride = kD * 2;
       }
       if (i < c.pv) {
-        const int64_t pg = checked_page(L.page_table_v[(int64_t)b * L.page_table_v_stride_b + i], L.cache_pages_v, bad_page);
+        const int64_t pg = checked_page(page_id(L.page_table_v, (int64_t)b * L.page_table_v_stride_b + i), L.cache_pages_v, bad_page);
         s.v_kind = SRC_PACKED;
         s.v_ptr = L.value_cache + pg * L.value_cache_stride_page + (int64_t)h * kVBytes;
         s.v_meta = (const uint8_t*)L.value_meta + pg * L.value_meta_stride_page + (int64_t)h * kPage * 4;
