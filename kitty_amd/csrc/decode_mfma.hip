@@ -928,16 +928,30 @@ __device__ __forceinline__ void settle_prologue_loads() {
   __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0); expcnt, lgkmcnt: no wait
 }
 
-// DMA: packed tiles are streamed global -> LDS (G <= 8); otherwise they are loaded into registers.
-// QUARTER (needs DMA; at most 4 query heads per kv head): body pages go through combine_quarter /
-// softmax_quarter / pv_quarter.
-template <bool BOOST, bool DMA, bool QUARTER>
-__global__ __launch_bounds__(64, 2) void decode_mfma_kernel(kitty_kv_layer L, const __half* __restrict__ q, int H_Q,
-                                                            float scaling, float* __restrict__ ws_ml,
-                                                            float* __restrict__ ws_acc, int num_splits,
-                                                            int n_simds) {
+// How many of the first splits of a (batch row, kv head) take its tail (see wave_work).
+__device__ __forceinline__ int tail_splits(const SeqCounts& c, int num_splits) {
+  const int nbt = c_div_up(c.nbody, kPage);
+  const int npp = min(min(c.pv, c.pk), nbt);
+  return num_splits >= 4 && npp < 12 * (num_splits - 3) ? 3 : (num_splits >= 2 ? 1 : 0);
+}
+
+// What one wave does.  DMA: packed tiles are streamed global -> LDS (G <= 8); otherwise they are
+// loaded into registers.  QUARTER (needs DMA; at most 4 query heads per kv head): body pages go
+// through combine_quarter / softmax_quarter / pv_quarter.
+// MODE: kWaveSolo - the launch has one split, whose wave does everything; kWaveBody - a split with
+// body tiles only; kWaveTail - a split with the sink and / or tiles with fp16 rows only.  The last
+// two are different FUNCTIONS (the kernel calls the tail's one without inlining it), not branches of
+// one: the tail's code needs every register there is and spills, and as a branch of the function
+// that holds the streaming loop it costs the loop, which it never runs beside, several percent - the
+// loop's code comes out with half again as many wait states and 256 registers instead of 162, and
+// when the pressure is on the wrong side of the edge, with spills of its own (a reload inside the
+// loop is a vector load that the hand-counted waits do not know of).
+enum WaveMode { kWaveSolo, kWaveBody, kWaveTail };
+template <bool BOOST, bool DMA, bool QUARTER, WaveMode MODE, class LDS>
+__device__ __forceinline__ void wave_work(const kitty_kv_layer& L, const __half* __restrict__ q, int H_Q, float scaling,
+                                          float* __restrict__ ws_ml, float* __restrict__ ws_acc, int num_splits,
+                                          int n_simds, LDS& S) {
   static_assert(DMA || !QUARTER, "quarter columns are a variant of the LDS-streamed kernel");
-  __shared__ WaveLds<DMA, QUARTER> S;
   Ctx x;
   x.L = &L;
   x.bad_page = 0;
@@ -1028,7 +1042,7 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(kitty_kv_layer L, co
   // from hiding the tail is spent.)
   const int nbt = c_div_up(x.c.nbody, kPage);
   const int npp = min(min(x.c.pv, x.c.pk), nbt);
-  const int n_tail = num_splits >= 4 && npp < 12 * (num_splits - 3) ? 3 : (num_splits >= 2 ? 1 : 0);
+  const int n_tail = tail_splits(x.c, num_splits);
   int t0 = 0, t1 = 0;          // body tiles of this split
   int u0 = nbt, u1 = nbt;      // tail tiles of this split
   bool do_sink = false;
@@ -1046,11 +1060,14 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(kitty_kv_layer L, co
     t0 = i_body * base + min(i_body, rem);
     t1 = t0 + base + (i_body < rem ? 1 : 0);
   }
-  const bool tail = do_sink || u0 < u1;
+  const bool tail = MODE != kWaveBody && (do_sink || u0 < u1);
   const uint8_t* qbuf_k = (const uint8_t*)L.qbuf_k + (int64_t)x.b * L.win_stride_b + (int64_t)x.h * L.win_stride_h;
 
   float4v C[8];
-  if constexpr (DMA) {
+  if constexpr (MODE == kWaveTail) {
+    t1 = t0;   // (a split with tail work has no body tiles; this tells the compiler)
+  }
+  if constexpr (MODE != kWaveTail && DMA) {
     // Tiles stream through LDS: two K buffers, one V buffer.  Issue order
     //   K(t0) K(t0+1) V(t0) | QK(i) -> K(i+2) -> softmax -> PV(i) -> V(i+1) | ...
     // so K(i) has a lead of one and a half iterations and V(i) of half an iteration.  The waits
@@ -1113,7 +1130,7 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(kitty_kv_layer L, co
       if (young) loop(std::true_type{}); else loop(std::false_type{});
       wait_vmcnt<0>();
     }
-  } else {
+  } else if constexpr (MODE != kWaveTail) {
     // Register-fed software pipeline: the V words of tile i are in flight during its QK phase,
     // the K words of tile i+1 during its softmax and PV phase.
     KRegs kb;
@@ -1131,7 +1148,7 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(kitty_kv_layer L, co
       pv_packed(S, x, A.out, A.lz, vb, C);
     }
   }
-  if (tail) {
+  if (MODE != kWaveBody && tail) {
     if constexpr (QUARTER) stage_generic_tables();   // the V tile is idle from here on
     to_true_units(A);
     KRegs kb;
@@ -1212,6 +1229,52 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(kitty_kv_layer L, co
   }
 }
 
+// The kernel's arguments, as one struct: the tail's function reads them where they lie.
+struct KernArgs {
+  kitty_kv_layer L;
+  const __half* q;
+  int H_Q;
+  float scaling;
+  float* ws_ml;
+  float* ws_acc;
+  int num_splits, n_simds;
+};
+
+// The tail's function: a call, not a branch (see wave_work).  Arguments of a function arrive in
+// vector registers, which the compiler takes for different from lane to lane - every branch on them
+// a divergent one, every load through them a vector load.  So the function gets two addresses, made
+// scalars again on arrival: of the kernel's argument block (the intrinsic that names it is only
+// valid in the kernel itself) and of the wave's LDS.  It ends the wave: nothing of the caller's needs
+// saving.
+template <bool BOOST, bool DMA, bool QUARTER>
+__device__ __attribute__((noinline, noreturn)) void tail_wave(const KernArgs* kernel_args,
+                                                               __attribute__((address_space(3))) WaveLds<DMA, QUARTER>* lds) {
+  const uint64_t v = (uint64_t)(uintptr_t)kernel_args;
+  const uint64_t u = ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(v >> 32)) << 32) |
+                     (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)v);
+  const KernArgs& a = *(const KernArgs*)(const __attribute__((address_space(4))) KernArgs*)(uintptr_t)u;
+  wave_work<BOOST, DMA, QUARTER, kWaveTail>(a.L, a.q, a.H_Q, a.scaling, a.ws_ml, a.ws_acc, a.num_splits, 0,
+                                             *(WaveLds<DMA, QUARTER>*)lds);
+  __builtin_amdgcn_endpgm();
+}
+
+// SOLO: the launch has one split.  Otherwise the first tail_splits() splits of a (batch row, kv head)
+// go through tail_wave and the others stream the body.
+template <bool BOOST, bool DMA, bool QUARTER, bool SOLO>
+__global__ __launch_bounds__(64, 2) void decode_mfma_kernel(KernArgs a) {
+  __shared__ WaveLds<DMA, QUARTER> S;
+  if constexpr (SOLO) {
+    wave_work<BOOST, DMA, QUARTER, kWaveSolo>(a.L, a.q, a.H_Q, a.scaling, a.ws_ml, a.ws_acc, a.num_splits, a.n_simds, S);
+  } else {
+    if ((int)blockIdx.x < tail_splits(load_counts(a.L, blockIdx.z), a.num_splits)) {
+      tail_wave<BOOST, DMA, QUARTER>(
+          (const KernArgs*)(const __attribute__((address_space(4))) KernArgs*)__builtin_amdgcn_kernarg_segment_ptr(),
+          (__attribute__((address_space(3))) WaveLds<DMA, QUARTER>*)&S);
+    }
+    wave_work<BOOST, DMA, QUARTER, kWaveBody>(a.L, a.q, a.H_Q, a.scaling, a.ws_ml, a.ws_acc, a.num_splits, a.n_simds, S);
+  }
+}
+
 }  // namespace
 
 bool decode_mfma_supported(const kitty_kv_layer& L, int H_Q) {
@@ -1221,28 +1284,41 @@ bool decode_mfma_supported(const kitty_kv_layer& L, int H_Q) {
 // ev_start / ev_stop (both or neither): events attached to the kernel's own dispatch, which then hold
 // the moments the kernel began and ended on the device (what a kernel trace reports) rather than the
 // moments the host enqueued around it.
+namespace {
+struct LaunchArgs {
+  KernArgs k;
+  int B;
+  hipStream_t stream;
+  hipEvent_t ev_start, ev_stop;
+};
+template <bool BOOST, bool DMA, bool QUARTER, bool SOLO>
+void launch_one(const LaunchArgs& a) {
+  const dim3 grid(a.k.num_splits, a.k.L.H_KV, a.B), block(64);
+  if (a.ev_start)
+    hipExtLaunchKernelGGL((decode_mfma_kernel<BOOST, DMA, QUARTER, SOLO>), grid, block, 0, a.stream, a.ev_start,
+                          a.ev_stop, 0, a.k);
+  else
+    hipLaunchKernelGGL((decode_mfma_kernel<BOOST, DMA, QUARTER, SOLO>), grid, block, 0, a.stream, a.k);
+}
+template <bool BOOST, bool DMA, bool QUARTER>
+void launch_variant(const LaunchArgs& a) {
+  if (a.k.num_splits == 1) launch_one<BOOST, DMA, QUARTER, true>(a);
+  else launch_one<BOOST, DMA, QUARTER, false>(a);
+}
+}  // namespace
+
 void launch_decode_mfma(const kitty_kv_layer& L, const void* q, int B, int H_Q, float scaling, float* ws_ml,
                         float* ws_acc, int num_splits, int n_simds, hipStream_t stream, hipEvent_t ev_start,
                         hipEvent_t ev_stop) {
-  const dim3 grid(num_splits, L.H_KV, B), block(64);
+  const LaunchArgs a{KernArgs{L, (const __half*)q, H_Q, scaling, ws_ml, ws_acc, num_splits, n_simds}, B, stream, ev_start, ev_stop};
   const int G = H_Q / L.H_KV;
   const bool boost = L.D_BOOSTED == 32, dma = G <= 8, quarter = G <= 4;
-#define KITTY_LAUNCH(BOOST, DMA, QUARTER)                                                                        \
-  do {                                                                                                           \
-    if (ev_start)                                                                                                \
-      hipExtLaunchKernelGGL((decode_mfma_kernel<BOOST, DMA, QUARTER>), grid, block, 0, stream, ev_start, ev_stop, 0, \
-                            L, (const __half*)q, H_Q, scaling, ws_ml, ws_acc, num_splits, n_simds);              \
-    else                                                                                                         \
-      hipLaunchKernelGGL((decode_mfma_kernel<BOOST, DMA, QUARTER>), grid, block, 0, stream, L, (const __half*)q,  \
-                         H_Q, scaling, ws_ml, ws_acc, num_splits, n_simds);                                      \
-  } while (0)
-  if (boost && quarter) KITTY_LAUNCH(true, true, true);
-  else if (boost && dma) KITTY_LAUNCH(true, true, false);
-  else if (boost) KITTY_LAUNCH(true, false, false);
-  else if (quarter) KITTY_LAUNCH(false, true, true);
-  else if (dma) KITTY_LAUNCH(false, true, false);
-  else KITTY_LAUNCH(false, false, false);
-#undef KITTY_LAUNCH
+  if (boost && quarter) launch_variant<true, true, true>(a);
+  else if (boost && dma) launch_variant<true, true, false>(a);
+  else if (boost) launch_variant<true, false, false>(a);
+  else if (quarter) launch_variant<false, true, true>(a);
+  else if (dma) launch_variant<false, true, false>(a);
+  else launch_variant<false, false, false>(a);
 }
 
 }  // namespace kitty
