@@ -928,10 +928,32 @@ __device__ __forceinline__ void settle_prologue_loads() {
   __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0); expcnt, lgkmcnt: no wait
 }
 
+// One split of one (batch row, kv head).  crowded: the launch has more workgroups than the device
+// holds at once (two per SIMD) and runs in rounds; a workgroup's fixed cost - dispatch, prologue,
+// filling and draining the tile pipeline, about two tiles' worth - then comes out of the throughput,
+// so the splits are cut for few, long shares (a short sequence leaves its last splits without work),
+// and the ORDER of the workgroups matters: the dispatcher hands them out by linear id as slots free
+// up.  With the split index fastest (the one-round layout) the splits without work come in bursts
+// between the busy ones and the slots they free are refilled late (ragged batch of 64: 1,500 of
+// 2,048 resident on average), and the launch ends with whatever sequence came last.  A crowded grid
+// is (units, splits) with the unit fastest and the split index reversed: first the high splits,
+// which only long sequences use, last the tail splits and the first body shares of every sequence,
+// so the final round is the fullest.
+struct WorkItem {
+  int b, h, split;
+  bool crowded;
+};
+__device__ __forceinline__ WorkItem work_item_of_block(int h_kv, int num_splits, bool crowded) {
+  if (!crowded) return WorkItem{(int)blockIdx.z, (int)blockIdx.y, (int)blockIdx.x, false};
+  return WorkItem{(int)blockIdx.x / h_kv, (int)blockIdx.x % h_kv, num_splits - 1 - (int)blockIdx.y, true};
+}
+constexpr int kCrowdedMinTiles = 8;    // body tiles per split a crowded launch aims for
+
 // How many of the first splits of a (batch row, kv head) take its tail (see wave_work).
-__device__ __forceinline__ int tail_splits(const SeqCounts& c, int num_splits) {
+__device__ __forceinline__ int tail_splits(const SeqCounts& c, int num_splits, bool crowded) {
   const int nbt = c_div_up(c.nbody, kPage);
   const int npp = min(min(c.pv, c.pk), nbt);
+  if (crowded) return num_splits >= 2 ? 1 : 0;   // one after the other costs least when nothing runs beside it for free
   return num_splits >= 4 && npp < 12 * (num_splits - 3) ? 3 : (num_splits >= 2 ? 1 : 0);
 }
 
@@ -950,14 +972,14 @@ enum WaveMode { kWaveSolo, kWaveBody, kWaveTail };
 template <bool BOOST, bool DMA, bool QUARTER, WaveMode MODE, class LDS>
 __device__ __forceinline__ void wave_work(const kitty_kv_layer& L, const __half* __restrict__ q, int H_Q, float scaling,
                                           float* __restrict__ ws_ml, float* __restrict__ ws_acc, int num_splits,
-                                          int n_simds, LDS& S) {
+                                          int n_simds, const WorkItem& w, LDS& S) {
   static_assert(DMA || !QUARTER, "quarter columns are a variant of the LDS-streamed kernel");
   Ctx x;
   x.L = &L;
   x.bad_page = 0;
-  x.b = blockIdx.z;
-  x.h = blockIdx.y;
-  const int split = blockIdx.x;
+  x.b = w.b;
+  x.h = w.h;
+  const int split = w.split;
   x.lane = threadIdx.x;
   x.kg = x.lane >> 4;
   x.n = x.lane & 15;
@@ -1042,7 +1064,7 @@ __device__ __forceinline__ void wave_work(const kitty_kv_layer& L, const __half*
   // from hiding the tail is spent.)
   const int nbt = c_div_up(x.c.nbody, kPage);
   const int npp = min(min(x.c.pv, x.c.pk), nbt);
-  const int n_tail = tail_splits(x.c, num_splits);
+  const int n_tail = tail_splits(x.c, num_splits, w.crowded);
   int t0 = 0, t1 = 0;          // body tiles of this split
   int u0 = nbt, u1 = nbt;      // tail tiles of this split
   bool do_sink = false;
@@ -1054,11 +1076,16 @@ __device__ __forceinline__ void wave_work(const kitty_kv_layer& L, const __half*
     else if (split == 1) { u0 = npp; u1 = min(nbt, npp + 1); }
     else u0 = min(nbt, npp + 1);
   } else {
-    // even shares: the first npp % n_body splits take one tile more
-    const int n_body = num_splits - n_tail, i_body = split - n_tail;
-    const int base = npp / n_body, rem = npp - base * n_body;
-    t0 = i_body * base + min(i_body, rem);
-    t1 = t0 + base + (i_body < rem ? 1 : 0);
+    // even shares: the first npp % n_body splits take one tile more.  A crowded launch gives a short
+    // sequence fewer, longer shares; the splits past them have nothing to do.
+    const int i_body = split - n_tail;
+    int n_body = num_splits - n_tail;
+    if (w.crowded) n_body = min(n_body, max(1, c_div_up(npp, kCrowdedMinTiles)));
+    if (i_body < n_body) {
+      const int base = npp / n_body, rem = npp - base * n_body;
+      t0 = i_body * base + min(i_body, rem);
+      t1 = t0 + base + (i_body < rem ? 1 : 0);
+    }
   }
   const bool tail = MODE != kWaveBody && (do_sink || u0 < u1);
   const uint8_t* qbuf_k = (const uint8_t*)L.qbuf_k + (int64_t)x.b * L.win_stride_b + (int64_t)x.h * L.win_stride_h;
@@ -1089,7 +1116,7 @@ __device__ __forceinline__ void wave_work(const kitty_kv_layer& L, const __half*
       const uint32_t kSimds = (uint32_t)n_simds;
       const uint32_t n_wg = gridDim.x * gridDim.y * gridDim.z;
       const uint32_t lin_id = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
-      const bool young = n_wg <= 2 * kSimds && lin_id >= kSimds;
+      const bool young = !w.crowded && n_wg <= 2 * kSimds && lin_id >= kSimds;
       auto loop = [&](auto switch_priority) {
       constexpr bool SWITCH = decltype(switch_priority)::value;
 #pragma unroll 1
@@ -1238,40 +1265,46 @@ struct KernArgs {
   float* ws_ml;
   float* ws_acc;
   int num_splits, n_simds;
+  int crowded;   // the grid is (units, reversed splits), see WorkItem
 };
+
+__device__ __forceinline__ const KernArgs& kernel_args_of(const KernArgs* p) {   // the address as a scalar again
+  const uint64_t v = (uint64_t)(uintptr_t)p;
+  const uint64_t u = ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(v >> 32)) << 32) |
+                     (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)v);
+  return *(const KernArgs*)(const __attribute__((address_space(4))) KernArgs*)(uintptr_t)u;
+}
 
 // The tail's function: a call, not a branch (see wave_work).  Arguments of a function arrive in
 // vector registers, which the compiler takes for different from lane to lane - every branch on them
-// a divergent one, every load through them a vector load.  So the function gets two addresses, made
+// a divergent one, every load through them a vector load.  So the function gets addresses, made
 // scalars again on arrival: of the kernel's argument block (the intrinsic that names it is only
-// valid in the kernel itself) and of the wave's LDS.  It ends the wave: nothing of the caller's needs
-// saving.
+// valid in the kernel itself) and of the wave's LDS.  This one ends the wave: nothing of the
+// caller's needs saving.
 template <bool BOOST, bool DMA, bool QUARTER>
 __device__ __attribute__((noinline, noreturn)) void tail_wave(const KernArgs* kernel_args,
                                                                __attribute__((address_space(3))) WaveLds<DMA, QUARTER>* lds) {
-  const uint64_t v = (uint64_t)(uintptr_t)kernel_args;
-  const uint64_t u = ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(v >> 32)) << 32) |
-                     (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)v);
-  const KernArgs& a = *(const KernArgs*)(const __attribute__((address_space(4))) KernArgs*)(uintptr_t)u;
-  wave_work<BOOST, DMA, QUARTER, kWaveTail>(a.L, a.q, a.H_Q, a.scaling, a.ws_ml, a.ws_acc, a.num_splits, 0,
+  const KernArgs& a = kernel_args_of(kernel_args);
+  const WorkItem w = work_item_of_block(a.L.H_KV, a.num_splits, a.crowded != 0);
+  wave_work<BOOST, DMA, QUARTER, kWaveTail>(a.L, a.q, a.H_Q, a.scaling, a.ws_ml, a.ws_acc, a.num_splits, 0, w,
                                              *(WaveLds<DMA, QUARTER>*)lds);
   __builtin_amdgcn_endpgm();
 }
-
 // SOLO: the launch has one split.  Otherwise the first tail_splits() splits of a (batch row, kv head)
 // go through tail_wave and the others stream the body.
 template <bool BOOST, bool DMA, bool QUARTER, bool SOLO>
 __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(KernArgs a) {
   __shared__ WaveLds<DMA, QUARTER> S;
+  const WorkItem w = work_item_of_block(a.L.H_KV, a.num_splits, a.crowded != 0);
   if constexpr (SOLO) {
-    wave_work<BOOST, DMA, QUARTER, kWaveSolo>(a.L, a.q, a.H_Q, a.scaling, a.ws_ml, a.ws_acc, a.num_splits, a.n_simds, S);
+    wave_work<BOOST, DMA, QUARTER, kWaveSolo>(a.L, a.q, a.H_Q, a.scaling, a.ws_ml, a.ws_acc, a.num_splits, a.n_simds, w, S);
   } else {
-    if ((int)blockIdx.x < tail_splits(load_counts(a.L, blockIdx.z), a.num_splits)) {
+    if (w.split < tail_splits(load_counts(a.L, w.b), a.num_splits, w.crowded)) {
       tail_wave<BOOST, DMA, QUARTER>(
           (const KernArgs*)(const __attribute__((address_space(4))) KernArgs*)__builtin_amdgcn_kernarg_segment_ptr(),
           (__attribute__((address_space(3))) WaveLds<DMA, QUARTER>*)&S);
     }
-    wave_work<BOOST, DMA, QUARTER, kWaveBody>(a.L, a.q, a.H_Q, a.scaling, a.ws_ml, a.ws_acc, a.num_splits, a.n_simds, S);
+    wave_work<BOOST, DMA, QUARTER, kWaveBody>(a.L, a.q, a.H_Q, a.scaling, a.ws_ml, a.ws_acc, a.num_splits, a.n_simds, w, S);
   }
 }
 
@@ -1293,7 +1326,8 @@ struct LaunchArgs {
 };
 template <bool BOOST, bool DMA, bool QUARTER, bool SOLO>
 void launch_one(const LaunchArgs& a) {
-  const dim3 grid(a.k.num_splits, a.k.L.H_KV, a.B), block(64);
+  const dim3 grid = a.k.crowded ? dim3(a.B * a.k.L.H_KV, a.k.num_splits, 1) : dim3(a.k.num_splits, a.k.L.H_KV, a.B);
+  const dim3 block(64);
   if (a.ev_start)
     hipExtLaunchKernelGGL((decode_mfma_kernel<BOOST, DMA, QUARTER, SOLO>), grid, block, 0, a.stream, a.ev_start,
                           a.ev_stop, 0, a.k);
@@ -1310,7 +1344,9 @@ void launch_variant(const LaunchArgs& a) {
 void launch_decode_mfma(const kitty_kv_layer& L, const void* q, int B, int H_Q, float scaling, float* ws_ml,
                         float* ws_acc, int num_splits, int n_simds, hipStream_t stream, hipEvent_t ev_start,
                         hipEvent_t ev_stop) {
-  const LaunchArgs a{KernArgs{L, (const __half*)q, H_Q, scaling, ws_ml, ws_acc, num_splits, n_simds}, B, stream, ev_start, ev_stop};
+  const int64_t n_wg = (int64_t)B * L.H_KV * num_splits;
+  const int crowded = num_splits > 1 && num_splits <= 65535 && n_wg > 2 * (int64_t)n_simds ? 1 : 0;
+  const LaunchArgs a{KernArgs{L, (const __half*)q, H_Q, scaling, ws_ml, ws_acc, num_splits, n_simds, crowded}, B, stream, ev_start, ev_stop};
   const int G = H_Q / L.H_KV;
   const bool boost = L.D_BOOSTED == 32, dma = G <= 8, quarter = G <= 4;
   if (boost && quarter) launch_variant<true, true, true>(a);
