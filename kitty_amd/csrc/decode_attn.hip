@@ -9,8 +9,8 @@ void launch_decode_merge(const float* ws_ml, const float* ws_acc, void* out, int
                          hipStream_t stream);
 bool decode_mfma_supported(const kitty_kv_layer& L, int H_Q);
 void launch_decode_mfma(const kitty_kv_layer& L, const void* q, int B, int H_Q, float scaling, float* ws_ml,
-                        float* ws_acc, int num_splits, int n_simds, hipStream_t stream, hipEvent_t ev_start,
-                        hipEvent_t ev_stop);
+                        float* ws_acc, uint32_t* ws_plan, int num_splits, int n_simds, hipStream_t stream,
+                        hipEvent_t ev_start, hipEvent_t ev_stop);
 void launch_prefill_attn(const kitty_kv_layer& L, const void* q, int64_t q_stride_b, int64_t q_stride_h,
                          int64_t q_stride_t, const void* k_new, const void* v_new, int64_t new_stride_b,
                          int64_t new_stride_h, int64_t new_stride_t, int B, int H_Q, int Tq, float scaling,
@@ -144,7 +144,9 @@ extern "C" int kitty_decode_attn_split(const kitty_kv_layer* layer, const void* 
   const hipEvent_t ev0 = g_ev_start, ev1 = g_ev_stop;
   g_ev_start = g_ev_stop = nullptr;
   if (variant == 0 && decode_mfma_supported(L, H_Q)) {
-    launch_decode_mfma(L, q, B, H_Q, scaling, ws_ml, ws_acc, num_splits, device_simds(), (hipStream_t)stream, ev0, ev1);
+    uint32_t* ws_plan = (uint32_t*)((uint8_t*)ws_acc + ws_acc_bytes(B, H_Q, num_splits));
+    launch_decode_mfma(L, q, B, H_Q, scaling, ws_ml, ws_acc, ws_plan, num_splits, device_simds(), (hipStream_t)stream,
+                       ev0, ev1);
   } else {
     if (ev0) (void)hipEventRecord(ev0, (hipStream_t)stream);
     launch_decode_plain(L, q, B, H_Q, scaling, ws_ml, ws_acc, num_splits, (hipStream_t)stream);

@@ -83,8 +83,19 @@ __host__ __device__ inline size_t ws_ml_bytes(int B, int H_Q, int splits) {
   size_t n = (size_t)B * H_Q * splits * 2 * sizeof(float);
   return (n + 255) & ~(size_t)255;
 }
+__host__ __device__ inline size_t ws_acc_bytes(int B, int H_Q, int splits) {
+  return (size_t)B * H_Q * splits * kD * sizeof(float);   // a multiple of 512
+}
+// After the partials: the work list of a launch that runs in several rounds (decode_plan_kernel) -
+// kPlanHeader words, of which the first is the number of items, then one word per item
+// (batch row << 16 | split), at most B * splits of them.
+constexpr int kPlanHeader = 4;
+__host__ __device__ inline size_t ws_plan_bytes(int B, int splits) {
+  size_t n = ((size_t)B * splits + kPlanHeader) * sizeof(uint32_t);
+  return (n + 255) & ~(size_t)255;
+}
 __host__ __device__ inline size_t ws_total_bytes(int B, int H_Q, int splits) {
-  return ws_ml_bytes(B, H_Q, splits) + (size_t)B * H_Q * splits * kD * sizeof(float);
+  return ws_ml_bytes(B, H_Q, splits) + ws_acc_bytes(B, H_Q, splits) + ws_plan_bytes(B, splits);
 }
 
 }  // namespace kitty

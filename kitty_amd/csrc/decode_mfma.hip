@@ -929,31 +929,89 @@ __device__ __forceinline__ void settle_prologue_loads() {
 }
 
 // One split of one (batch row, kv head).  crowded: the launch has more workgroups than the device
-// holds at once (two per SIMD) and runs in rounds; a workgroup's fixed cost - dispatch, prologue,
+// holds at once (two per SIMD) and runs in rounds.  A workgroup's fixed cost - dispatch, prologue,
 // filling and draining the tile pipeline, about two tiles' worth - then comes out of the throughput,
-// so the splits are cut for few, long shares (a short sequence leaves its last splits without work),
-// and the ORDER of the workgroups matters: the dispatcher hands them out by linear id as slots free
-// up.  With the split index fastest (the one-round layout) the splits without work come in bursts
-// between the busy ones and the slots they free are refilled late (ragged batch of 64: 1,500 of
-// 2,048 resident on average), and the launch ends with whatever sequence came last.  A crowded grid
-// is (units, splits) with the unit fastest and the split index reversed: first the high splits,
-// which only long sequences use, last the tail splits and the first body shares of every sequence,
-// so the final round is the fullest.
+// so the splits are cut for few, long shares (one split for the tail, body shares of at least
+// kCrowdedMinTiles tiles; a short sequence leaves its last splits without work), and the ORDER of
+// the workgroups matters: the dispatcher hands them out by linear id as slots free up.  With the
+// grid laid out (splits, heads, rows) the splits without work come in bursts between the busy ones,
+// the slots they free are refilled late (ragged batch of 64: 1,500 of 2,048 resident on average)
+// and the launch ends with whatever sequence came last.  So a crowded launch runs from a work
+// list: decode_plan_kernel, one small workgroup ahead of the split pass, reads the sequences'
+// counters and writes the items that have work, the longest first; workgroup j of the split pass
+// takes item j / H_KV for kv head j % H_KV, and the workgroups past the end of the list - all at
+// the end of the dispatch order - leave at once.
 struct WorkItem {
   int b, h, split;
-  bool crowded;
+  bool crowded, valid;
 };
-__device__ __forceinline__ WorkItem work_item_of_block(int h_kv, int num_splits, bool crowded) {
-  if (!crowded) return WorkItem{(int)blockIdx.z, (int)blockIdx.y, (int)blockIdx.x, false};
-  return WorkItem{(int)blockIdx.x / h_kv, (int)blockIdx.x % h_kv, num_splits - 1 - (int)blockIdx.y, true};
+__device__ __forceinline__ WorkItem work_item_of_block(int h_kv, const uint32_t* plan) {
+  if (!plan) return WorkItem{(int)blockIdx.z, (int)blockIdx.y, (int)blockIdx.x, false, true};
+  const uint32_t j = blockIdx.x / (uint32_t)h_kv;
+  if (j >= plan[0]) return WorkItem{0, 0, 0, true, false};
+  const uint32_t item = plan[kPlanHeader + j];
+  return WorkItem{(int)(item >> 16), (int)(blockIdx.x % (uint32_t)h_kv), (int)(item & 0xFFFFu), true, true};
 }
-constexpr int kCrowdedMinTiles = 8;    // body tiles per split a crowded launch aims for
+constexpr int kCrowdedMinTiles = 16;   // body tiles per split a crowded launch aims for
+constexpr int kCrowdedTailCost = 12;   // what the tail's split takes, in body tiles (for the order)
+// Body splits of a sequence with npp body tiles in a crowded launch (its split 0 is the tail's).
+__device__ __forceinline__ int crowded_body_splits(int npp, int num_splits) {
+  return npp > 0 ? min(num_splits - 1, c_div_up(npp, kCrowdedMinTiles)) : 0;
+}
+__device__ __forceinline__ int body_tiles_of(const SeqCounts& c) {
+  return min(min(c.pv, c.pk), c_div_up(c.nbody, kPage));
+}
+
+// The work list of a crowded launch: one workgroup.  Items are sorted by what they cost, longest
+// first (a counting sort over the cost in tiles), so that the last round is made of the shortest.
+constexpr int kPlanBuckets = 64;
+__global__ __launch_bounds__(256) void decode_plan_kernel(kitty_kv_layer L, int B, int num_splits,
+                                                          uint32_t* __restrict__ plan) {
+  __shared__ uint32_t s_n[kPlanBuckets], s_at[kPlanBuckets];
+  if (threadIdx.x < kPlanBuckets) s_n[threadIdx.x] = 0;
+  __syncthreads();
+  auto bucket = [](int cost) { return kPlanBuckets - 1 - min(cost, kPlanBuckets - 1); };   // longest first
+  // the shares of a sequence: nb body splits, of which the first rem have one tile more
+  auto shares = [&](int b, int& nb, int& base, int& rem) {
+    const int npp = body_tiles_of(load_counts(L, b));
+    nb = crowded_body_splits(npp, num_splits);
+    base = nb ? npp / nb : 0;
+    rem = nb ? npp - base * nb : 0;
+  };
+  for (int b = threadIdx.x; b < B; b += blockDim.x) {
+    int nb, base, rem;
+    shares(b, nb, base, rem);
+    atomicAdd(&s_n[bucket(kCrowdedTailCost)], 1u);
+    if (rem) atomicAdd(&s_n[bucket(base + 3)], (uint32_t)rem);
+    if (nb - rem) atomicAdd(&s_n[bucket(base + 2)], (uint32_t)(nb - rem));
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    uint32_t at = 0;
+    for (int i = 0; i < kPlanBuckets; ++i) { s_at[i] = at; at += s_n[i]; }
+    plan[0] = at;
+  }
+  __syncthreads();
+  for (int b = threadIdx.x; b < B; b += blockDim.x) {
+    int nb, base, rem;
+    shares(b, nb, base, rem);
+    const uint32_t row = (uint32_t)b << 16;
+    plan[kPlanHeader + atomicAdd(&s_at[bucket(kCrowdedTailCost)], 1u)] = row;
+    if (rem) {
+      const uint32_t at = atomicAdd(&s_at[bucket(base + 3)], (uint32_t)rem);
+      for (int i = 0; i < rem; ++i) plan[kPlanHeader + at + i] = row | (uint32_t)(1 + i);
+    }
+    if (nb - rem) {
+      const uint32_t at = atomicAdd(&s_at[bucket(base + 2)], (uint32_t)(nb - rem));
+      for (int i = rem; i < nb; ++i) plan[kPlanHeader + at + i - rem] = row | (uint32_t)(1 + i);
+    }
+  }
+}
 
 // How many of the first splits of a (batch row, kv head) take its tail (see wave_work).
 __device__ __forceinline__ int tail_splits(const SeqCounts& c, int num_splits, bool crowded) {
-  const int nbt = c_div_up(c.nbody, kPage);
-  const int npp = min(min(c.pv, c.pk), nbt);
-  if (crowded) return num_splits >= 2 ? 1 : 0;   // one after the other costs least when nothing runs beside it for free
+  if (crowded) return 1;   // one after the other costs least when nothing runs beside it for free
+  const int npp = body_tiles_of(c);
   return num_splits >= 4 && npp < 12 * (num_splits - 3) ? 3 : (num_splits >= 2 ? 1 : 0);
 }
 
@@ -1079,8 +1137,7 @@ __device__ __forceinline__ void wave_work(const kitty_kv_layer& L, const __half*
     // even shares: the first npp % n_body splits take one tile more.  A crowded launch gives a short
     // sequence fewer, longer shares; the splits past them have nothing to do.
     const int i_body = split - n_tail;
-    int n_body = num_splits - n_tail;
-    if (w.crowded) n_body = min(n_body, max(1, c_div_up(npp, kCrowdedMinTiles)));
+    const int n_body = w.crowded ? crowded_body_splits(npp, num_splits) : num_splits - n_tail;
     if (i_body < n_body) {
       const int base = npp / n_body, rem = npp - base * n_body;
       t0 = i_body * base + min(i_body, rem);
@@ -1254,6 +1311,20 @@ __device__ __forceinline__ void wave_work(const kitty_kv_layer& L, const __half*
 #pragma unroll
       for (int j = 0; j < 4; ++j) ws_acc[row * kD + 32 * x.kg + 8 * j + u] = A.out[u][j] + z;
   }
+  if constexpr (MODE == kWaveTail) {
+    // a crowded launch has no workgroups for the splits without work: the tail's split marks their
+    // partials as empty (the merge pass then does not read their accumulator rows)
+    if (w.crowded) {
+      const int s0 = 1 + crowded_body_splits(npp, num_splits);
+      const int n_empty = num_splits - s0;
+      for (int i = x.lane; i < G * n_empty; i += 64) {
+        const int g = i / n_empty, s = s0 + i - g * n_empty;
+        const int64_t row = ((int64_t)x.b * H_Q + (int64_t)x.h * G + g) * num_splits + s;
+        ws_ml[row * 2] = -INFINITY;
+        ws_ml[row * 2 + 1] = 0.f;
+      }
+    }
+  }
 }
 
 // The kernel's arguments, as one struct: the tail's function reads them where they lie.
@@ -1265,7 +1336,7 @@ struct KernArgs {
   float* ws_ml;
   float* ws_acc;
   int num_splits, n_simds;
-  int crowded;   // the grid is (units, reversed splits), see WorkItem
+  const uint32_t* plan;   // the work list of a crowded launch (see WorkItem), else NULL
 };
 
 __device__ __forceinline__ const KernArgs& kernel_args_of(const KernArgs* p) {   // the address as a scalar again
@@ -1285,7 +1356,7 @@ template <bool BOOST, bool DMA, bool QUARTER>
 __device__ __attribute__((noinline, noreturn)) void tail_wave(const KernArgs* kernel_args,
                                                                __attribute__((address_space(3))) WaveLds<DMA, QUARTER>* lds) {
   const KernArgs& a = kernel_args_of(kernel_args);
-  const WorkItem w = work_item_of_block(a.L.H_KV, a.num_splits, a.crowded != 0);
+  const WorkItem w = work_item_of_block(a.L.H_KV, a.plan);
   wave_work<BOOST, DMA, QUARTER, kWaveTail>(a.L, a.q, a.H_Q, a.scaling, a.ws_ml, a.ws_acc, a.num_splits, 0, w,
                                              *(WaveLds<DMA, QUARTER>*)lds);
   __builtin_amdgcn_endpgm();
@@ -1295,7 +1366,8 @@ __device__ __attribute__((noinline, noreturn)) void tail_wave(const KernArgs* ke
 template <bool BOOST, bool DMA, bool QUARTER, bool SOLO>
 __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(KernArgs a) {
   __shared__ WaveLds<DMA, QUARTER> S;
-  const WorkItem w = work_item_of_block(a.L.H_KV, a.num_splits, a.crowded != 0);
+  const WorkItem w = work_item_of_block(a.L.H_KV, a.plan);
+  if (!w.valid) return;
   if constexpr (SOLO) {
     wave_work<BOOST, DMA, QUARTER, kWaveSolo>(a.L, a.q, a.H_Q, a.scaling, a.ws_ml, a.ws_acc, a.num_splits, a.n_simds, w, S);
   } else {
@@ -1326,11 +1398,22 @@ struct LaunchArgs {
 };
 template <bool BOOST, bool DMA, bool QUARTER, bool SOLO>
 void launch_one(const LaunchArgs& a) {
-  const dim3 grid = a.k.crowded ? dim3(a.B * a.k.L.H_KV, a.k.num_splits, 1) : dim3(a.k.num_splits, a.k.L.H_KV, a.B);
+  const bool crowded = a.k.plan != nullptr;
+  const dim3 grid = crowded ? dim3((uint32_t)(a.B * a.k.L.H_KV * a.k.num_splits), 1, 1)
+                            : dim3(a.k.num_splits, a.k.L.H_KV, a.B);
   const dim3 block(64);
+  // a crowded launch is two kernels: the events take in both
+  if (crowded) {
+    uint32_t* plan = const_cast<uint32_t*>(a.k.plan);
+    if (a.ev_start)
+      hipExtLaunchKernelGGL(decode_plan_kernel, dim3(1), dim3(256), 0, a.stream, a.ev_start, nullptr, 0, a.k.L, a.B,
+                            a.k.num_splits, plan);
+    else
+      hipLaunchKernelGGL(decode_plan_kernel, dim3(1), dim3(256), 0, a.stream, a.k.L, a.B, a.k.num_splits, plan);
+  }
   if (a.ev_start)
-    hipExtLaunchKernelGGL((decode_mfma_kernel<BOOST, DMA, QUARTER, SOLO>), grid, block, 0, a.stream, a.ev_start,
-                          a.ev_stop, 0, a.k);
+    hipExtLaunchKernelGGL((decode_mfma_kernel<BOOST, DMA, QUARTER, SOLO>), grid, block, 0, a.stream,
+                          crowded ? nullptr : a.ev_start, a.ev_stop, 0, a.k);
   else
     hipLaunchKernelGGL((decode_mfma_kernel<BOOST, DMA, QUARTER, SOLO>), grid, block, 0, a.stream, a.k);
 }
@@ -1342,11 +1425,13 @@ void launch_variant(const LaunchArgs& a) {
 }  // namespace
 
 void launch_decode_mfma(const kitty_kv_layer& L, const void* q, int B, int H_Q, float scaling, float* ws_ml,
-                        float* ws_acc, int num_splits, int n_simds, hipStream_t stream, hipEvent_t ev_start,
-                        hipEvent_t ev_stop) {
+                        float* ws_acc, uint32_t* ws_plan, int num_splits, int n_simds, hipStream_t stream,
+                        hipEvent_t ev_start, hipEvent_t ev_stop) {
   const int64_t n_wg = (int64_t)B * L.H_KV * num_splits;
-  const int crowded = num_splits > 1 && num_splits <= 65535 && n_wg > 2 * (int64_t)n_simds ? 1 : 0;
-  const LaunchArgs a{KernArgs{L, (const __half*)q, H_Q, scaling, ws_ml, ws_acc, num_splits, n_simds, crowded}, B, stream, ev_start, ev_stop};
+  const bool crowded = num_splits > 1 && n_wg > 2 * (int64_t)n_simds && n_wg <= INT32_MAX;
+  const LaunchArgs a{KernArgs{L, (const __half*)q, H_Q, scaling, ws_ml, ws_acc, num_splits, n_simds,
+                              crowded ? ws_plan : nullptr},
+                     B, stream, ev_start, ev_stop};
   const int G = H_Q / L.H_KV;
   const bool boost = L.D_BOOSTED == 32, dma = G <= 8, quarter = G <= 4;
   if (boost && quarter) launch_variant<true, true, true>(a);

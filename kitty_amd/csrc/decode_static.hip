@@ -45,7 +45,7 @@ extern "C" int kitty_decode_attn_static(const kitty_kv_layer* layer, const void*
                                         void* out, int num_splits, int variant, void* stream) {
   KITTY_REQUIRE(layer && q && out, KITTY_E_NULL, "layer / q / out is NULL");
   KITTY_REQUIRE(B >= 1 && H_Q >= 1 && layer->H_KV >= 1, KITTY_E_RANGE, "bad B=%d, H_Q=%d or H_KV=%d", B, H_Q, layer->H_KV);
-  const size_t per_split = ws_total_bytes(B, H_Q, 1) + 256;   // an upper bound of the growth per split
+  const size_t per_split = ws_total_bytes(B, H_Q, 1) + 768;   // an upper bound of the growth per split
   if (num_splits <= 0) {
     // the default of kitty_decode_attn, cut back to what the array holds
     int max_tiles = 2 + layer->MAX_PAGE;

@@ -433,22 +433,26 @@ def test_decode_steps_cross_flushes(K):
     assert checked > 20 and ol.PageCount_K == 2 and ol.PageCount_V == 1 and ol.Write_Offset_Local_V != 0
 
 
-def test_ragged_batch_per_sequence_counts(K):
+@pytest.mark.parametrize("splits", [None, 3, 256])
+def test_ragged_batch_per_sequence_counts(K, splits):
     """Per-sequence occupancy (BASELINE config 2, scaled down): every row of the batch has its own
-    page counts, residual fill and ring offset; the oracle attends each row with its own counts."""
-    B, H_KV, H_Q = 5, 2, 8
+    page counts, residual fill and ring offset; the oracle attends each row with its own counts.
+    Rows 0 and 1 are shorter than the sink / than one page (no packed tiles at all).  256 splits:
+    more workgroups than the device holds at once (7 x 2 x 256 > 2 per SIMD), which the split pass
+    runs from a device-made work list."""
+    B, H_KV, H_Q = 7, 2, 8
     rng = np.random.default_rng(123)
     max_len = 32 + 128 * 12
     cache = K.KittyCache(K.u.cfg(H_KV, H_Q), B, max_len)
     L = cache.kv_cache[0]
     ols, counts = [], []
     for b in range(B):
-        T = int(rng.integers(40, max_len - 130))
+        T = 20 if b == 0 else 100 if b == 1 else int(rng.integers(40, max_len - 130))
         k, v = make_kv(1, H_KV, T + 150, seed=500 + b)
         ol = O.OracleLayer(1, max_len, H_KV)
         ol.update(k[:, :, :T], v[:, :, :T])
         ol.quantize_prefill()
-        for s in range(int(rng.integers(0, 150))):           # some decode steps: ring offset != 0
+        for s in range(0 if b < 2 else int(rng.integers(0, 150))):   # some decode steps: ring offset != 0
             ol.update(k[:, :, T + s:T + s + 1], v[:, :, T + s:T + s + 1])
             ol.quantize_decode()
         ols.append(ol)
@@ -462,7 +466,7 @@ def test_ragged_batch_per_sequence_counts(K):
     L.seq_counts = torch.tensor(counts, dtype=torch.int32, device="cuda")
     q = make_q(B, H_Q, seed=9)
     for variant in (0, 1):
-        out, _ = K.attn(K.u.module(H_KV, H_Q), K.u.to_dev(q), L, 128 ** -0.5, variant=variant)
+        out, _ = K.attn(K.u.module(H_KV, H_Q), K.u.to_dev(q), L, 128 ** -0.5, variant=variant, num_splits=splits)
         got = _np16(out).astype(np.float64)
         for b in range(B):
             _check_attn(got[b:b + 1], ols[b], q[b:b + 1], what=f"variant {variant} row {b}", variant=variant)
