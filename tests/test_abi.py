@@ -114,7 +114,9 @@ def test_host_side_rejection_without_gpu(lib):
     L.cache_pages_v = 4
     L.PAGE_SIZE = 256
     assert lib.kitty_flush_full(ctypes.byref(L), 1, None) == E_SHAPE
-    assert lib.kitty_decode_attn_workspace_bytes(16, 32, 128, 16) == 16 * 32 * 16 * 2 * 4 + 16 * 32 * 16 * 128 * 4
+    # the partials (max / sum pairs, then accumulator rows) and, 256-aligned, a work list of 4 + B * splits words
+    assert lib.kitty_decode_attn_workspace_bytes(16, 32, 128, 16) == (
+        16 * 32 * 16 * 2 * 4 + 16 * 32 * 16 * 128 * 4 + (4 + 16 * 16) * 4 + 240)
     assert lib.kitty_decode_attn_workspace_bytes(16, 32, 64, 16) == 0
     ds = lib.kitty_decode_attn_default_splits
     assert 1 <= ds(16, 8, 257, 0) <= 257
