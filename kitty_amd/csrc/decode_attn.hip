@@ -41,24 +41,32 @@ int device_simds() {
 }
 }  // namespace kitty
 
-// Enough single-wave workgroups to put two on every SIMD of the device, but no body split with fewer
-// than 4 tiles (a wave's fixed cost is about one tile's worth); three more for the sink and the
-// tiles with fp16 rows when the body splits are short.  When the splits are short (under 8 tiles)
-// the waves with the fp16 rows are the critical path, and a launch that fills the machine exactly
-// puts two of them on the same SIMD (workgroup i shares a SIMD with i + SIMDs): 15/16 of the
-// machine is faster then (B=1, 128k tokens: 32 us with 240 splits, 40 us with 256).  Sequences with
-// their own lengths (per_sequence_counts) get at least 12 splits when they can be long: more,
-// shorter splits even out the load.
+// Enough single-wave workgroups to put two on every SIMD of the device.  When the splits are short
+// (under 8 tiles) the waves with the fp16 rows are the critical path, and a launch that fills the
+// machine exactly puts two of them on the same SIMD (workgroup i shares a SIMD with i + SIMDs):
+// 15/16 of the machine is faster then (B=1, 128k tokens: 32 us with 240 splits, 40 us with 256).
+// A short context is latency, not bandwidth: a body split of 2.5 tiles (a wave's fixed cost is
+// about two tiles' worth) plus three splits for the sink and the tiles with fp16 rows (B=1, 4k
+// tokens: 11.4 us with 16 splits, 13.5 with 12, 17.4 with 8; 16k tokens: 14.0 us with 54, 15.8 with
+// 36), and then, if it can be had with body splits of 4 tiles or fewer, a launch of at most 3/4 of
+// a workgroup per SIMD, in which no two waves share one (B=4, 8k tokens: 15.0 us with 24 splits,
+// 16.8 with 32, 23.9 with 64).  Sequences with their own lengths (per_sequence_counts) get at least
+// 12 splits when they can be long: more, shorter splits even out the load.
 extern "C" int kitty_decode_attn_default_splits(int B, int H_KV, int max_tiles, int per_sequence_counts) {
   if (B <= 0 || H_KV <= 0 || max_tiles <= 0) return 1;
-  const int units = B * H_KV, slots = 2 * device_simds();
-  int s = (slots + units - 1) / units;
+  const int64_t units = (int64_t)B * H_KV;
+  const int simds = device_simds(), slots = 2 * simds;
+  int64_t s = (slots + units - 1) / units;
   if (max_tiles < 8 * s) s = (slots - slots / 16 + units - 1) / units;
-  const int by_tiles = (max_tiles + 3) / 4 + 3;
-  if (s > by_tiles) s = by_tiles;
+  const int by_tiles = 2 * max_tiles / 5 + 3, by_tiles_long = (max_tiles + 3) / 4 + 3;
+  if (s > by_tiles) {
+    s = by_tiles;
+    const int64_t calm = 3 * simds / 4 / units;
+    if (s > calm) s = calm > by_tiles_long ? calm : (s < by_tiles_long ? s : by_tiles_long);
+  }
   if (per_sequence_counts && s < 12 && max_tiles >= 48) s = 12;
   if (s > 512) s = 512;
-  return s < 1 ? 1 : s;
+  return s < 1 ? 1 : (int)s;
 }
 
 namespace {
