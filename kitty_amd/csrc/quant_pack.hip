@@ -144,7 +144,10 @@ __device__ __forceinline__ void quant_k_page(const ROWS row_of, int d_boost,
   constexpr int kPitch = kD + 16;
   __shared__ __attribute__((aligned(16))) float s_pmin[16][kPitch];   // later: the low plane on its way out
   __shared__ float s_pmax[16][kPitch];
-  __shared__ double s_psum[MODE == 0 ? 1 : 16][kPitch];
+  __shared__ float s_psum[MODE == 0 ? 1 : 16][kPitch];
+  __shared__ unsigned long long s_exact[MODE == 0 ? 1 : kD];   // [pos]: exact sum of |x| * 2^24 where fp32 leaves a doubt
+  __shared__ uint8_t s_doubt[MODE == 0 ? 1 : kD];              // [pos]
+  __shared__ int s_any_doubt;
   __shared__ float4 s_q[kD];   // [pos]: min, scale, refined reciprocal of the scale, qmax + 0.5
   __shared__ float s_c0[kD];   // [pos]: the fast path's offset (fast_offset)
   __shared__ __attribute__((aligned(16))) uint32_t s_key[kD];   // score << 8 | (127 - channel): larger sorts first
@@ -158,7 +161,8 @@ __device__ __forceinline__ void quant_k_page(const ROWS row_of, int d_boost,
   for (int r = 0; r < 8; ++r) rows[r] = nt_load16(row_of(tg * 8 + r) + c8 * 16);
 
   // this thread's 8 tokens x 8 channels as floats, and per channel the partial min / max (/ sum
-  // of |x|: exact in fp64, every term is a multiple of 2^-24 below 2^16)
+  // of |x| in fp32: good enough to rank nearly every channel, see below)
+  if (MODE != 0 && tid == 0) s_any_doubt = 0;
   float xs[8][8];   // [channel j][token r]
 #pragma unroll
   for (int j = 0; j < 8; ++j) {
@@ -168,16 +172,16 @@ __device__ __forceinline__ void quant_k_page(const ROWS row_of, int d_boost,
       xs[j][r] = h2f((j & 1) ? (uint16_t)(w >> 16) : (uint16_t)(w & 0xffffu));
     }
     float mn = xs[j][0], mx = xs[j][0];
-    double sum = 0.0;
 #pragma unroll
     for (int r = 0; r < 8; ++r) {
       mn = fminf(mn, xs[j][r]);
       mx = fmaxf(mx, xs[j][r]);
-      if (MODE != 0) sum += (double)fabsf(xs[j][r]);
     }
     s_pmin[tg][j * 16 + c8] = mn;
     s_pmax[tg][j * 16 + c8] = mx;
-    if (MODE != 0) s_psum[tg][j * 16 + c8] = sum;
+    if (MODE != 0)   // added as a tree: every term goes through three additions
+      s_psum[tg][j * 16 + c8] = ((fabsf(xs[j][0]) + fabsf(xs[j][1])) + (fabsf(xs[j][2]) + fabsf(xs[j][3]))) +
+                                ((fabsf(xs[j][4]) + fabsf(xs[j][5])) + (fabsf(xs[j][6]) + fabsf(xs[j][7])));
   }
   __syncthreads();
 
@@ -195,15 +199,61 @@ __device__ __forceinline__ void quant_k_page(const ROWS row_of, int d_boost,
   ch_min = fminf(ch_min, __shfl_xor(ch_min, 1));
   ch_max = fmaxf(ch_max, __shfl_xor(ch_max, 1));
   if (MODE != 0) {
-    double sum = 0.0;
-#pragma unroll
-    for (int i = 0; i < 16; i += 2) sum += s_psum[i + hf][pos];
+    // The score is the mean of |x| over the page, rounded ONCE to fp16.  In the fp32 sum of the 128
+    // non-negative terms every term went through 7 additions (3 in its thread, 3 in this fold, 1
+    // between the lanes), each with a relative error of at most 2^-24, so the exact mean lies within
+    // 7.01 * 2^-24 (relative) of sum / 128.  The ends of the interval tested are that mean times
+    // 1 -+ 10 * 2^-24 (both factors are fp32 numbers; the products round once more).  If both ends
+    // round to the same fp16 number, that is the score; otherwise (one channel in about 600: the
+    // interval contains a midpoint between two fp16 numbers; one page-head in five has such a
+    // channel), or when the mean is so small that fp16 has no normal number for it, the channel's
+    // 16 threads add their terms exactly - every |x| is a multiple of 2^-24 below 2^16 - into a
+    // 64-bit integer.
+    float sum = ((s_psum[hf][pos] + s_psum[2 + hf][pos]) + (s_psum[4 + hf][pos] + s_psum[6 + hf][pos])) +
+                ((s_psum[8 + hf][pos] + s_psum[10 + hf][pos]) + (s_psum[12 + hf][pos] + s_psum[14 + hf][pos]));
     sum += __shfl_xor(sum, 1);
-    // an integer below 2^47 (or inf / nan for non-finite inputs, which saturate)
-    if (hf == 0)
-      s_key[ch] = ((uint32_t)mean_abs_fp16_bits(sum < 1.8e19 ? (uint64_t)(sum * 16777216.0) : ~0ull) << 8) |
-                  (uint32_t)(kD - 1 - ch);
+    if (hf == 0) {
+      uint32_t score = 0;
+      bool doubt = false;
+      if (!(sum < 3.0e38f)) {
+        score = 0x7C00;   // inf or NaN among the inputs: saturates
+      } else if (sum != 0.f) {
+        const float mean = sum * (1.0f / kPage);
+        const uint16_t lo = __half_as_ushort(__float2half_rn(mean * (1.0f - 0x1.4p-21f)));
+        const uint16_t hi = __half_as_ushort(__float2half_rn(mean * (1.0f + 0x1.4p-21f)));
+        doubt = lo != hi || mean < 0x1p-13f;
+        score = lo;
+      }
+      s_doubt[pos] = doubt;
+      if (doubt) {
+        s_exact[pos] = 0;
+        s_any_doubt = 1;
+      } else {
+        s_key[ch] = (score << 8) | (uint32_t)(kD - 1 - ch);
+      }
+    }
     __syncthreads();
+    if (s_any_doubt) {   // the same for every thread of the workgroup
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        if (s_doubt[j * 16 + c8]) {
+          // |x| * 2^24 is an integer below 2^40: its bits from 2^20 up and the rest, added apart
+          uint32_t up = 0, low = 0;
+#pragma unroll
+          for (int r = 0; r < 8; ++r) {
+            const float v = fabsf(xs[j][r]) * 0x1p24f;
+            const float u = floorf(v * 0x1p-20f);
+            up += (uint32_t)u;
+            low += (uint32_t)__builtin_fmaf(u, -0x1p20f, v);
+          }
+          atomicAdd(&s_exact[j * 16 + c8], ((unsigned long long)up << 20) + low);
+        }
+      }
+      __syncthreads();
+      if (hf == 0 && s_doubt[pos])
+        s_key[ch] = ((uint32_t)mean_abs_fp16_bits(s_exact[pos]) << 8) | (uint32_t)(kD - 1 - ch);
+      __syncthreads();
+    }
     // rank = number of channels that sort before this one: higher score, or equal score and
     // lower channel index
     const uint32_t mine = s_key[ch];

@@ -168,6 +168,55 @@ def test_quantize_pack_bit_exact_awkward_groups(K):
     assert np.array_equal(_np16(vc), ovc)
 
 
+def test_boost_selection_scores_at_fp16_midpoints(K):
+    """The selection ranks channels by mean |k| rounded once to fp16.  The kernel adds in fp32 and
+    redoes a channel exactly when that leaves the rounding open; these channels are built so that it
+    does: means exactly on the midpoint between two fp16 numbers (round to even), one fp16 subnormal
+    (2^-24 in one token of 128) above or below it, ties between channels (lower index first), means
+    below the smallest normal fp16 number, and a mean that overflows fp16."""
+    rng = np.random.default_rng(5)
+    B, H, P, t0 = 1, 2, 2, 32
+    T = t0 + P * 128
+    k = (0.05 * rng.standard_normal((B, H, T, 128))).astype(np.float16)   # background: small scores
+    pg = np.ones((128, 40), np.float64)                  # 40 crafted channels with scores near 1
+    pg[0, 0] = 1.0625                                    # sum 128 + 2^-4: mean 1 + 2^-11, the midpoint -> 1 (even)
+    pg[0, 1], pg[1, 1] = 1.0625, 1.0 + 2.0 ** -10        # just above the midpoint -> 1 + 2^-10
+    pg[0, 2], pg[1, 2] = 1.0625, 1.0 - 2.0 ** -11        # just below -> 1
+    pg[0, 3], pg[1, 3], pg[2, 3] = 1.0625, 2.0, 2.0 ** -24   # 128.0625 + 2^-24: above by less than fp32 can tell
+    pg[0, 4] = 1.0 + 3 * 2.0 ** -4                       # mean 1 + 3 * 2^-11: midpoint -> 1 + 2^-9 (even)
+    pg[:, 5] = 1.0                                       # ties with channels 0 and 2: index order
+    pg[0, 6], pg[1, 6], pg[2, 6] = 1.0625, 0.5, 1.5      # the first midpoint again, from other terms
+    pg[:, 7] = 1000.0; pg[0, 7] = 1032.0                 # mean 1000.25: midpoint of spacing 0.5 -> 1000 (even)
+    pg[:, 8] = 1000.0; pg[0, 8], pg[1, 8], pg[2, 8] = 1032.0, 2000.0, 2.0 ** -24   # 2^-24 above it -> 1000.5
+    pg[:, 9] = 1000.0; pg[0, 9], pg[1, 9] = 1032.0, 1000.5   # well above -> 1000.5
+    pg[:, 10] = 65504.0                                  # mean 65504 = the largest fp16 number
+    pg[:, 11] = 65504.0; pg[0, 11] = 65472.0             # just below it
+    pg[:, 12:20] = 2.0 ** -24 * rng.integers(0, 3, size=(128, 8))         # means of a few fp16 subnormal steps
+    pg[:, 20:28] = 2.0 ** -14 * rng.integers(0, 2, size=(128, 8))         # means around the smallest normal
+    pg[:, 28:40] = 1.0 + 2.0 ** -10 * rng.integers(0, 2, size=(128, 12))  # many near-ties on a 2^-17 grid
+    pg[0, 28:40] += 0.0625
+    pg16 = pg.astype(np.float16)
+    assert np.array_equal(pg16.astype(np.float64), pg)   # every crafted value is an fp16 number
+    for h in range(H):
+        for p_ in range(P):
+            cols = rng.permutation(128)[:40]             # scattered over the head's channels
+            sign = rng.choice([-1.0, 1.0], size=(128, 40))
+            k[0, h, t0 + p_ * 128:t0 + (p_ + 1) * 128, cols] = (pg16 * sign).astype(np.float16).T
+    pt = np.arange(B * 4, dtype=np.int64).reshape(B, 4)
+    lay = O.Layout(H_KV=H)
+    okc = np.zeros((B * 4, lay.bytes_per_page_K), np.uint8)
+    okm = np.zeros((B * 4, H, 128, 2), np.float16)
+    used = O.quantize_pack_k(k, t0, P, pt, 0, okc, okm, 128, 32)
+    kc, km = K.u.to_dev(np.zeros_like(okc)), K.u.to_dev(np.zeros_like(okm))
+    kd, ptd = K.u.to_dev(k), K.u.to_dev(pt)
+    K.qk(kd, t0, P, ptd, 0, kc, km, 128, 32)
+    sm = K.sel(kd, t0, P, 128, 32)
+    torch.cuda.synchronize()
+    assert np.array_equal(_np16(sm), used)
+    assert np.array_equal(_np16(kc), okc)
+    assert np.array_equal(_np16(km).view(np.uint16), okm.view(np.uint16))
+
+
 def test_quantize_strided_source_no_copy(K):
     """[B, T, H, D] projections transposed to [B, H, T, D] are read through their strides."""
     B, H, T = 1, 2, 128 * 2
