@@ -99,3 +99,60 @@ def test_static_entry_point_rejects_what_does_not_fit(K):
     assert lib.kitty_decode_attn_static(L.descriptor(), q.data_ptr(), 2, 7, SC, out.data_ptr(), 2, 0, st) == -2
     torch.cuda.synchronize()
     assert not out.any()
+
+
+def test_decode_step_replayed_from_a_graph(K):
+    """What the entry point is for: one decode step of a layer - append the new token, attend, flush
+    the full Q-buffers - captured once in a HIP graph (per-sequence counters on the device, so the
+    kernels' arguments never change) and replayed step after step, with eager copies into the
+    graph's input buffers and synchronisations in between.  Every replay must give, bit for bit,
+    what the same step gives eagerly on a twin cache through the workspace entry point; the steps
+    cross a flush of both Q-buffers."""
+    from kitty_amd.kvcache.kernels import kitty_attention_forward
+    B, H_KV, H_Q, T, steps = 2, 2, 8, 32 + 128 + 100, 40
+    k, v = make_kv(B, H_KV, T + steps, seed=71)
+    twins = []
+    for _ in range(2):
+        c = K.KittyCache(K.u.cfg(H_KV, H_Q), B, 1024)
+        assert c.update(K.u.to_dev(k[:, :, :T]), K.u.to_dev(v[:, :, :T]), 0) is True
+        c.quantize_prefill(0)
+        c.enable_device_counters()
+        twins.append(c)
+    eager, graphed = twins
+    lib = K.lib.lib()
+    L = graphed.kv_cache[0]
+    kin = torch.zeros((B, H_KV, 1, 128), dtype=torch.float16, device="cuda")
+    vin, qin = torch.zeros_like(kin), torch.zeros((B, H_Q, 1, 128), dtype=torch.float16, device="cuda")
+    out = torch.zeros((B, 1, H_Q, 128), dtype=torch.float16, device="cuda")
+    desc = L.descriptor()
+
+    def step(stream):
+        rc = lib.kitty_append_token(desc, kin.data_ptr(), vin.data_ptr(), kin.stride(0) * 2, kin.stride(1) * 2,
+                                    None, None, 0, B, stream)
+        rc = rc or lib.kitty_decode_attn_static(desc, qin.data_ptr(), B, H_Q, SC, out.data_ptr(), 0, 0, stream)
+        return rc or lib.kitty_flush_full(desc, B, stream)
+
+    # the first call on a device asks the runtime where the library's array lies: not under capture
+    assert lib.kitty_decode_attn_static(desc, qin.data_ptr(), B, H_Q, SC, out.data_ptr(), 0, 0,
+                                        K.lib.current_stream_ptr(qin.device)) == 0
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):   # capture records, it does not run: the cache is untouched until the first replay
+        rc = step(torch.cuda.current_stream().cuda_stream)
+    assert rc == 0, lib.kitty_last_error()
+    mod = K.u.module(H_KV, H_Q)
+    for s in range(steps):
+        kn, vn = K.u.to_dev(k[:, :, T + s:T + s + 1]), K.u.to_dev(v[:, :, T + s:T + s + 1])
+        q = K.u.to_dev(make_q(B, H_Q, seed=200 + s))
+        assert eager.update(kn, vn, 0) is False
+        want, _ = kitty_attention_forward(mod, q, eager.kv_cache[0], SC)
+        eager.quantize_decode(0)
+        kin.copy_(kn), vin.copy_(vn), qin.copy_(q)
+        g.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, want), f"step {s}"
+    a, b = eager.kv_cache[0], L
+    assert torch.equal(a.seq_counts, b.seq_counts)
+    assert int(a.seq_counts[0, 1]) == 2 and int(a.seq_counts[0, 3]) == 1          # both Q-buffers were flushed
+    for name in ("KeyCache", "KeyCache_metadata", "ValueCache", "ValueCache_metadata", "Q_Buffer_K", "Local_Buffer_V"):
+        assert torch.equal(getattr(a, name), getattr(b, name)), name
