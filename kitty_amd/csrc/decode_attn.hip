@@ -98,6 +98,8 @@ int check_layer(const kitty_kv_layer* layer, const void* q, int B, int H_Q, int*
                     ((uintptr_t)L.local_v % 16) == 0 && L.sink_stride_b % 16 == 0 && L.sink_stride_h % 16 == 0 &&
                     L.win_stride_b % 16 == 0 && L.win_stride_h % 16 == 0 && ((uintptr_t)q % 16) == 0,
                 KITTY_E_ALIGN, "cache tensors and q need 16-byte alignment");
+  KITTY_REQUIRE(L.cache_pages_k <= INT32_MAX && L.cache_pages_v <= INT32_MAX, KITTY_E_RANGE,
+                "cache_pages_k / cache_pages_v beyond 2^31 - 1 (page ids travel as 32-bit numbers inside the kernels)");
   KITTY_REQUIRE(L.cache_pages_k >= 0 && L.cache_pages_v >= 0 && ((uintptr_t)L.status % 4) == 0 &&
                     ((uintptr_t)L.seq_counts % 4) == 0,
                 KITTY_E_RANGE, "negative cache_pages_k / cache_pages_v, or misaligned status / seq_counts");

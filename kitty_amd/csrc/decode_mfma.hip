@@ -978,23 +978,34 @@ __global__ __launch_bounds__(256) void decode_plan_kernel(kitty_kv_layer L, int 
     base = nb ? npp / nb : 0;
     rem = nb ? npp - base * nb : 0;
   };
+  // (a thread keeps the shares of its first sequence for the second pass: with up to 256 sequences
+  // the counters are read once)
+  int nb0 = 0, base0 = 0, rem0 = 0;
   for (int b = threadIdx.x; b < B; b += blockDim.x) {
     int nb, base, rem;
     shares(b, nb, base, rem);
+    if (b == (int)threadIdx.x) nb0 = nb, base0 = base, rem0 = rem;
     atomicAdd(&s_n[bucket(kCrowdedTailCost)], 1u);
     if (rem) atomicAdd(&s_n[bucket(base + 3)], (uint32_t)rem);
     if (nb - rem) atomicAdd(&s_n[bucket(base + 2)], (uint32_t)(nb - rem));
   }
   __syncthreads();
-  if (threadIdx.x == 0) {
-    uint32_t at = 0;
-    for (int i = 0; i < kPlanBuckets; ++i) { s_at[i] = at; at += s_n[i]; }
-    plan[0] = at;
+  if (threadIdx.x < kPlanBuckets) {   // the first wave: where each bucket starts
+    static_assert(kPlanBuckets == 64, "one bucket per lane");
+    const uint32_t n = s_n[threadIdx.x];
+    uint32_t upto = n;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+      const uint32_t v = __shfl_up(upto, o);
+      if ((int)threadIdx.x >= o) upto += v;
+    }
+    s_at[threadIdx.x] = upto - n;
+    if (threadIdx.x == kPlanBuckets - 1) plan[0] = upto;
   }
   __syncthreads();
   for (int b = threadIdx.x; b < B; b += blockDim.x) {
-    int nb, base, rem;
-    shares(b, nb, base, rem);
+    int nb = nb0, base = base0, rem = rem0;
+    if (b != (int)threadIdx.x) shares(b, nb, base, rem);
     const uint32_t row = (uint32_t)b << 16;
     plan[kPlanHeader + atomicAdd(&s_at[bucket(kCrowdedTailCost)], 1u)] = row;
     if (rem) {

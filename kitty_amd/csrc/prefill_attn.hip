@@ -133,6 +133,31 @@ struct Prefill {
   int n_tiles;       // sink + body + chunk tiles actually walked
   int first_body, first_chunk;
   mutable int bad_page = 0;   // a page id outside the cache was met (checked_page)
+  // Page ids reach tile() through LDS, checked: kIdChunk body tiles at a time, the K and V ids are
+  // read by one thread each, range-checked (checked_page) and left as 32-bit numbers in one of two
+  // chunk buffers; the chunk after the current one is staged when the walk is half way through the
+  // current one, and the barrier that ends every iteration of the walk publishes it.  Reading and
+  // checking the ids where they are used - a load whose value the next instructions need, in every
+  // iteration of every workgroup - cost this kernel 10 %.
+  static constexpr int kIdChunk = 64;
+  int32_t (*page_ids)[2][kIdChunk];   // [chunk & 1][K, V][body tile % kIdChunk]
+
+  __device__ __forceinline__ void stage_page_ids(int chunk) const {
+    if (tid < 2 * kIdChunk) {
+      const int side = tid / kIdChunk, i = chunk * kIdChunk + tid % kIdChunk;
+      if (i < (side ? c.pv : c.pk)) {
+        const int64_t pg = side ? L.page_table_v[(int64_t)b * L.page_table_v_stride_b + i]
+                                : L.page_table_k[(int64_t)b * L.page_table_k_stride_b + i];
+        page_ids[chunk & 1][side][tid % kIdChunk] =
+            (int32_t)checked_page(pg, side ? L.cache_pages_v : L.cache_pages_k, bad_page);
+      }
+    }
+  }
+  // (every lane reads the same word and keeps it in a vector register: made a scalar again with
+  // v_readfirstlane, with the tile addresses then computed on the scalar unit, the kernel is 4 % slower)
+  __device__ __forceinline__ int64_t staged_page(int side, int i) const {
+    return page_ids[(i / kIdChunk) & 1][side][i % kIdChunk];
+  }
 
   __device__ TileSrc tile(int t) const {
     TileSrc s;
@@ -151,7 +176,7 @@ struct Prefill {
       const int i = t - first_body;
       s.ntok = min(kPage, c.nbody - i * kPage);
       if (i < c.pk) {
-        const int64_t pg = checked_page(page_id(L.page_table_k, (int64_t)b * L.page_table_k_stride_b + i), L.cache_pages_k, bad_page);
+        const int64_t pg = staged_page(0, i);
         s.k_kind = SRC_PACKED;
         s.k_ptr = L.key_cache + pg * L.key_cache_stride_page + (int64_t)h * k_head_bytes(L.D_BOOSTED);
         s.k_meta = (const uint8_t*)L.key_meta + pg * L.key_meta_stride_page + (int64_t)h * kD * 4;
@@ -161,7 +186,7 @@ struct Prefill {
         s.k_stride = kD * 2;
       }
       if (i < c.pv) {
-        const int64_t pg = checked_page(page_id(L.page_table_v, (int64_t)b * L.page_table_v_stride_b + i), L.cache_pages_v, bad_page);
+        const int64_t pg = staged_page(1, i);
         s.v_kind = SRC_PACKED;
         s.v_ptr = L.value_cache + pg * L.value_cache_stride_page + (int64_t)h * kVBytes;
         s.v_meta = (const uint8_t*)L.value_meta + pg * L.value_meta_stride_page + (int64_t)h * kPage * 4;
@@ -449,6 +474,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(kWaves
     const uint8_t* __restrict__ k_new, const uint8_t* __restrict__ v_new, int64_t new_stride_b,
     int64_t new_stride_h, int64_t new_stride_t, int H_Q, int Tq, float scaling, __half* __restrict__ out) {
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+  __shared__ int32_t s_page_ids[2][2][Prefill<BOOST>::kIdChunk];
   const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, kg = lane >> 4, n = lane & 15;
   const int b = blockIdx.z, h = blockIdx.y;
   const int G = H_Q / L.H_KV;
@@ -461,6 +487,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(kWaves
                    k_new + (int64_t)b * new_stride_b + (int64_t)h * new_stride_h,
                    v_new + (int64_t)b * new_stride_b + (int64_t)h * new_stride_h,
                    new_stride_t, min(Tq, p0 + PB), 0, 0, 0, 0};
+  P.page_ids = s_page_ids;
   P.n_body = c_div_up(cnt.nbody, kPage);
   P.first_body = cnt.sink > 0 ? 1 : 0;
   P.first_chunk = P.first_body + P.n_body;
@@ -506,6 +533,8 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(kWaves
   const int nt_ = P.n_tiles;
   const bool convert_first = w < kWaves / 2;
   Stage ga, gb;                       // tile t+1, tile t+2
+  P.stage_page_ids(0);
+  __syncthreads();
   TileSrc cur = P.tile(0), nxt = cur, nn = cur;
   P.issue(cur, ga);
   P.finish(cur, ga, lds, lds + 2 * kTile);
@@ -521,6 +550,10 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(kWaves
     if (t + 2 < nt_) {
       nn = P.tile(t + 2);
       P.issue(nn, gb);
+    }
+    {   // half way through a chunk of page ids: stage the next one (tile() is at body tile t + 2 - first_body)
+      const int i = t + 2 - P.first_body;
+      if (i >= 0 && i % Prefill<BOOST>::kIdChunk == Prefill<BOOST>::kIdChunk / 2) P.stage_page_ids(i / Prefill<BOOST>::kIdChunk + 1);
     }
     uint8_t* kn = lds + (buf ^ 1) * kTile;
     uint8_t* vn = lds + (2 + (buf ^ 1)) * kTile;
@@ -565,7 +598,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(kWaves
       *(__half2*)(orow + 16 * ct + 2 * kg + 8) = __floats2half2_rn(o[1], o[3]);
     }
   }
-  if (tid == 0) report_bad_page(L, b, P.bad_page);
+  report_bad_page(L, b, P.bad_page);   // by whichever thread met one
 }
 
 }  // namespace
