@@ -521,6 +521,49 @@ def test_ragged_batch_per_sequence_counts(K, splits):
             _check_attn(got[b:b + 1], ols[b], q[b:b + 1], what=f"variant {variant} row {b}", variant=variant)
 
 
+def test_more_sequences_than_the_device_holds_workgroups(K):
+    """260 sequences x 8 kv heads: more (row, kv head) units than the device holds workgroups at
+    once, so even two splits make a launch of several rounds, and the kernel that lists the work
+    walks more rows than it has threads.  Five prototype sequences (sink only, no packed page, one
+    to three pages, some with decode steps behind them) repeated over the rows, each row with its own
+    query; the oracle attends every row with its prototype's counters."""
+    B, H_KV, H_Q = 260, 8, 8
+    max_len = 32 + 128 * 4
+    cache = K.KittyCache(K.u.cfg(H_KV, H_Q), B, max_len)
+    L = cache.kv_cache[0]
+    protos = []
+    for i, (T, steps) in enumerate([(20, 0), (100, 0), (32 + 128 + 5, 0), (32 + 128 * 2 + 77, 60), (32 + 128 * 3 + 100, 20)]):
+        k, v = make_kv(1, H_KV, T + steps, seed=700 + i)
+        ol = O.OracleLayer(1, max_len, H_KV)
+        ol.update(k[:, :, :T], v[:, :, :T])
+        ol.quantize_prefill()
+        for s_ in range(steps):
+            ol.update(k[:, :, T + s_:T + s_ + 1], v[:, :, T + s_:T + s_ + 1])
+            ol.quantize_decode()
+        dev = {name: K.u.to_dev(getattr(ol, name)) for name in
+               ("Sink_Buffer_K", "Sink_Buffer_V", "Q_Buffer_K", "Q_Buffer_V", "Local_Buffer_V", "KeyCache",
+                "KeyCache_metadata", "ValueCache", "ValueCache_metadata")}
+        protos.append((ol, dev, [ol.Sink_Count, ol.PageCount_K, ol.Q_Buffer_Count_K, ol.PageCount_V, ol.Q_Buffer_Count_V,
+                                 ol.Local_Count_V, ol.Write_Offset_Local_V, 0]))
+    rng = np.random.default_rng(8)
+    which = rng.integers(0, len(protos), size=B)
+    for b in range(B):
+        ol, dev, _ = protos[which[b]]
+        for name in ("Sink_Buffer_K", "Sink_Buffer_V", "Q_Buffer_K", "Q_Buffer_V", "Local_Buffer_V"):
+            getattr(L, name)[b].copy_(dev[name][0])
+        for name in ("KeyCache", "KeyCache_metadata", "ValueCache", "ValueCache_metadata"):
+            getattr(L, name)[b * L.MAX_PAGE:(b + 1) * L.MAX_PAGE].copy_(dev[name])
+    L.seq_counts = torch.tensor([protos[w][2] for w in which], dtype=torch.int32, device="cuda")
+    q = make_q(B, H_Q, seed=10)
+    want = {}
+    for splits in (2, 5):
+        out, _ = K.attn(K.u.module(H_KV, H_Q), K.u.to_dev(q), L, 128 ** -0.5, variant=0, num_splits=splits)
+        got = _np16(out).astype(np.float64)
+        assert np.isfinite(got).all()
+        for b in range(0, B, 1 if splits == 2 else 7):
+            _check_attn(got[b:b + 1], protos[which[b]][0], q[b:b + 1], what=f"splits {splits} row {b}", variant=0)
+
+
 def test_all_equal_keys_give_mean_of_values(K):
     """Closed form: identical keys -> uniform weights -> output = mean of the dequantized values."""
     B, H_KV, H_Q, T = 1, 1, 4, 32 + 128 * 3
