@@ -50,8 +50,10 @@ int device_simds() {
 // tokens: 11.4 us with 16 splits, 13.5 with 12, 17.4 with 8; 16k tokens: 14.0 us with 54, 15.8 with
 // 36), and then, if it can be had with body splits of 4 tiles or fewer, a launch of at most 3/4 of
 // a workgroup per SIMD, in which no two waves share one (B=4, 8k tokens: 15.0 us with 24 splits,
-// 16.8 with 32, 23.9 with 64).  Sequences with their own lengths (per_sequence_counts) get at least
-// 12 splits when they can be long: more, shorter splits even out the load.
+// 16.8 with 32, 23.9 with 64), else one of at most six workgroups per compute unit (B=2, 32k tokens:
+// 18.0 us with 96 splits, 19.5 with 48 or 68, 18.6 with 120; B=1, 64k: 18.8 with 192, 20.2 with 132).
+// Sequences with their own lengths (per_sequence_counts) get at least 12 splits when they can be
+// long: more, shorter splits even out the load.
 extern "C" int kitty_decode_attn_default_splits(int B, int H_KV, int max_tiles, int per_sequence_counts) {
   if (B <= 0 || H_KV <= 0 || max_tiles <= 0) return 1;
   const int64_t units = (int64_t)B * H_KV;
@@ -61,8 +63,8 @@ extern "C" int kitty_decode_attn_default_splits(int B, int H_KV, int max_tiles, 
   const int by_tiles = 2 * max_tiles / 5 + 3, by_tiles_long = (max_tiles + 3) / 4 + 3;
   if (s > by_tiles) {
     s = by_tiles;
-    const int64_t calm = 3 * simds / 4 / units;
-    if (s > calm) s = calm > by_tiles_long ? calm : (s < by_tiles_long ? s : by_tiles_long);
+    const int64_t calm = 3 * simds / 4 / units, six_per_cu = 3 * simds / 2 / units;
+    if (s > calm) s = calm > by_tiles_long ? calm : (s < six_per_cu ? s : six_per_cu);
   }
   if (per_sequence_counts && s < 12 && max_tiles >= 48) s = 12;
   if (s > 512) s = 512;

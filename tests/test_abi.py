@@ -123,14 +123,14 @@ def test_host_side_rejection_without_gpu(lib):
     assert ds(1, 8, 1025, 0) > ds(16, 8, 1025, 0)
     # long splits: two waves per SIMD of the device (256 compute units when there is none to ask); short
     # splits (under 8 tiles): 15/16 of that; body splits of 2.5 tiles at least, and then at most 3/4
-    # of a workgroup per SIMD if body splits of 4 tiles or fewer allow it; at least 12 for long
-    # sequences with their own lengths
+    # of a workgroup per SIMD if body splits of 4 tiles or fewer allow it, else at most six
+    # workgroups per compute unit; at least 12 for long sequences with their own lengths
     assert ds(16, 8, 257, 0) == 16
     assert ds(1, 8, 1025, 0) == 240
     assert ds(1, 8, 33, 0) == 2 * 33 // 5 + 3 == 16
     assert ds(1, 8, 129, 0) == 54
     assert ds(4, 8, 65, 0) == 768 // 32 == 24 and ds(2, 8, 129, 0) == 48
-    assert ds(8, 8, 65, 0) == 65 // 4 + 1 + 3 == 20
+    assert ds(8, 8, 65, 0) == 1536 // 64 == 24 and ds(2, 8, 257, 0) == 1536 // 16 == 96 and ds(1, 8, 513, 0) == 192
     assert ds(0, 8, 33, 0) == 1
     assert ds(64, 8, 131, 0) == 4 and ds(64, 8, 131, 1) == 12 and ds(64, 8, 40, 1) == 4
 
