@@ -377,13 +377,14 @@ struct TileAttend {
           }
       asm volatile("" ::: "memory");   // keep this a branch, not selects on every tile
     }
+    // this lane's maxima; a logit above the running maximum of its row (the logits are relative to
+    // it) shows in the lane that holds it, so the maxima over the four lane groups are only formed
+    // when some row's maximum really moves
     float mt_[kNT];
 #pragma unroll
     for (int nt = 0; nt < kNT; ++nt) {
       float mx = vmax3(vmax3(S[0][nt][0], S[0][nt][1], S[0][nt][2]), S[0][nt][3], S[1][nt][0]);
-      mx = vmax3(vmax3(mx, S[1][nt][1], S[1][nt][2]), S[1][nt][3], mx);
-      mx = max_over_lane_groups(mx);
-      mt_[nt] = mx;
+      mt_[nt] = vmax3(vmax3(mx, S[1][nt][1], S[1][nt][2]), S[1][nt][3], mx);
     }
     bool move = A.first;
 #pragma unroll
@@ -391,7 +392,8 @@ struct TileAttend {
     if (__any(move)) {
 #pragma unroll
       for (int nt = 0; nt < kNT; ++nt) {
-        const float dm = A.first ? mt_[nt] : fmaxf(mt_[nt], 0.f);
+        const float col = max_over_lane_groups(mt_[nt]);
+        const float dm = A.first ? col : fmaxf(col, 0.f);
 #pragma unroll
         for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
