@@ -656,11 +656,11 @@ def main():
         if stable >= 3:
             settle["settled"] = True
             break
-    for i in range(args.warmup):
+    events = [(hip.create(), hip.create()) for _ in range(args.steps)]   # before the warm-up: no host work (and no
+    for i in range(args.warmup):                                          # idle device) between it and the timed steps
         step(n_done + i)
     n_done += args.warmup
     torch.cuda.synchronize()
-    events = [(hip.create(), hip.create()) for _ in range(args.steps)]
     t0 = time.perf_counter()
     for i in range(args.steps):
         step(n_done + i, events[i])
