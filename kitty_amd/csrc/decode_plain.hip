@@ -174,20 +174,22 @@ __global__ __launch_bounds__(256) void decode_plain_kernel(kitty_kv_layer L, con
 }
 
 // out[b, 0, hq, :] = sum_s acc_s * 2^(m_s - m) / sum_s l_s * 2^(m_s - m); the running maxima of
-// the partials are in log2 units.  One block per (32 channels, query head, batch row).  The maximum
+// the partials are in log2 units.  One block per (CH channels, query head, batch row).  The maximum
 // over the splits is taken with one load per thread and a block reduction; then GROUPS groups of
-// 32 lanes stride over the splits, four loads in flight each, and combine through LDS in a fixed
-// order.  GROUPS = 8 up to 32 splits (2 when there are thousands of blocks), 32 beyond (a long
-// sequence at batch 1 has hundreds of splits).
-constexpr int kMergeChannels = 32;
-template <int GROUPS>
+// CH lanes stride over the splits, four loads in flight each, and combine through LDS in a fixed
+// order (the result depends on GROUPS, not on CH).  GROUPS = 8 up to 32 splits (2 for a large
+// batch), 32 beyond (a long sequence at batch 1 has hundreds of splits).  CH: blocks are handed
+// out at some 700 per microsecond, so a launch of thousands of one-wave blocks is bound by that
+// and not by its loads - all 128 channels of a head in one block where there are many heads.
+template <int GROUPS, int kMergeChannels>
 __global__ __launch_bounds__(GROUPS * kMergeChannels) void decode_merge_kernel(
     const float* __restrict__ ws_ml, const float* __restrict__ ws_acc, __half* __restrict__ out, int num_splits) {
+  static_assert(kD % kMergeChannels == 0 && (GROUPS * kMergeChannels) % 64 == 0, "whole waves, whole heads");
   constexpr int kThreads = GROUPS * kMergeChannels, kWaves = kThreads / 64;
   __shared__ float s_m[kWaves], s_l[GROUPS], s_o[GROUPS][kMergeChannels];
   const int64_t head = (int64_t)blockIdx.z * gridDim.y + blockIdx.y;
   const int64_t row0 = head * num_splits;
-  const int lane = threadIdx.x & (kMergeChannels - 1), grp = threadIdx.x / kMergeChannels;
+  const int lane = threadIdx.x % kMergeChannels, grp = threadIdx.x / kMergeChannels;
   const int d = blockIdx.x * kMergeChannels + lane;
   float m = -INFINITY;
   for (int s = threadIdx.x; s < num_splits; s += kThreads) m = fmaxf(m, ws_ml[(row0 + s) * 2]);
@@ -227,15 +229,18 @@ void launch_decode_plain(const kitty_kv_layer& L, const void* q, int B, int H_Q,
 
 void launch_decode_merge(const float* ws_ml, const float* ws_acc, void* out, int B, int H_Q, int num_splits,
                          hipStream_t stream) {
-  const dim3 grid(kD / kMergeChannels, H_Q, B);
-  if (num_splits <= 32 && (int64_t)grid.x * grid.y * grid.z >= 4096)   // large batch: one wave per block, all resident at once
-    hipLaunchKernelGGL(decode_merge_kernel<2>, grid, dim3(2 * kMergeChannels), 0, stream, ws_ml, ws_acc, (__half*)out,
-                       num_splits);
+  const int64_t heads = (int64_t)B * H_Q;
+  if (num_splits <= 32 && heads >= 1024)   // large batch
+    hipLaunchKernelGGL((decode_merge_kernel<2, kD>), dim3(1, H_Q, B), dim3(2 * kD), 0, stream, ws_ml, ws_acc,
+                       (__half*)out, num_splits);
+  else if (num_splits <= 32 && heads >= 256)
+    hipLaunchKernelGGL((decode_merge_kernel<8, 64>), dim3(kD / 64, H_Q, B), dim3(8 * 64), 0, stream, ws_ml, ws_acc,
+                       (__half*)out, num_splits);
   else if (num_splits <= 32)
-    hipLaunchKernelGGL(decode_merge_kernel<8>, grid, dim3(8 * kMergeChannels), 0, stream, ws_ml, ws_acc, (__half*)out,
-                       num_splits);
+    hipLaunchKernelGGL((decode_merge_kernel<8, 32>), dim3(kD / 32, H_Q, B), dim3(8 * 32), 0, stream, ws_ml, ws_acc,
+                       (__half*)out, num_splits);
   else
-    hipLaunchKernelGGL(decode_merge_kernel<32>, grid, dim3(32 * kMergeChannels), 0, stream, ws_ml, ws_acc,
+    hipLaunchKernelGGL((decode_merge_kernel<32, 32>), dim3(kD / 32, H_Q, B), dim3(32 * 32), 0, stream, ws_ml, ws_acc,
                        (__half*)out, num_splits);
 }
 
