@@ -174,49 +174,65 @@ __global__ __launch_bounds__(256) void decode_plain_kernel(kitty_kv_layer L, con
 }
 
 // out[b, 0, hq, :] = sum_s acc_s * 2^(m_s - m) / sum_s l_s * 2^(m_s - m); the running maxima of
-// the partials are in log2 units.  One block per (CH channels, query head, batch row).  The maximum
-// over the splits is taken with one load per thread and a block reduction; then GROUPS groups of
-// CH lanes stride over the splits, four loads in flight each, and combine through LDS in a fixed
-// order (the result depends on GROUPS, not on CH).  GROUPS = 8 up to 32 splits (2 for a large
-// batch), 32 beyond (a long sequence at batch 1 has hundreds of splits).  CH: blocks are handed
-// out at some 700 per microsecond, so a launch of thousands of one-wave blocks is bound by that
-// and not by its loads - all 128 channels of a head in one block where there are many heads.
-template <int GROUPS, int kMergeChannels>
+// the partials are in log2 units.  One block per (CH channels, query head, batch row).  GROUPS
+// groups of CH lanes stride over the splits; a thread asks for everything it will read - the
+// (max, sum) pairs and its channel of the accumulator rows of up to eight splits at a time, the
+// indices clamped instead of tested so that no load waits for a branch - and folds the splits into
+// one partial of its own as they arrive (the partials were written by other XCDs a moment ago and
+// come from memory: one round trip instead of the two that "first the maximum, then the sums"
+// costs).  The groups' partials are combined through LDS in a fixed order.  GROUPS = 8 up to 32
+// splits (2 for a large batch), 32 beyond (a long sequence at batch 1 has hundreds of splits).
+// CH: a launch of thousands of one-wave blocks is bound by the rate at which blocks are handed out,
+// not by its loads - all 128 channels of a head in one block where there are many heads.
+// kBatch: splits a thread asks for at a time (the launcher picks the smallest of 2, 4, 8 that covers a
+// group's share).
+template <int GROUPS, int kMergeChannels, int kBatch>
 __global__ __launch_bounds__(GROUPS * kMergeChannels) void decode_merge_kernel(
     const float* __restrict__ ws_ml, const float* __restrict__ ws_acc, __half* __restrict__ out, int num_splits) {
   static_assert(kD % kMergeChannels == 0 && (GROUPS * kMergeChannels) % 64 == 0, "whole waves, whole heads");
-  constexpr int kThreads = GROUPS * kMergeChannels, kWaves = kThreads / 64;
-  __shared__ float s_m[kWaves], s_l[GROUPS], s_o[GROUPS][kMergeChannels];
+  __shared__ float s_m[GROUPS], s_l[GROUPS], s_o[GROUPS][kMergeChannels];
   const int64_t head = (int64_t)blockIdx.z * gridDim.y + blockIdx.y;
   const int64_t row0 = head * num_splits;
   const int lane = threadIdx.x % kMergeChannels, grp = threadIdx.x / kMergeChannels;
   const int d = blockIdx.x * kMergeChannels + lane;
-  float m = -INFINITY;
-  for (int s = threadIdx.x; s < num_splits; s += kThreads) m = fmaxf(m, ws_ml[(row0 + s) * 2]);
+  float m = -INFINITY, l = 0.f, o = 0.f;
+  for (int s0 = grp; s0 < num_splits; s0 += GROUPS * kBatch) {
+    float ms[kBatch], ls[kBatch], as[kBatch];
 #pragma unroll
-  for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o));
-  if ((threadIdx.x & 63) == 0) s_m[threadIdx.x >> 6] = m;
-  __syncthreads();
+    for (int i = 0; i < kBatch; ++i) {
+      const int s = s0 + i * GROUPS;
+      const int64_t row = row0 + (s < num_splits ? s : s0);
+      ms[i] = ws_ml[row * 2];
+      ls[i] = ws_ml[row * 2 + 1];
+      as[i] = ws_acc[row * kD + d];
+      if (s >= num_splits) ms[i] = -INFINITY;
+    }
 #pragma unroll
-  for (int w = 0; w < kWaves; ++w) m = fmaxf(m, s_m[w]);
-  float l = 0.f, o = 0.f;
-#pragma unroll 4
-  for (int s = grp; s < num_splits; s += GROUPS) {
-    const float ms = ws_ml[(row0 + s) * 2];
-    const float ls = ws_ml[(row0 + s) * 2 + 1];
-    const float as = ws_acc[(row0 + s) * kD + d];
-    if (ms == -INFINITY) continue;   // an empty split: its accumulator row may never have been written
-    const float w = exp2f(ms - m);
-    l += ls * w;
-    o += as * w;
+    for (int i = 0; i < kBatch; ++i) {
+      // an empty split (max = -inf; its accumulator row may never have been written) changes nothing
+      const bool live = ms[i] != -INFINITY;
+      const float mn = live ? fmaxf(m, ms[i]) : m;
+      const float wa = live ? exp2f(m - mn) : 1.f;   // (m = -inf at first: 2^-inf = 0)
+      const float wb = live ? exp2f(ms[i] - mn) : 0.f;
+      l = l * wa + (live ? ls[i] : 0.f) * wb;
+      o = o * wa + (live ? as[i] : 0.f) * wb;
+      m = mn;
+    }
   }
-  if (lane == 0) s_l[grp] = l;
+  if (lane == 0) s_m[grp] = m, s_l[grp] = l;
   s_o[grp][lane] = o;
   __syncthreads();
   if (grp == 0) {
+    float mm = -INFINITY;
+#pragma unroll
+    for (int g = 0; g < GROUPS; ++g) mm = fmaxf(mm, s_m[g]);
     l = 0.f, o = 0.f;
 #pragma unroll
-    for (int g = 0; g < GROUPS; ++g) { l += s_l[g]; o += s_o[g][lane]; }
+    for (int g = 0; g < GROUPS; ++g) {
+      const float w = s_m[g] != -INFINITY ? exp2f(s_m[g] - mm) : 0.f;
+      l += s_l[g] * w;
+      o += s_o[g][lane] * w;
+    }
     out[head * kD + d] = __float2half_rn(l > 0.f ? o / l : 0.f);
   }
 }
@@ -227,21 +243,27 @@ void launch_decode_plain(const kitty_kv_layer& L, const void* q, int B, int H_Q,
                      H_Q, scaling, ws_ml, ws_acc, num_splits);
 }
 
+namespace {
+template <int GROUPS, int CH>
+void launch_merge(const float* ws_ml, const float* ws_acc, void* out, int B, int H_Q, int num_splits, hipStream_t stream) {
+  const dim3 grid(kD / CH, H_Q, B), block(GROUPS * CH);
+  const int share = (num_splits + GROUPS - 1) / GROUPS;
+  if (share <= 2)
+    hipLaunchKernelGGL((decode_merge_kernel<GROUPS, CH, 2>), grid, block, 0, stream, ws_ml, ws_acc, (__half*)out, num_splits);
+  else if (share <= 4)
+    hipLaunchKernelGGL((decode_merge_kernel<GROUPS, CH, 4>), grid, block, 0, stream, ws_ml, ws_acc, (__half*)out, num_splits);
+  else
+    hipLaunchKernelGGL((decode_merge_kernel<GROUPS, CH, 8>), grid, block, 0, stream, ws_ml, ws_acc, (__half*)out, num_splits);
+}
+}  // namespace
+
 void launch_decode_merge(const float* ws_ml, const float* ws_acc, void* out, int B, int H_Q, int num_splits,
                          hipStream_t stream) {
   const int64_t heads = (int64_t)B * H_Q;
-  if (num_splits <= 32 && heads >= 1024)   // large batch
-    hipLaunchKernelGGL((decode_merge_kernel<2, kD>), dim3(1, H_Q, B), dim3(2 * kD), 0, stream, ws_ml, ws_acc,
-                       (__half*)out, num_splits);
-  else if (num_splits <= 32 && heads >= 256)
-    hipLaunchKernelGGL((decode_merge_kernel<8, 64>), dim3(kD / 64, H_Q, B), dim3(8 * 64), 0, stream, ws_ml, ws_acc,
-                       (__half*)out, num_splits);
-  else if (num_splits <= 32)
-    hipLaunchKernelGGL((decode_merge_kernel<8, 32>), dim3(kD / 32, H_Q, B), dim3(8 * 32), 0, stream, ws_ml, ws_acc,
-                       (__half*)out, num_splits);
-  else
-    hipLaunchKernelGGL((decode_merge_kernel<32, 32>), dim3(kD / 32, H_Q, B), dim3(32 * 32), 0, stream, ws_ml, ws_acc,
-                       (__half*)out, num_splits);
+  if (num_splits <= 32 && heads >= 1024) launch_merge<2, kD>(ws_ml, ws_acc, out, B, H_Q, num_splits, stream);   // large batch
+  else if (num_splits <= 32 && heads >= 256) launch_merge<8, 64>(ws_ml, ws_acc, out, B, H_Q, num_splits, stream);
+  else if (num_splits <= 32) launch_merge<8, 32>(ws_ml, ws_acc, out, B, H_Q, num_splits, stream);
+  else launch_merge<32, 32>(ws_ml, ws_acc, out, B, H_Q, num_splits, stream);
 }
 
 }  // namespace kitty
