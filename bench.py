@@ -63,6 +63,7 @@ class HipEvents:
         self.hip = ctypes.CDLL("libamdhip64.so")
         self.hip.hipEventCreate.argtypes = [ctypes.POINTER(ctypes.c_void_p)]
         self.hip.hipEventElapsedTime.argtypes = [ctypes.POINTER(ctypes.c_float), ctypes.c_void_p, ctypes.c_void_p]
+        self.hip.hipEventSynchronize.argtypes = [ctypes.c_void_p]
 
     def create(self):
         ev = self.ct.c_void_p()
@@ -70,6 +71,11 @@ class HipEvents:
         if rc != 0:
             raise RuntimeError(f"hipEventCreate failed ({rc})")
         return ev
+
+    def synchronize(self, ev) -> None:
+        rc = self.hip.hipEventSynchronize(ev)
+        if rc != 0:
+            raise RuntimeError(f"hipEventSynchronize failed ({rc})")
 
     def elapsed_us(self, a, b) -> float:
         ms = self.ct.c_float()
@@ -141,6 +147,10 @@ def cpu_baseline(K, V, q, H_Q, H_KV):
 
 
 def bench_chunked_prefill(args):
+    print(json.dumps(chunked_prefill_result(args)))
+
+
+def chunked_prefill_result(args):
     """configs[3]: a step = chunked-prefill attention of one layer; the append is timed beside it."""
     import torch
     import kitty_amd
@@ -215,7 +225,7 @@ def bench_chunked_prefill(args):
         result["cpu_baseline"] = {"value": dt * B * H_KV * 1e3, "unit": "ms/step", "cores": torch.get_num_threads(),
                                   "kind": "port", "sample": f"dense fp32 causal attention of 1 of {B * H_KV} "
                                   f"(sequence, KV head) units, {dt:.2f} s, scaled x{B * H_KV}"}
-    print(json.dumps(result))
+    return result
 
 
 def bench_fake_quant(args):
@@ -288,6 +298,10 @@ def bench_fake_quant(args):
 
 
 def bench_generate(args):
+    print(json.dumps(generate_result(args)))
+
+
+def generate_result(args):
     """End-to-end as the reference measures it (latency_benchmarking/benchmark_kitty.py:127-197): a stock
     transformers model - random-init Llama-3.1-8B or Qwen3-8B shapes from a local config, nothing is
     downloaded - with ``attn_implementation="kitty"`` and a fresh ``KittyHFCache`` per run, ``generate()``
@@ -338,7 +352,7 @@ def bench_generate(args):
     assert tuple(out.shape) == (B, max_len) and cache.get_seq_length(0) == max_len - 1
     cache.check_status()
     new = max_len - T0
-    print(json.dumps({
+    return {
         "metric": "end_to_end_generate_tokens_per_s", "value": B * new / dt, "unit": "tokens/s", "n_gpus": 1,
         "steps": args.e2e_repeat_runs, "warmup": args.e2e_warmup_runs, "ms_per_step": dt * 1e3 / new,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16 model, 2/4-bit packed KV",
@@ -350,7 +364,7 @@ def bench_generate(args):
         "generate_s_per_run": dt, "new_tokens_per_sequence": new,
         "note": "one step = one decode iteration of generate(); the host-side launch sequence of the stock model's "
                 "dense layers is inside the timed region, as in the reference's benchmark",
-    }))
+    }
 
 
 def bench_end_to_end(args):
@@ -505,6 +519,269 @@ def bench_decode_loop(args):
     }))
 
 
+def lib_check():
+    import torch
+    from kitty_amd import _lib
+    _lib.lib()                           # raises when the HIP library is not built: no fallback
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+
+
+class DecodeBench:
+    """One decode workload resident in HBM: the packed caches (made by the quantizer under test, enough
+    independent copies to rotate over more than 3x the Infinity Cache), q, the workspace, and the
+    byte counts a step has to move."""
+
+    def __init__(self, workload, variant, args):
+        import torch
+        import kitty_amd
+        from kitty_amd import _lib
+        self.lib, self._lib, self.torch = _lib.lib(), _lib, torch
+        dev = self.dev = torch.device("cuda:0")
+        self.workload, self.variant = workload, variant
+        B, H_Q, H_KV, T, self.desc = WORKLOADS[workload]
+        self.B, self.H_Q, self.H_KV, self.T = B, H_Q, H_KV, T
+        D = self.D = 128
+        cfg = types.SimpleNamespace(num_hidden_layers=1, head_dim=D, num_key_value_heads=H_KV,
+                                    num_attention_heads=H_Q, hidden_size=H_Q * D)
+        max_len = T + 256
+        K, V = self.K, self.V = synth_kv(B, H_KV, T, D, 1000 + int(workload[1]), dev)
+        probe = kitty_amd.KittyCache(cfg, B, max_len, device=dev)
+        probe.update(K, V, 0)
+        probe.quantize_prefill(0)
+        seq_counts = None
+        if workload == "c2":
+            import numpy as np
+            rng = np.random.default_rng(1002)
+            rows = []
+            for _ in range(B):
+                Ti, Ri = int(rng.integers(1024, 16385)), int(rng.integers(0, 128))
+                pk = (Ti - 32 - Ri) // 128
+                rows.append([32, pk, Ri, pk - 1, Ri, 128, int(rng.integers(0, 128)), 0])
+            seq_counts = torch.tensor(rows, dtype=torch.int32, device=dev)
+            self.total_bytes = sum(H_KV * (5760 * r[1] + 4608 * r[3] + 256 * (2 * r[0] + r[2] + r[4] + r[5]))
+                                   + 2 * H_Q * 128 * 2 for r in rows)
+            self.packed_bytes = sum(H_KV * (5760 * r[1] + 4608 * r[3]) for r in rows)
+        else:
+            self.total_bytes, self.packed_bytes = algorithmic_bytes(B, H_Q, H_KV, probe.kv_cache[0])
+        copies = args.copies or max(2, -(-3 * 256 * 2 ** 20 // self.total_bytes))      # > 3x the Infinity Cache
+        copies = min(copies, 256)
+        caches = [probe]
+        quant_ms = []
+        for i in range(1, copies + 2):       # the extra rounds only time the quantizer
+            c = caches[i] if i < len(caches) else kitty_amd.KittyCache(cfg, B, max_len, device=dev)
+            c.update(K, V, 0)
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            c.quantize_prefill(0)
+            e1.record()
+            torch.cuda.synchronize()
+            quant_ms.append(e0.elapsed_time(e1))
+            if i < copies:
+                caches.append(c)
+        if args.scatter_pages:
+            gen = torch.Generator(device=dev).manual_seed(5)
+            for c in caches:
+                L = c.kv_cache[0]
+                for codes, meta, table in ((L.KeyCache, L.KeyCache_metadata, L.PageTable_K),
+                                           (L.ValueCache, L.ValueCache_metadata, L.PageTable_V)):
+                    perm = torch.randperm(codes.shape[0], generator=gen, device=dev)
+                    for t in (codes, meta):
+                        moved = torch.empty_like(t)
+                        moved[perm] = t
+                        t.copy_(moved)
+                    table.copy_(perm[table])
+            del moved
+        self.caches = caches
+        L0 = self.L0 = probe.kv_cache[0]
+        self.quant_ms = min(quant_ms)
+        self.quant_in_bytes = 2 * B * H_KV * (L0.PageCount_K + L0.PageCount_V) * 128 * D
+        self.q = torch.randn((B, H_Q, 1, D), generator=torch.Generator(device=dev).manual_seed(7), device=dev,
+                             dtype=torch.float32).half()
+        self.out = torch.empty((B, 1, H_Q, D), dtype=torch.float16, device=dev)
+        max_tiles = (2 + L0.MAX_PAGE) if seq_counts is not None else 1 + (T - L0.Sink_Count + 127) // 128
+        self.splits = args.splits or self.lib.kitty_decode_attn_default_splits(B, H_KV, max_tiles,
+                                                                               int(seq_counts is not None))
+        self.ws_bytes = self.lib.kitty_decode_attn_workspace_bytes(B, H_Q, D, self.splits)
+        self.ws = torch.empty(self.ws_bytes, dtype=torch.uint8, device=dev)
+        if seq_counts is not None:
+            for c in caches:
+                c.kv_cache[0].seq_counts = seq_counts
+        self.descs = [c.kv_cache[0].descriptor() for c in caches]
+        self.stream = torch.cuda.current_stream(dev).cuda_stream
+        self.scaling = D ** -0.5
+        self.hip = HipEvents()
+
+    def step(self, i, ev=None, variant=None):
+        lib, _lib = self.lib, self._lib
+        d = self.descs[i % len(self.descs)]
+        if ev is not None:     # the events ride on the split kernel's own dispatch: its duration on the device
+            _lib.check(lib.kitty_profile_next_split(ev[0], ev[1]), "profile")
+        rc = lib.kitty_decode_attn_split(d, self.q.data_ptr(), self.B, self.H_Q, self.scaling, self.ws.data_ptr(),
+                                         self.ws_bytes, self.splits, self.variant if variant is None else variant,
+                                         self.stream)
+        _lib.check(rc, "split")
+        _lib.check(lib.kitty_decode_attn_merge(self.ws.data_ptr(), self.ws_bytes, self.B, self.H_Q, self.D, self.splits,
+                                               self.out.data_ptr(), self.stream), "merge")
+
+    def settle(self, variant=None, max_windows=150):
+        """Untimed launches until the kernel's duration has reached its SUSTAINED level.  After idle the
+        clocks first rise (the first ~100 launches run 5-8 % slower) and then, under a load that keeps
+        the package at its power limit, come down again over some thousand launches to the level they
+        hold for good; a window that is separated from the next by a host synchronisation reads the
+        level in between.  So the windows run back to back, 100 launches each with the events on every
+        fifth launch, and the run counts as settled once the median of a window stays within 1 % of
+        the previous one for three windows in a row after at least 10 windows (1000 launches)."""
+        hip = self.hip
+        n_win, every = 100, 5
+        sets = [[(hip.create(), hip.create()) for _ in range(n_win // every)] for _ in range(2)]
+        settle = {"windows": 0, "launches": 0, "median_us": None, "settled": False, "window_medians_us": []}
+        prev, stable, pending = None, 0, None
+        for w in range(max_windows):
+            cur = sets[w % 2]
+            for j in range(n_win):
+                self.step(self.n_done, cur[j // every] if j % every == 0 else None, variant)
+                self.n_done += 1
+            if pending is not None:   # read window w - 1 while window w runs: the device is never idle in between
+                hip.synchronize(pending[-1][1])
+                med = sorted(hip.elapsed_us(a, b) for a, b in pending)[len(pending) // 2]
+                settle["window_medians_us"].append(round(med, 2))
+                stable = stable + 1 if prev is not None and abs(med - prev) <= 0.01 * prev else 0
+                prev = med
+                settle.update(windows=w, launches=w * n_win, median_us=med)
+                if stable >= 3 and w >= 10:
+                    settle["settled"] = True
+                    break
+            pending = cur
+        return settle
+
+    def timed(self, steps, warmup, variant=None):
+        """`steps` steps as a caller runs them (wall clock, synchronised on both sides), then the same
+        steps once more with events on the split kernel's dispatch."""
+        torch, hip = self.torch, self.hip
+        events = [(hip.create(), hip.create()) for _ in range(steps)]   # before the warm-up: no host work (and no
+        for i in range(warmup):                                          # idle device) between it and the timed steps
+            self.step(self.n_done + i, None, variant)
+        self.n_done += warmup
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(steps):
+            self.step(self.n_done + i, None, variant)
+        torch.cuda.synchronize()
+        us_per_step = (time.perf_counter() - t0) / steps * 1e6
+        t0 = time.perf_counter()
+        for i in range(steps):
+            self.step(self.n_done + i, events[i], variant)
+        torch.cuda.synchronize()
+        us_per_step_events = (time.perf_counter() - t0) / steps * 1e6
+        self.n_done += 2 * steps
+        kern_us = sorted(hip.elapsed_us(a, b) for a, b in events)
+        return us_per_step, us_per_step_events, kern_us
+
+    n_done = 0
+
+    def summary(self, steps, warmup, variant=None, max_windows=30):
+        """The fields of the headline for a side workload: settled briefly, then timed."""
+        settle = self.settle(variant, max_windows=max_windows)
+        us_per_step, _, kern_us = self.timed(steps, warmup, variant)
+        avg = sum(kern_us) / len(kern_us)
+        gbps = self.total_bytes / (avg * 1e-6) / 1e9
+        return {"workload": self.desc, "variant": self.variant if variant is None else variant,
+                "num_splits": self.splits, "value": us_per_step, "unit": "us/step", "steps": steps,
+                "kernel": "decode split pass" + (" (work-list kernel + split kernel)" if self.workload == "c2" else ""),
+                "kernel_avg_us": avg, "kernel_median_us": kern_us[len(kern_us) // 2],
+                "algorithmic_bytes_per_launch": self.total_bytes, "packed_bytes_per_launch": self.packed_bytes,
+                "achieved_gbps": gbps, "frac": gbps / HBM_PEAK_GBPS,
+                "packed_frac": self.packed_bytes / (avg * 1e-6) / 1e9 / HBM_PEAK_GBPS,
+                "settled_after_launches": settle["launches"], "settled": settle["settled"]}
+
+    def headline(self, args):
+        torch, hip = self.torch, self.hip
+        settle = self.settle()
+        us_per_step, us_per_step_events, kern_us = self.timed(args.steps, args.warmup)
+        kern_avg_us = sum(kern_us) / len(kern_us)
+        achieved = self.total_bytes / (kern_avg_us * 1e-6) / 1e9
+        # cache-hot figure (same copy every step), reported separately
+        win = [(hip.create(), hip.create()) for _ in range(20)]
+        for i in range(20):
+            self.step(0, win[i])
+        torch.cuda.synchronize()
+        hot_us = sorted(hip.elapsed_us(a, b) for a, b in win)[len(win) // 2]
+        if args.copy_calibration:
+            src = torch.empty(1 << 30, dtype=torch.uint8, device=self.dev).fill_(3)
+            dst = torch.empty_like(src)
+            for _ in range(5):
+                dst.copy_(src)
+            torch.cuda.synchronize()
+        L0 = self.L0
+        return {
+            "metric": "packed_kv_decode_attention_us_per_step",
+            "value": us_per_step,
+            "unit": "us/step",
+            "n_gpus": 1,
+            "steps": args.steps,
+            "warmup": args.warmup,
+            "ms_per_step": us_per_step * 1e-3,
+            "higher_is_better": False,
+            "scaling": "weak",
+            "vs_baseline": None,
+            "dtype": "u8 codes + f16 scales/zeros, f32 accumulate",
+            "data": "synthetic (seeded N(0,1) K with 8 outlier channels/head x10, N(0,1) V, random-init)",
+            "config": {"workload": self.desc, "batch": self.B, "q_heads": self.H_Q, "kv_heads": self.H_KV,
+                       "head_dim": self.D, "context": self.T, "pages_k": L0.PageCount_K, "pages_v": L0.PageCount_V,
+                       "num_splits": self.splits, "variant": self.variant, "cache_copies_rotated": len(self.caches),
+                       "page_placement": "scattered" if args.scatter_pages else "identity"},
+            "roofline": {
+                "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                "frac": achieved / HBM_PEAK_GBPS, "traffic": measured_traffic(self.workload, self.splits),
+                "kernel": "decode split pass", "kernel_avg_us": kern_avg_us,
+                "kernel_median_us": kern_us[len(kern_us) // 2],
+                "algorithmic_bytes_per_launch": self.total_bytes, "packed_bytes_per_launch": self.packed_bytes,
+                "packed_gbps": self.packed_bytes / (kern_avg_us * 1e-6) / 1e9,
+                "packed_frac": self.packed_bytes / (kern_avg_us * 1e-6) / 1e9 / HBM_PEAK_GBPS,
+                "cache_hot_kernel_us": hot_us,
+                "timing": "HIP events attached to the split kernel's dispatch on the launch stream (kernel begin to "
+                          "end), averaged over the timed steps run a second time with the events attached (their "
+                          "marker packets cost a step about 5 us, so `value` is timed without them)",
+                "us_per_step_with_events": us_per_step_events,
+                "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE summary committed under profiles/ (a run "
+                                  "of its own, calibrated by a 1 GiB copy), not measured in this run",
+                "clock_settling": settle,
+            },
+            "quantizer": {"gbps_in": self.quant_in_bytes / (self.quant_ms * 1e-3) / 1e9, "ms": self.quant_ms,
+                          "input_bytes": self.quant_in_bytes,
+                          "what": "quantize_prefill of the whole context (K select+quantize+pack, V quantize+pack)"},
+        }
+
+
+def other_workloads(headline, args):
+    """The other BASELINE configs and the plain kernel, measured in this process after the headline so
+    that one run of the default command holds a figure for each: same fields as the headline's
+    roofline, fewer steps.  A workload that fails leaves its error text instead of stopping the run."""
+    import gc
+    import torch
+    out = {}
+
+    def guarded(name, fn):
+        try:
+            out[name] = fn()
+        except Exception as e:                       # noqa: BLE001 - the headline must survive a side workload
+            out[name] = {"error": f"{type(e).__name__}: {e}"[:300]}
+        gc.collect()
+        torch.cuda.empty_cache()
+
+    side = types.SimpleNamespace(copies=0, splits=0, scatter_pages=False)
+    guarded("c1_variant1", lambda: headline.summary(10, 3, variant=1, max_windows=4))
+    for name in ("c0", "c2", "c4"):
+        guarded(name, lambda name=name: DecodeBench(name, 0, side).summary(40, 5))
+    c3_args = types.SimpleNamespace(steps=5, warmup=2, no_cpu_baseline=True)
+    guarded("c3", lambda: chunked_prefill_result(c3_args))
+    e2e = types.SimpleNamespace(e2e_batch=16, e2e_prompt=64, e2e_max_len=192, e2e_model="llama", e2e_warmup_runs=1,
+                                e2e_repeat_runs=1)
+    guarded("e2e_generate", lambda: generate_result(e2e))
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -529,6 +806,9 @@ def main():
     ap.add_argument("--splits", type=int, default=0)
     ap.add_argument("--variant", type=int, default=0)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-other-workloads", action="store_true",
+                    help="default workload only: leave out the `workloads` key (configs[0], [2], [3], [4], the plain "
+                         "kernel on configs[1] and a short generate() run, each measured after the headline)")
     ap.add_argument("--scatter-pages", action="store_true",
                     help="place every packed page at a random position of the page arrays (page tables to match), "
                          "as a page pool leaves them after sequences have come and gone; default: the reference's "
@@ -548,189 +828,14 @@ def main():
         return bench_end_to_end(args)
     if args.workload == "fq":
         return bench_fake_quant(args)
-    import torch
-    import kitty_amd
-    from kitty_amd import _lib
-    lib = _lib.lib()                     # raises when the HIP library is not built: no fallback
-    assert torch.cuda.is_available(), "bench.py needs a GPU"
-    dev = torch.device("cuda:0")
-    B, H_Q, H_KV, T, desc = WORKLOADS[args.workload]
-    D = 128
-    cfg = types.SimpleNamespace(num_hidden_layers=1, head_dim=D, num_key_value_heads=H_KV,
-                                num_attention_heads=H_Q, hidden_size=H_Q * D)
-    max_len = T + 256
-
-    # ---- build the packed caches with the quantizer under test ---------------------------------
-    K, V = synth_kv(B, H_KV, T, D, 1000 + int(args.workload[1]), dev)
-    probe = kitty_amd.KittyCache(cfg, B, max_len, device=dev)
-    probe.update(K, V, 0)
-    probe.quantize_prefill(0)
-    seq_counts = None
-    if args.workload == "c2":
-        import numpy as np
-        rng = np.random.default_rng(1002)
-        rows = []
-        for _ in range(B):
-            Ti, Ri = int(rng.integers(1024, 16385)), int(rng.integers(0, 128))
-            pk = (Ti - 32 - Ri) // 128
-            rows.append([32, pk, Ri, pk - 1, Ri, 128, int(rng.integers(0, 128)), 0])
-        seq_counts = torch.tensor(rows, dtype=torch.int32, device=dev)
-        total_bytes = sum(H_KV * (5760 * r[1] + 4608 * r[3] + 256 * (2 * r[0] + r[2] + r[4] + r[5])) + 2 * H_Q * 128 * 2
-                          for r in rows)
-        packed_bytes = sum(H_KV * (5760 * r[1] + 4608 * r[3]) for r in rows)
-    else:
-        total_bytes, packed_bytes = algorithmic_bytes(B, H_Q, H_KV, probe.kv_cache[0])
-    copies = args.copies or max(2, -(-3 * 256 * 2 ** 20 // total_bytes))      # > 3x the Infinity Cache
-    caches = [probe]
-    quant_ms = []
-    for i in range(1, copies + 2):       # the extra rounds only time the quantizer
-        c = caches[i] if i < len(caches) else kitty_amd.KittyCache(cfg, B, max_len, device=dev)
-        c.update(K, V, 0)
-        torch.cuda.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        c.quantize_prefill(0)
-        e1.record()
-        torch.cuda.synchronize()
-        quant_ms.append(e0.elapsed_time(e1))
-        if i < copies:
-            caches.append(c)
-    if args.scatter_pages:
-        gen = torch.Generator(device=dev).manual_seed(5)
-        for c in caches:
-            L = c.kv_cache[0]
-            for codes, meta, table in ((L.KeyCache, L.KeyCache_metadata, L.PageTable_K),
-                                       (L.ValueCache, L.ValueCache_metadata, L.PageTable_V)):
-                perm = torch.randperm(codes.shape[0], generator=gen, device=dev)
-                for t in (codes, meta):
-                    moved = torch.empty_like(t)
-                    moved[perm] = t
-                    t.copy_(moved)
-                table.copy_(perm[table])
-        del moved
-    L0 = probe.kv_cache[0]
-    quant_in_bytes = 2 * B * H_KV * (L0.PageCount_K + L0.PageCount_V) * 128 * D
-    quant_gbps = quant_in_bytes / (min(quant_ms) * 1e-3) / 1e9
-
-    q = torch.randn((B, H_Q, 1, D), generator=torch.Generator(device=dev).manual_seed(7), device=dev,
-                    dtype=torch.float32).half()
-    out = torch.empty((B, 1, H_Q, D), dtype=torch.float16, device=dev)
-    max_tiles = (2 + L0.MAX_PAGE) if seq_counts is not None else 1 + (T - L0.Sink_Count + 127) // 128
-    splits = args.splits or lib.kitty_decode_attn_default_splits(B, H_KV, max_tiles, int(seq_counts is not None))
-    ws_bytes = lib.kitty_decode_attn_workspace_bytes(B, H_Q, D, splits)
-    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
-    if seq_counts is not None:
-        for c in caches:
-            c.kv_cache[0].seq_counts = seq_counts
-    descs = [c.kv_cache[0].descriptor() for c in caches]
-    stream = torch.cuda.current_stream(dev).cuda_stream
-    scaling = D ** -0.5
-
-    hip = HipEvents()
-
-    def step(i, ev=None):
-        d = descs[i % len(descs)]
-        if ev is not None:     # the events ride on the split kernel's own dispatch: its duration on the device
-            _lib.check(lib.kitty_profile_next_split(ev[0], ev[1]), "profile")
-        rc = lib.kitty_decode_attn_split(d, q.data_ptr(), B, H_Q, scaling, ws.data_ptr(), ws_bytes, splits,
-                                         args.variant, stream)
-        _lib.check(rc, "split")
-        _lib.check(lib.kitty_decode_attn_merge(ws.data_ptr(), ws_bytes, B, H_Q, D, splits, out.data_ptr(), stream),
-                   "merge")
-
-    # Untimed, whatever --warmup says: after idle the clocks need some hundred launches to settle, and a
-    # short run would time the ramp.  Windows of 20 launches until the median kernel duration moves by
-    # less than 1 % three windows in a row (at most 150 windows).
-    n_done, settle = 0, {"windows": 0, "median_us": None, "settled": False}
-    win = [(hip.create(), hip.create()) for _ in range(20)]
-    prev, stable = None, 0
-    for w in range(150):
-        for e in win:
-            step(n_done, e)
-            n_done += 1
-        torch.cuda.synchronize()
-        med = sorted(hip.elapsed_us(a, b) for a, b in win)[len(win) // 2]
-        stable = stable + 1 if prev is not None and abs(med - prev) <= 0.01 * prev else 0
-        prev = med
-        settle.update(windows=w + 1, median_us=med)
-        if stable >= 3:
-            settle["settled"] = True
-            break
-    events = [(hip.create(), hip.create()) for _ in range(args.steps)]   # before the warm-up: no host work (and no
-    for i in range(args.warmup):                                          # idle device) between it and the timed steps
-        step(n_done + i)
-    n_done += args.warmup
-    # The timed region: K steps as a caller runs them.  Then the same K steps once more with events
-    # attached to the split kernel's dispatch, for the kernel's own duration: the two marker packets
-    # per step that the events put into the queue cost the step about 5 us (70 -> 75 us), which is
-    # the measurement's and not the path's, so they stay out of `value`.
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for i in range(args.steps):
-        step(n_done + i)
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
-    ms_per_step = wall / args.steps * 1e3
-    t0 = time.perf_counter()
-    for i in range(args.steps):
-        step(n_done + i, events[i])
-    torch.cuda.synchronize()
-    ms_per_step_events = (time.perf_counter() - t0) / args.steps * 1e3
-    kern_us = sorted(hip.elapsed_us(a, b) for a, b in events)
-    kern_avg_us = sum(kern_us) / len(kern_us)
-    achieved = total_bytes / (kern_avg_us * 1e-6) / 1e9
-
-    # cache-hot figure (same copy every step), reported separately
-    for i in range(20):
-        step(0, win[i])
-    torch.cuda.synchronize()
-    hot_us = sorted(hip.elapsed_us(a, b) for a, b in win)[len(win) // 2]
-
-    if args.copy_calibration:
-        src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).fill_(3)
-        dst = torch.empty_like(src)
-        for _ in range(5):
-            dst.copy_(src)
-        torch.cuda.synchronize()
-
-    result = {
-        "metric": "packed_kv_decode_attention_us_per_step",
-        "value": ms_per_step * 1e3,
-        "unit": "us/step",
-        "n_gpus": 1,
-        "steps": args.steps,
-        "warmup": args.warmup,
-        "ms_per_step": ms_per_step,
-        "higher_is_better": False,
-        "scaling": "weak",
-        "vs_baseline": None,
-        "dtype": "u8 codes + f16 scales/zeros, f32 accumulate",
-        "data": "synthetic (seeded N(0,1) K with 8 outlier channels/head x10, N(0,1) V, random-init)",
-        "config": {"workload": desc, "batch": B, "q_heads": H_Q, "kv_heads": H_KV, "head_dim": D, "context": T,
-                   "pages_k": L0.PageCount_K, "pages_v": L0.PageCount_V, "num_splits": splits,
-                   "variant": args.variant, "cache_copies_rotated": len(caches),
-                   "page_placement": "scattered" if args.scatter_pages else "identity"},
-        "roofline": {
-            "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-            "frac": achieved / HBM_PEAK_GBPS, "traffic": measured_traffic(args.workload, splits),
-            "kernel": "decode split pass", "kernel_avg_us": kern_avg_us, "kernel_median_us": kern_us[len(kern_us) // 2],
-            "algorithmic_bytes_per_launch": total_bytes, "packed_bytes_per_launch": packed_bytes,
-            "packed_gbps": packed_bytes / (kern_avg_us * 1e-6) / 1e9,
-            "packed_frac": packed_bytes / (kern_avg_us * 1e-6) / 1e9 / HBM_PEAK_GBPS,
-            "cache_hot_kernel_us": hot_us,
-            "timing": "HIP events attached to the split kernel's dispatch on the launch stream (kernel begin to end), "
-                      "averaged over the timed steps run a second time with the events attached (their marker "
-                      "packets cost a step about 5 us, so `value` is timed without them)",
-            "us_per_step_with_events": ms_per_step_events * 1e3,
-            "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE summary committed under profiles/ (a run of "
-                              "its own, calibrated by a 1 GiB copy), not measured in this run",
-            "clock_settling": settle,
-        },
-        "quantizer": {"gbps_in": quant_gbps, "ms": min(quant_ms), "input_bytes": quant_in_bytes,
-                      "what": "quantize_prefill of the whole context (K select+quantize+pack, V quantize+pack)"},
-    }
+    lib_check()
+    headline = DecodeBench(args.workload, args.variant, args)
+    result = headline.headline(args)
     if not args.no_cpu_baseline:
-        result["cpu_baseline"] = cpu_baseline(K.cpu(), V.cpu(), q.cpu(), H_Q, H_KV)
+        result["cpu_baseline"] = cpu_baseline(headline.K.cpu(), headline.V.cpu(), headline.q.cpu(), headline.H_Q,
+                                              headline.H_KV)
+    if args.workload == "c1" and not args.no_other_workloads:
+        result["workloads"] = other_workloads(headline, args)
     print(json.dumps(result))
 
 

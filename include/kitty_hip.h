@@ -2,8 +2,10 @@
  * kitty_hip.h - C ABI of the MI355X (gfx950) implementation of Kitty's quantized-KV hot path.
  *
  * Every entry point is asynchronous and ordered on the HIP stream passed in (NULL = the default
- * stream), allocates nothing, frees nothing and keeps no state between calls except a thread-local
- * error string (kitty_decode_attn_static also remembers where its array lies on each device).  All data pointers are device pointers owned by the caller.  Return value: 0 on
+ * stream), allocates nothing and frees nothing.  State kept between calls: a thread-local error
+ * string, the thread-local events of kitty_profile_next_split, the device's SIMD count (asked once)
+ * and, for kitty_decode_attn_static, the address of its array on each device.  All data pointers
+ * are device pointers owned by the caller.  Return value: 0 on
  * success, a negative KITTY_E_* code when an argument is rejected on the host before anything is
  * launched, a positive hipError_t when a launch fails.  kitty_last_error() describes the last
  * failure on the calling thread.
@@ -187,7 +189,10 @@ int kitty_decode_attn_merge(const void* workspace, size_t workspace_bytes, int B
  * kernel's own dispatch, so that hipEventElapsedTime between them is the kernel's duration on the
  * device - the figure a kernel trace reports - without the host's enqueue gaps that an event pair
  * recorded around the call includes.  The events must have timing enabled and outlive the launch.
- * (NULL, NULL) cancels.  The plain variant records the events around its launch instead.
+ * (NULL, NULL) cancels.  The plain variant records the events around its launch instead.  The pair
+ * belongs to the next kitty_decode_attn_split call of the thread whether that call launches or is
+ * rejected: a rejected call disarms it too.  Measurement plumbing only: a caller that never calls
+ * this can ignore it.
  */
 int kitty_profile_next_split(void* start_event, void* stop_event);
 
@@ -202,6 +207,9 @@ int kitty_profile_next_split(void* start_event, void* stop_event);
  * KITTY_E_WORKSPACE.  The device that owns the tensors must be the current device.  All calls on one
  * device share the array: calls that overlap there (different streams or threads) race; calls
  * ordered on one stream do not, and nothing in the array needs clearing between them.
+ * The first call on a device looks the array's address up in the runtime (hipGetSymbolAddress, under
+ * a mutex): make it before capturing a stream, not inside the capture - a first call on a capturing
+ * stream is rejected with KITTY_E_RANGE.  Later calls only read the cached address.
  */
 #define KITTY_STATIC_WORKSPACE_BYTES (16u << 20)
 int kitty_decode_attn_static(const kitty_kv_layer* layer, const void* q, int B, int H_Q, float scaling,

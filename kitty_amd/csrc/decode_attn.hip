@@ -143,9 +143,22 @@ int check_workspace(const void* workspace, size_t workspace_bytes, int B, int H_
 
 }  // namespace
 
+namespace kitty {
+// check_layer for other translation units: the argument checks of every attention entry point, and
+// the tile count (1 + the 128-token tiles after the sink of the longest sequence) the default split
+// rule is evaluated on.
+int decode_check_layer(const kitty_kv_layer* layer, const void* q, int B, int H_Q, int* max_tiles) {
+  return check_layer(layer, q, B, H_Q, max_tiles);
+}
+}  // namespace kitty
+
 extern "C" int kitty_decode_attn_split(const kitty_kv_layer* layer, const void* q, int B, int H_Q, float scaling,
                                        void* workspace, size_t workspace_bytes, int num_splits, int variant,
                                        void* stream) {
+  // armed events belong to THIS call, whether it launches or is rejected: taken and disarmed before
+  // anything can return, so that they never ride on a later, unrelated launch of this thread
+  const hipEvent_t ev0 = g_ev_start, ev1 = g_ev_stop;
+  g_ev_start = g_ev_stop = nullptr;
   int max_tiles = 0;
   if (int rc = check_layer(layer, q, B, H_Q, &max_tiles)) return rc;
   if (int rc = check_workspace(workspace, workspace_bytes, B, H_Q, num_splits)) return rc;
@@ -153,8 +166,6 @@ extern "C" int kitty_decode_attn_split(const kitty_kv_layer* layer, const void* 
   const kitty_kv_layer& L = *layer;
   float* ws_ml = (float*)workspace;
   float* ws_acc = (float*)((uint8_t*)workspace + ws_ml_bytes(B, H_Q, num_splits));
-  const hipEvent_t ev0 = g_ev_start, ev1 = g_ev_stop;
-  g_ev_start = g_ev_stop = nullptr;
   if (variant == 0 && decode_mfma_supported(L, H_Q)) {
     uint32_t* ws_plan = (uint32_t*)((uint8_t*)ws_acc + ws_acc_bytes(B, H_Q, num_splits));
     launch_decode_mfma(L, q, B, H_Q, scaling, ws_ml, ws_acc, ws_plan, num_splits, device_simds(), (hipStream_t)stream,

@@ -282,10 +282,36 @@ __device__ __forceinline__ void k_load_regs(const Ctx& x, int page_index, KRegs&
   kb.meta = *(const uint2*)(meta + x.lane * 8);                          // [s0|z0], [s1|z1]
 }
 
-// Global -> LDS loads of one K page-head (no registers involved): scalar base + per-lane offset,
-// the LDS destination is M0 + instruction offset + lane * size.  8 instructions with the high
-// plane, 6 without.  Every tile is read exactly once, so the loads are marked non-temporal (2 % on the
-// whole launch; a read-only stream runs at 6.5 TB/s with the hint and 5.9 TB/s without).
+// Global -> LDS loads (no registers involved): scalar base + per-lane offset; the LDS destination of
+// lane l is M0 + instruction offset + l * BYTES, and the instruction offset advances the global
+// address as well.  N instructions of BYTES (4 or 16) per lane, 64 * BYTES apart.  M0 reaches the
+// instructions as an operand bound to that register (the compiler loads it and knows it is read),
+// not through a clobber.  Every tile is read exactly once, so the loads are marked non-temporal.
+template <int N, int BYTES>
+__device__ __forceinline__ void lds_dma(uint32_t lane_off, const uint8_t* base, uint32_t lds) {
+  static_assert((BYTES == 16 && (N == 1 || N == 4)) || (BYTES == 4 && (N == 1 || N == 2)), "forms in use");
+  register uint32_t m0_lds asm("m0") = lds;
+  if constexpr (BYTES == 16 && N == 4)
+    asm volatile(
+        "global_load_lds_dwordx4 %0, %1 nt\n\t"
+        "global_load_lds_dwordx4 %0, %1 offset:1024 nt\n\t"
+        "global_load_lds_dwordx4 %0, %1 offset:2048 nt\n\t"
+        "global_load_lds_dwordx4 %0, %1 offset:3072 nt"
+        :: "v"(lane_off), "s"(base), "s"(m0_lds) : "memory");
+  else if constexpr (BYTES == 16)
+    asm volatile("global_load_lds_dwordx4 %0, %1 nt" :: "v"(lane_off), "s"(base), "s"(m0_lds) : "memory");
+  else if constexpr (N == 2)
+    asm volatile(
+        "global_load_lds_dword %0, %1 nt\n\t"
+        "global_load_lds_dword %0, %1 offset:256 nt"
+        :: "v"(lane_off), "s"(base), "s"(m0_lds) : "memory");
+  else
+    asm volatile("global_load_lds_dword %0, %1 nt" :: "v"(lane_off), "s"(base), "s"(m0_lds) : "memory");
+}
+
+// Global -> LDS loads of one K page-head: 8 instructions with the high plane, 6 without
+// (non-temporal: 2 % on the whole launch; a read-only stream runs at 6.5 TB/s with the hint and
+// 5.9 TB/s without).
 template <bool BOOST>
 constexpr int kDmaK = BOOST ? 8 : 6;
 constexpr int kDmaV = 6;
@@ -297,24 +323,12 @@ __device__ __forceinline__ void dma_k(const Ctx& x, int page_index, uint32_t lds
   const uint8_t* page = L.key_cache + pg * L.key_cache_stride_page + (int64_t)x.h * k_head_bytes(BOOST ? 32 : 0);
   const uint8_t* meta = (const uint8_t*)L.key_meta + pg * L.key_meta_stride_page + (int64_t)x.h * kD * 4;
   const uint32_t off16 = x.lane * 16, off4 = x.lane * 4, off4dup = (x.lane & 31) * 4;
-  asm volatile(
-      "s_mov_b32 m0, %2\n\t"
-      "global_load_lds_dwordx4 %0, %1 nt\n\t"
-      "global_load_lds_dwordx4 %0, %1 offset:1024 nt\n\t"
-      "global_load_lds_dwordx4 %0, %1 offset:2048 nt\n\t"
-      "global_load_lds_dwordx4 %0, %1 offset:3072 nt"
-      :: "v"(off16), "s"(page), "s"(lds) : "memory", "m0");
+  lds_dma<4, 16>(off16, page, lds);
   if (BOOST) {
-    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1 nt"
-                 :: "v"(off16), "s"(page + kLoBytes), "s"(lds + kKOffHi) : "memory", "m0");
-    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dword %0, %1 nt"
-                 :: "v"(off4dup), "s"(page + kLoBytes + 1024), "s"(lds + kKOffIdx) : "memory", "m0");
+    lds_dma<1, 16>(off16, page + kLoBytes, lds + kKOffHi);
+    lds_dma<1, 4>(off4dup, page + kLoBytes + 1024, lds + kKOffIdx);
   }
-  asm volatile(
-      "s_mov_b32 m0, %2\n\t"
-      "global_load_lds_dword %0, %1 nt\n\t"
-      "global_load_lds_dword %0, %1 offset:256 nt"
-      :: "v"(off4), "s"(meta), "s"(lds + kKOffMeta) : "memory", "m0");
+  lds_dma<2, 4>(off4, meta, lds + kKOffMeta);
 }
 
 // Stage the page-head's (scale, zero) pairs and slot map in LDS in the order the operands need:
@@ -716,19 +730,9 @@ __device__ __forceinline__ void dma_v(const Ctx& x, int page_index, uint32_t lds
   const uint8_t* page = L.value_cache + pg * L.value_cache_stride_page + (int64_t)x.h * kVBytes;
   const uint8_t* meta = (const uint8_t*)L.value_meta + pg * L.value_meta_stride_page + (int64_t)x.h * kPage * 4;
   const uint32_t off16 = x.lane * 16;
-  asm volatile(
-      "s_mov_b32 m0, %2\n\t"
-      "global_load_lds_dwordx4 %0, %1 nt\n\t"
-      "global_load_lds_dwordx4 %0, %1 offset:1024 nt\n\t"
-      "global_load_lds_dwordx4 %0, %1 offset:2048 nt\n\t"
-      "global_load_lds_dwordx4 %0, %1 offset:3072 nt"
-      :: "v"(off16), "s"(page), "s"(lds) : "memory", "m0");
+  lds_dma<4, 16>(off16, page, lds);
   const uint32_t off4 = x.lane * 4;
-  asm volatile(
-      "s_mov_b32 m0, %2\n\t"
-      "global_load_lds_dword %0, %1 nt\n\t"
-      "global_load_lds_dword %0, %1 offset:256 nt"
-      :: "v"(off4), "s"(meta), "s"(lds + kVOffMeta) : "memory", "m0");
+  lds_dma<2, 4>(off4, meta, lds + kVOffMeta);
 }
 
 template <class LDS, class VSRC>

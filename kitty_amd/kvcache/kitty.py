@@ -319,6 +319,13 @@ class KittyCache(_HFCache):
         entirely inside the chunk are quantized straight from it; only pages that start with
         rows already buffered go through the Q-buffer.  On an empty layer this is
         ``update`` + ``quantize_prefill``.
+
+        With device counters the kernels decide per sequence whether the chunk fits: a sequence it
+        does not fit (it would pass ``MAX_PAGE``, or a page-table entry it needs is not a valid page
+        id) keeps its state and has its T tokens counted in the ``tokens_dropped`` status word,
+        while the host ints - a shadow of the longest sequence, advanced in closed form without
+        reading the device - move on regardless.  Call ``check_status()`` after chunk appends on such
+        caches when the tables or counters were written by anyone but this class.
         """
         L = self.kv_cache[layer_idx]
         if key_states.shape != value_states.shape or key_states.dim() != 4:

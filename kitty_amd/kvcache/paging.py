@@ -212,6 +212,10 @@ class PagedKittyCache(KittyCache):
             raise RuntimeError("one admission at a time")
         self._admit_slot, self._admit_len = slot, None
         self._admit_layers: set[int] = set()
+        # the status words are sticky and per slot: what the previous tenant of the slot left (a dry
+        # pool is an ordinary event here) must not be read as the new sequence's
+        for L in self.kv_cache:
+            L.status[slot].zero_()
         try:
             yield self
             if self._admit_len is None or len(self._admit_layers) != len(self.kv_cache):

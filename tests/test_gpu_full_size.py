@@ -34,6 +34,10 @@ def K():
 # 1.0e-2 / 3.1e-3 (config 2: peaked softmaxes, where "two" and "fma" themselves sit 1.3e-2 apart),
 # 2.9e-3 / 1.6e-3 (config 4), each with a quarter on top.  Against the affine value: 2e-3 everywhere.
 TOLS = {"c1": (7.5e-3, 1.0e-3), "c2": (1.3e-2, 4.0e-3), "c4": (3.7e-3, 2.0e-3)}
+# Both variants against the reference's output as it comes out (fp16 logits, probabilities and output over
+# the twice-rounded dequantization): (matrix-core kernel, plain kernel).  Measured 3.4e-3 / 3.4e-3 (config 1),
+# 1.37e-2 / 3.9e-3 (config 2), 1.95e-3 / 1.95e-3 (config 4); about 30 % on top.
+TOLS_LITERAL = {"c1": (4.5e-3, 4.5e-3), "c2": (1.8e-2, 5.0e-3), "c4": (2.6e-3, 2.6e-3)}
 
 
 def _sampled_check(K, L, out, q, units, max_len, config, counts=None, variant=0):
@@ -42,7 +46,8 @@ def _sampled_check(K, L, out, q, units, max_len, config, counts=None, variant=0)
         ol = K.u.oracle_head_view(L, b, h, max_len, None if counts is None else counts[b][:7])
         qs = q[b:b + 1, h * G:(h + 1) * G].cpu().numpy()
         got = out[b:b + 1, :, h * G:(h + 1) * G].cpu().numpy().astype(np.float64)
-        _check_attn(got, ol, qs, what=f"b={b} h={h}", variant=variant, tol_two=TOLS[config][0], tol_fma=TOLS[config][1])
+        _check_attn(got, ol, qs, what=f"{config} b={b} h={h}", variant=variant, tol_two=TOLS[config][0],
+                    tol_fma=TOLS[config][1], tol_literal=TOLS_LITERAL[config][variant])
 
 
 def _sampled_quantizer_check(L, k, v, units):

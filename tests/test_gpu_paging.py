@@ -221,6 +221,15 @@ def test_a_dry_pool_stalls_the_sequence_until_pages_return(K):
     for l in range(LAYERS):
         assert np.array_equal(dev[l], cache._shadow), l
     cache.check_tables()
+    # the stall left its record in slot 1's sticky status words, in every layer; the slot's next tenant
+    # starts with clean ones
+    st = cache.check_status(raise_on_error=False)
+    assert st["tokens_dropped"][:, 1].all() and st["flush_skipped"][:, 1].all() and not st["tokens_dropped"][:, 0].any()
+    with pytest.raises(RuntimeError, match="skipped work"):
+        cache.check_status()
+    cache.release(1)
+    Seq(9, 32 + 50, 1000, max_len).admit(K, cache, 1)
+    cache.check_status()
 
 
 def test_decode_step_graph_survives_admission_and_release(K):

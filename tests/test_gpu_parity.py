@@ -296,9 +296,17 @@ def _build(K, B, H_KV, H_Q, T, max_len, seed, student_t=False):
 # tests/test_gpu_full_size.py).  Measured worst cases over this file: 7.8e-3 against "two", 3.2e-3
 # against "fma", 9.8e-4 against "affine"; the bounds leave a quarter on top.
 TOL_TWO, TOL_FMA = 1.0e-2, 4.0e-3
+# Bound of BOTH variants against the reference's output as it actually comes out: "two" dequantization
+# AND fp16 logits, fp16 probabilities, fp16 output (kitty_attention.py:162-169, 317-320, 473, 389).  The
+# kernels keep logits and probabilities in fp32, which is where most of this distance comes from.
+# Measured over this file: 7.8e-3 (matrix-core kernel), 4.8e-3 (plain kernel, whose dequantization IS the
+# reference's: its whole distance is the reference's fp16 logits and probabilities); a quarter on top.
+TOL_LITERAL = {0: 1.0e-2, 1: 6.5e-3}
+LITERAL_LOG = []   # (what, variant, error against the literal reference output) of every check of a session
 
 
-def _check_attn(got, ol, q, seq_counts=None, what="", variant=0, elementwise=True, tol_two=TOL_TWO, tol_fma=TOL_FMA):
+def _check_attn(got, ol, q, seq_counts=None, what="", variant=0, elementwise=True, tol_two=TOL_TWO, tol_fma=TOL_FMA,
+                tol_literal=None):
     """The tolerance contract of decode attention: max-abs error of the fp16 outputs against
     dequantize-then-attend in float64 over the same packed cache, with constants only.
 
@@ -315,6 +323,12 @@ def _check_attn(got, ol, q, seq_counts=None, what="", variant=0, elementwise=Tru
       fp16 readings it is held to the fixed bounds ``tol_two`` / ``tol_fma``: what was measured on the
       case, plus a quarter, so that a regression shows.
     Returns the error against the kernel's own reading."""
+    literal = O.decode_attention(ol, q, 128 ** -0.5, seq_counts=seq_counts, reference_rounding=True, dequant="two")
+    err_literal = np.abs(got - literal.astype(np.float64)).max()
+    LITERAL_LOG.append((what, variant, float(err_literal)))
+    tol_literal = TOL_LITERAL[variant] if tol_literal is None else tol_literal
+    assert err_literal <= tol_literal, (f"{what}: {err_literal:.3e} vs the reference's own output (fp16 logits and "
+                                        f"probabilities over twice-rounded dequantization; bound {tol_literal:.1e})")
     kw = dict(seq_counts=seq_counts, reference_rounding=False)
     two = O.decode_attention(ol, q, 128 ** -0.5, dequant="two", **kw)
     err_two = np.abs(got - two).max()
@@ -598,3 +612,32 @@ def test_attention_rejects_bad_arguments(K):
     L.Q_Buffer_Count_K = 0
     with pytest.raises(ValueError):
         cache.quantize_prefill(0)                            # update() was never called
+
+
+def test_profile_events_belong_to_the_next_call_even_a_rejected_one(K):
+    """kitty_profile_next_split arms two events for the calling thread's next split pass.  A call that is
+    rejected on the host takes them too: they must not ride on a later, unrelated launch."""
+    import ctypes
+
+    import bench
+    from kitty_amd import _lib
+    lib, hip = _lib.lib(), bench.HipEvents()
+    cache, _ = _build(K, 1, 2, 8, 32 + 128 * 2 + 9, 1024, seed=77)
+    d = cache.kv_cache[0].descriptor()
+    q = K.u.to_dev(make_q(1, 8, seed=77))
+    n = 2
+    ws = torch.empty(lib.kitty_decode_attn_workspace_bytes(1, 8, 128, n), dtype=torch.uint8, device="cuda")
+    st = _lib.current_stream_ptr(q.device)
+    split = lambda nbytes: lib.kitty_decode_attn_split(d, q.data_ptr(), 1, 8, 128 ** -0.5, ws.data_ptr(), nbytes, n, 0, st)
+    e0, e1 = hip.create(), hip.create()
+    assert lib.kitty_profile_next_split(e0, e1) == 0
+    assert split(16) == -5                                   # KITTY_E_WORKSPACE: nothing launched
+    assert split(ws.numel()) == 0
+    torch.cuda.synchronize()
+    ms = ctypes.c_float()
+    assert hip.hip.hipEventElapsedTime(ctypes.byref(ms), e0, e1) != 0, "events of a rejected call were recorded later"
+    hip.hip.hipGetLastError()                                # (the failed query above is this thread's last error)
+    assert lib.kitty_profile_next_split(e0, e1) == 0
+    assert split(ws.numel()) == 0
+    torch.cuda.synchronize()
+    assert hip.elapsed_us(e0, e1) > 0

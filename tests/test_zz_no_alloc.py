@@ -156,3 +156,51 @@ def test_decode_step_replayed_from_a_graph(K):
     assert int(a.seq_counts[0, 1]) == 2 and int(a.seq_counts[0, 3]) == 1          # both Q-buffers were flushed
     for name in ("KeyCache", "KeyCache_metadata", "ValueCache", "ValueCache_metadata", "Q_Buffer_K", "Local_Buffer_V"):
         assert torch.equal(getattr(a, name), getattr(b, name)), name
+
+
+def test_first_call_on_a_capturing_stream_is_refused_with_a_reason():
+    """The first call on a device looks the array's address up in the runtime, which a stream capture
+    must not contain.  In a fresh process, a first call under capture is rejected (KITTY_E_RANGE, nothing
+    recorded), and after one eager call the same capture works."""
+    import os
+    import subprocess
+    import sys
+    if not torch.cuda.is_available():
+        pytest.skip("needs a GPU")
+    code = r"""
+import sys, torch
+sys.path.insert(0, %r)
+import kitty_amd
+from kitty_amd import _lib
+from tests import gpu_util as u
+from tests.helpers import make_kv, make_q
+lib = _lib.lib()
+k, v = make_kv(1, 2, 32 + 128 * 2 + 5, seed=5)
+c = kitty_amd.KittyCache(u.cfg(2, 8), 1, 1024)
+c.update(u.to_dev(k), u.to_dev(v), 0)
+c.quantize_prefill(0)
+L = c.kv_cache[0]
+q = u.to_dev(make_q(1, 8, seed=5))
+out = torch.zeros((1, 1, 8, 128), dtype=torch.float16, device="cuda")
+call = lambda: lib.kitty_decode_attn_static(L.descriptor(), q.data_ptr(), 1, 8, 128 ** -0.5, out.data_ptr(), 2, 0,
+                                            _lib.current_stream_ptr(q.device))
+torch.cuda.synchronize()
+g = torch.cuda.CUDAGraph()
+with torch.cuda.graph(g):
+    rc = call()
+msg = lib.kitty_last_error().decode()
+assert rc == -3 and "before capturing" in msg, (rc, msg)
+assert call() == 0
+torch.cuda.synchronize()
+eager = out.clone()
+out.zero_()
+g2 = torch.cuda.CUDAGraph()
+with torch.cuda.graph(g2):
+    assert call() == 0
+g2.replay()
+torch.cuda.synchronize()
+assert torch.equal(out, eager) and bool(out.abs().sum() > 0)
+print("ok")
+""" % os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0 and "ok" in r.stdout, r.stdout + r.stderr
