@@ -15,13 +15,22 @@ void launch_prefill_attn(const kitty_kv_layer& L, const void* q, int64_t q_strid
                          int64_t q_stride_t, const void* k_new, const void* v_new, int64_t new_stride_b,
                          int64_t new_stride_h, int64_t new_stride_t, int B, int H_Q, int Tq, float scaling,
                          void* out, hipStream_t stream);
+// head dimensions other than 128 (any_dim.hip)
+void launch_decode_any(const kitty_kv_layer& L, const void* q, int B, int H_Q, float scaling, float* ws_ml,
+                       float* ws_acc, int num_splits, hipStream_t stream);
+void launch_merge_any(int D, const float* ws_ml, const float* ws_acc, void* out, int B, int H_Q, int num_splits,
+                      hipStream_t stream);
+void launch_prefill_any(const kitty_kv_layer& L, const void* q, int64_t q_stride_b, int64_t q_stride_h,
+                        int64_t q_stride_t, const void* k_new, const void* v_new, int64_t new_stride_b,
+                        int64_t new_stride_h, int64_t new_stride_t, int B, int H_Q, int Tq, float scaling, void* out,
+                        hipStream_t stream);
 }  // namespace kitty
 
 using namespace kitty;
 
 extern "C" size_t kitty_decode_attn_workspace_bytes(int B, int H_Q, int D, int num_splits) {
-  if (B <= 0 || H_Q <= 0 || D != kD || num_splits <= 0) return 0;
-  return ws_total_bytes(B, H_Q, num_splits);
+  if (B <= 0 || H_Q <= 0 || !head_dim_supported(D) || num_splits <= 0) return 0;
+  return ws_total_bytes(B, H_Q, num_splits, D);
 }
 
 namespace kitty {
@@ -79,13 +88,15 @@ thread_local hipEvent_t g_ev_start = nullptr, g_ev_stop = nullptr;
 int check_layer(const kitty_kv_layer* layer, const void* q, int B, int H_Q, int* max_tiles) {
   KITTY_REQUIRE(layer && q, KITTY_E_NULL, "layer / q is NULL");
   const kitty_kv_layer& L = *layer;
-  KITTY_REQUIRE(L.D == kD && L.PAGE_SIZE == kPage, KITTY_E_SHAPE,
-                "kernels are built for head_dim 128 and page_size 128, got D=%d page_size=%d", L.D, L.PAGE_SIZE);
+  KITTY_REQUIRE(head_dim_supported(L.D) && L.PAGE_SIZE == kPage, KITTY_E_SHAPE,
+                "kernels are built for head_dim 64, 128 or 256 and page_size 128, got D=%d page_size=%d", L.D,
+                L.PAGE_SIZE);
   KITTY_REQUIRE(L.H_KV >= 1 && H_Q >= L.H_KV && H_Q % L.H_KV == 0, KITTY_E_SHAPE,
                 "H_Q=%d must be a positive multiple of H_KV=%d", H_Q, L.H_KV);
   KITTY_REQUIRE(H_Q / L.H_KV <= 16, KITTY_E_SHAPE, "KV_GROUP (%d) exceeds MAX_KV_GROUP (16)", H_Q / L.H_KV);
-  KITTY_REQUIRE(L.D_BOOSTED >= 0 && L.D_BOOSTED <= kD && k_head_bytes(L.D_BOOSTED) % 16 == 0, KITTY_E_SHAPE,
-                "unsupported D_BOOSTED=%d", L.D_BOOSTED);
+  KITTY_REQUIRE(L.D_BOOSTED >= 0 && L.D_BOOSTED <= L.D && L.D_BOOSTED <= 255 &&
+                    k_head_bytes_d(L.D, L.D_BOOSTED) % 16 == 0,
+                KITTY_E_SHAPE, "unsupported D_BOOSTED=%d", L.D_BOOSTED);
   KITTY_REQUIRE(L.S >= 0 && L.S <= kPage && L.MAX_PAGE >= 0, KITTY_E_SHAPE, "S=%d must be in [0, 128]", L.S);
   KITTY_REQUIRE(B >= 1 && B <= 65535 && L.H_KV <= 65535, KITTY_E_RANGE, "bad batch size %d", B);
   KITTY_REQUIRE(L.key_cache && L.key_meta && L.value_cache && L.value_meta && L.page_table_k && L.page_table_v &&
@@ -105,9 +116,9 @@ int check_layer(const kitty_kv_layer* layer, const void* q, int B, int H_Q, int*
   KITTY_REQUIRE(L.cache_pages_k >= 0 && L.cache_pages_v >= 0 && ((uintptr_t)L.status % 4) == 0 &&
                     ((uintptr_t)L.seq_counts % 4) == 0,
                 KITTY_E_RANGE, "negative cache_pages_k / cache_pages_v, or misaligned status / seq_counts");
-  KITTY_REQUIRE(L.key_cache_stride_page >= (int64_t)L.H_KV * k_head_bytes(L.D_BOOSTED) &&
-                    L.value_cache_stride_page >= (int64_t)L.H_KV * kVBytes &&
-                    L.key_meta_stride_page >= (int64_t)L.H_KV * kD * 4 &&
+  KITTY_REQUIRE(L.key_cache_stride_page >= (int64_t)L.H_KV * k_head_bytes_d(L.D, L.D_BOOSTED) &&
+                    L.value_cache_stride_page >= (int64_t)L.H_KV * v_head_bytes_d(L.D) &&
+                    L.key_meta_stride_page >= (int64_t)L.H_KV * L.D * 4 &&
                     L.value_meta_stride_page >= (int64_t)L.H_KV * kPage * 4,
                 KITTY_E_RANGE, "a page stride is smaller than one page");
   *max_tiles = 2 + L.MAX_PAGE;
@@ -131,13 +142,13 @@ int check_layer(const kitty_kv_layer* layer, const void* q, int B, int H_Q, int*
   return 0;
 }
 
-int check_workspace(const void* workspace, size_t workspace_bytes, int B, int H_Q, int num_splits) {
+int check_workspace(const void* workspace, size_t workspace_bytes, int B, int H_Q, int num_splits, int D = kD) {
   KITTY_REQUIRE(workspace != nullptr, KITTY_E_NULL, "workspace is NULL");
   KITTY_REQUIRE(((uintptr_t)workspace % 256) == 0, KITTY_E_ALIGN, "workspace needs 256-byte alignment");
   KITTY_REQUIRE(num_splits >= 1 && num_splits <= 65535, KITTY_E_RANGE, "num_splits=%d out of range", num_splits);
-  KITTY_REQUIRE(workspace_bytes >= ws_total_bytes(B, H_Q, num_splits), KITTY_E_WORKSPACE,
+  KITTY_REQUIRE(workspace_bytes >= ws_total_bytes(B, H_Q, num_splits, D), KITTY_E_WORKSPACE,
                 "workspace of %zu bytes is smaller than the %zu needed for %d splits", workspace_bytes,
-                ws_total_bytes(B, H_Q, num_splits), num_splits);
+                ws_total_bytes(B, H_Q, num_splits, D), num_splits);
   return 0;
 }
 
@@ -161,12 +172,16 @@ extern "C" int kitty_decode_attn_split(const kitty_kv_layer* layer, const void* 
   g_ev_start = g_ev_stop = nullptr;
   int max_tiles = 0;
   if (int rc = check_layer(layer, q, B, H_Q, &max_tiles)) return rc;
-  if (int rc = check_workspace(workspace, workspace_bytes, B, H_Q, num_splits)) return rc;
+  if (int rc = check_workspace(workspace, workspace_bytes, B, H_Q, num_splits, layer->D)) return rc;
   KITTY_REQUIRE(variant == 0 || variant == 1, KITTY_E_SHAPE, "unknown variant %d", variant);
   const kitty_kv_layer& L = *layer;
   float* ws_ml = (float*)workspace;
   float* ws_acc = (float*)((uint8_t*)workspace + ws_ml_bytes(B, H_Q, num_splits));
-  if (variant == 0 && decode_mfma_supported(L, H_Q)) {
+  if (L.D != kD) {   // one kernel for both variants: the reference's order of operations on the vector ALUs
+    if (ev0) (void)hipEventRecord(ev0, (hipStream_t)stream);
+    launch_decode_any(L, q, B, H_Q, scaling, ws_ml, ws_acc, num_splits, (hipStream_t)stream);
+    if (ev1) (void)hipEventRecord(ev1, (hipStream_t)stream);
+  } else if (variant == 0 && decode_mfma_supported(L, H_Q)) {
     uint32_t* ws_plan = (uint32_t*)((uint8_t*)ws_acc + ws_acc_bytes(B, H_Q, num_splits));
     launch_decode_mfma(L, q, B, H_Q, scaling, ws_ml, ws_acc, ws_plan, num_splits, device_simds(), (hipStream_t)stream,
                        ev0, ev1);
@@ -188,12 +203,14 @@ extern "C" int kitty_profile_next_split(void* start_event, void* stop_event) {
 extern "C" int kitty_decode_attn_merge(const void* workspace, size_t workspace_bytes, int B, int H_Q, int D,
                                        int num_splits, void* out, void* stream) {
   KITTY_REQUIRE(out != nullptr, KITTY_E_NULL, "out is NULL");
-  KITTY_REQUIRE(D == kD && B >= 1 && B <= 65535 && H_Q >= 1, KITTY_E_SHAPE, "bad B=%d H_Q=%d D=%d", B, H_Q, D);
+  KITTY_REQUIRE(head_dim_supported(D) && B >= 1 && B <= 65535 && H_Q >= 1 && H_Q <= 65535, KITTY_E_SHAPE,
+                "bad B=%d H_Q=%d D=%d", B, H_Q, D);
   KITTY_REQUIRE(((uintptr_t)out % 16) == 0, KITTY_E_ALIGN, "out needs 16-byte alignment");
-  if (int rc = check_workspace(workspace, workspace_bytes, B, H_Q, num_splits)) return rc;
+  if (int rc = check_workspace(workspace, workspace_bytes, B, H_Q, num_splits, D)) return rc;
   const float* ws_ml = (const float*)workspace;
   const float* ws_acc = (const float*)((const uint8_t*)workspace + ws_ml_bytes(B, H_Q, num_splits));
-  launch_decode_merge(ws_ml, ws_acc, out, B, H_Q, num_splits, (hipStream_t)stream);
+  if (D != kD) launch_merge_any(D, ws_ml, ws_acc, out, B, H_Q, num_splits, (hipStream_t)stream);
+  else launch_decode_merge(ws_ml, ws_acc, out, B, H_Q, num_splits, (hipStream_t)stream);
   return check_launch("kitty_decode_attn_merge");
 }
 
@@ -223,8 +240,13 @@ extern "C" int kitty_prefill_attn(const kitty_kv_layer* layer, const void* q, in
                     q_stride_b % 16 == 0 && q_stride_h % 16 == 0 && q_stride_t % 16 == 0 &&
                     new_stride_b % 16 == 0 && new_stride_h % 16 == 0 && new_stride_t % 16 == 0,
                 KITTY_E_ALIGN, "q, k_new, v_new and out need 16-byte aligned bases and strides");
-  KITTY_REQUIRE(q_stride_t >= kD * 2 && new_stride_t >= kD * 2, KITTY_E_ALIGN,
+  KITTY_REQUIRE(q_stride_t >= layer->D * 2 && new_stride_t >= layer->D * 2, KITTY_E_ALIGN,
                 "a token stride is smaller than one row of D fp16 values");
+  if (layer->D != kD) {
+    launch_prefill_any(*layer, q, q_stride_b, q_stride_h, q_stride_t, k_new, v_new, new_stride_b, new_stride_h,
+                       new_stride_t, B, H_Q, T_q, scaling, out, (hipStream_t)stream);
+    return check_launch("kitty_prefill_attn");
+  }
   launch_prefill_attn(*layer, q, q_stride_b, q_stride_h, q_stride_t, k_new, v_new, new_stride_b, new_stride_h,
                       new_stride_t, B, H_Q, T_q, scaling, out, (hipStream_t)stream);
   return check_launch("kitty_prefill_attn");

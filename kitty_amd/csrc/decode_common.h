@@ -69,11 +69,12 @@ __device__ __forceinline__ void report_bad_page(const kitty_kv_layer& L, int b, 
 }
 
 // fp16 row of V for token u of the region that follows the V pages
-__device__ inline const __half* v_tail_row(const kitty_kv_layer& L, const SeqCounts& c, int b, int h, int u) {
+__device__ inline const __half* v_tail_row(const kitty_kv_layer& L, const SeqCounts& c, int b, int h, int u,
+                                          int head_dim = kD) {
   const int64_t base = (int64_t)b * L.win_stride_b + (int64_t)h * L.win_stride_h;
-  if (u < c.rv) return (const __half*)((const uint8_t*)L.qbuf_v + base) + (int64_t)u * kD;
+  if (u < c.rv) return (const __half*)((const uint8_t*)L.qbuf_v + base) + (int64_t)u * head_dim;
   const int r = (c.off + (u - c.rv)) & (kPage - 1);
-  return (const __half*)((const uint8_t*)L.local_v + base) + (int64_t)r * kD;
+  return (const __half*)((const uint8_t*)L.local_v + base) + (int64_t)r * head_dim;
 }
 
 // Split-K workspace: [B*H_Q*splits][2] floats (running max of the logits in log2 units, i.e.
@@ -83,8 +84,8 @@ __host__ __device__ inline size_t ws_ml_bytes(int B, int H_Q, int splits) {
   size_t n = (size_t)B * H_Q * splits * 2 * sizeof(float);
   return (n + 255) & ~(size_t)255;
 }
-__host__ __device__ inline size_t ws_acc_bytes(int B, int H_Q, int splits) {
-  return (size_t)B * H_Q * splits * kD * sizeof(float);   // a multiple of 512
+__host__ __device__ inline size_t ws_acc_bytes(int B, int H_Q, int splits, int head_dim = kD) {
+  return (size_t)B * H_Q * splits * head_dim * sizeof(float);   // a multiple of 256
 }
 // After the partials: the work list of a launch that runs in several rounds (decode_plan_kernel) -
 // kPlanHeader words, of which the first is the number of items, then one word per item
@@ -94,8 +95,8 @@ __host__ __device__ inline size_t ws_plan_bytes(int B, int splits) {
   size_t n = ((size_t)B * splits + kPlanHeader) * sizeof(uint32_t);
   return (n + 255) & ~(size_t)255;
 }
-__host__ __device__ inline size_t ws_total_bytes(int B, int H_Q, int splits) {
-  return ws_ml_bytes(B, H_Q, splits) + ws_acc_bytes(B, H_Q, splits) + ws_plan_bytes(B, splits);
+__host__ __device__ inline size_t ws_total_bytes(int B, int H_Q, int splits, int head_dim = kD) {
+  return ws_ml_bytes(B, H_Q, splits) + ws_acc_bytes(B, H_Q, splits, head_dim) + ws_plan_bytes(B, splits);
 }
 
 }  // namespace kitty

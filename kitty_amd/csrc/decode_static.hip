@@ -59,7 +59,7 @@ extern "C" int kitty_decode_attn_static(const kitty_kv_layer* layer, const void*
   // the checks, and the tile count behind the default split rule, are kitty_decode_attn's own
   int max_tiles = 0;
   if (int rc = decode_check_layer(layer, q, B, H_Q, &max_tiles)) return rc;
-  const size_t per_split = ws_total_bytes(B, H_Q, 1) + 768;   // an upper bound of the growth per split
+  const size_t per_split = ws_total_bytes(B, H_Q, 1, layer->D) + 768;   // an upper bound of the growth per split
   if (num_splits <= 0) {
     // the default of kitty_decode_attn, cut back to what the array holds
     num_splits = kitty_decode_attn_default_splits(B, layer->H_KV, max_tiles, layer->seq_counts != nullptr);
@@ -67,13 +67,13 @@ extern "C" int kitty_decode_attn_static(const kitty_kv_layer* layer, const void*
     if ((size_t)num_splits > fit) num_splits = (int)fit;
     KITTY_REQUIRE(num_splits >= 1, KITTY_E_WORKSPACE,
                   "B=%d x H_Q=%d query heads need %zu bytes of partials per split, the library's array holds %zu", B,
-                  H_Q, ws_total_bytes(B, H_Q, 1), (size_t)KITTY_STATIC_WORKSPACE_BYTES);
+                  H_Q, ws_total_bytes(B, H_Q, 1, layer->D), (size_t)KITTY_STATIC_WORKSPACE_BYTES);
   }
-  KITTY_REQUIRE(num_splits <= 65535 && ws_total_bytes(B, H_Q, num_splits) <= KITTY_STATIC_WORKSPACE_BYTES,
+  KITTY_REQUIRE(num_splits <= 65535 && ws_total_bytes(B, H_Q, num_splits, layer->D) <= KITTY_STATIC_WORKSPACE_BYTES,
                 KITTY_E_WORKSPACE,
                 "%d splits of B=%d x H_Q=%d query heads need %zu bytes of partials, the library's array holds %zu: "
                 "ask for fewer splits or use kitty_decode_attn with a workspace of your own",
-                num_splits, B, H_Q, ws_total_bytes(B, H_Q, num_splits), (size_t)KITTY_STATIC_WORKSPACE_BYTES);
+                num_splits, B, H_Q, ws_total_bytes(B, H_Q, num_splits, layer->D), (size_t)KITTY_STATIC_WORKSPACE_BYTES);
   void* ws = nullptr;
   if (int rc = scratch_of_current_device(&ws, (hipStream_t)stream)) return rc;
   return kitty_decode_attn(layer, q, B, H_Q, scaling, out, ws, KITTY_STATIC_WORKSPACE_BYTES, num_splits, variant, stream);

@@ -18,6 +18,14 @@ constexpr int kLoBytes = kD * kRowBytes;                 // 4096: low plane of a
 constexpr int kVBytes = kPage * kRowBytes;               // 4096: a V page-head
 
 __host__ __device__ inline int k_head_bytes(int d_boost) { return kRowBytes * (kD + d_boost) + kD; }
+// Other head dimensions (the reference derives everything from config.head_dim, kitty.py:39-44, and its
+// kernels take D as a parameter, kitty_quant_pack.py:42-45, kitty_attention.py:59-62): 64 and 256 run
+// on plain kernels of their own (any_dim.hip); the tuned kernels are those for 128.
+__host__ __device__ inline bool head_dim_supported(int d) { return d == 64 || d == kD || d == 256; }
+__host__ __device__ inline int k_head_bytes_d(int head_dim, int d_boost) {
+  return kRowBytes * (head_dim + d_boost) + head_dim;
+}
+__host__ __device__ inline int v_head_bytes_d(int head_dim) { return kPage * head_dim / 4; }
 
 // v_max_f32 / v_max3_f32 as single instructions.  In front of fmaxf the compiler puts a NaN-quieting
 // `v_max_f32 x, x, x` for every operand it cannot prove canonical (anything that crosses a basic

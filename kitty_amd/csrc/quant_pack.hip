@@ -9,36 +9,24 @@
 // 106-112, 201-204, 227-230): min/max, range, scale = range / qmax (IEEE fp32 divide, floored at
 // 1e-6), (x - min) / scale in fp32, floor(. + 0.5), clamp to [0, qmax]; the stored scale is the
 // fp32 scale rounded to fp16, the stored zero point is the minimum itself.
-#include "kitty_common.h"
+#include "quant_arith.h"
+
+namespace kitty {
+// head dimensions other than 128 (any_dim.hip)
+void launch_quant_k_any(int D, int mode, const void* key, int64_t sb, int64_t sh, int64_t st, int B, int H,
+                        int t_offset, int pages, int d_boost, const uint8_t* slot_in, uint8_t* slot_out,
+                        const int64_t* page_table, int64_t pt_stride, int page_offset, uint8_t* cache,
+                        int64_t cache_stride, void* meta, int64_t meta_stride, int64_t cache_pages, int32_t* status,
+                        hipStream_t stream);
+void launch_quant_v_any(int D, const void* value, int64_t sb, int64_t sh, int64_t st, int B, int H, int t_offset,
+                        int pages, const int64_t* page_table, int64_t pt_stride, int page_offset, uint8_t* cache,
+                        int64_t cache_stride, void* meta, int64_t meta_stride, int64_t cache_pages, int32_t* status,
+                        hipStream_t stream);
+}  // namespace kitty
 
 using namespace kitty;
 
 namespace {
-
-// fp16 bit pattern of (S * 2^-31) rounded to nearest even, S = sum over 128 tokens of |x| * 2^24,
-// i.e. the mean of |x| rounded once.  Positive fp16 patterns order like their values.
-__device__ inline uint16_t mean_abs_fp16_bits(uint64_t S) {
-  if (S == 0) return 0;
-  int msb = 63 - __clzll((long long)S);
-  int E = msb - 31;
-  if (E >= -14) {
-    int shift = msb - 10;
-    uint64_t q;
-    if (shift > 0) {
-      q = S >> shift;
-      uint64_t rem = S & ((1ull << shift) - 1), half = 1ull << (shift - 1);
-      if (rem > half || (rem == half && (q & 1))) q++;
-    } else {
-      q = S << (-shift);
-    }
-    if (q == 2048) { q = 1024; E++; }
-    if (E > 15) return 0x7C00;
-    return (uint16_t)(((uint32_t)(E + 15) << 10) | (uint32_t)(q & 1023));
-  }
-  uint64_t q = S >> 7, rem = S & 127;
-  if (rem > 64 || (rem == 64 && (q & 1))) q++;
-  return (uint16_t)q;
-}
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 // 16 bytes of the source, which is read exactly once: a non-temporal load (a read-only stream
@@ -48,35 +36,6 @@ __device__ __forceinline__ uint4 nt_load16(const uint8_t* p) {
   return uint4{v.x, v.y, v.z, v.w};
 }
 
-__device__ inline float h2f(uint16_t bits) { return __half2float(__ushort_as_half(bits)); }
-
-// IEEE fp32 division by a divisor that is shared by a whole group.  This is the correctly rounded
-// sequence the compiler emits for `/` (reciprocal, one Newton step, quotient, two residual
-// corrections) without its range scaling and special-case fix-up, which cannot trigger here: the
-// divisor is a scale in [1e-6, 4.4e4], the dividend x - min is 0 or in [2^-24, 1.4e5].  The
-// reciprocal part depends on the divisor only and is computed once per group.  Bit-identical to
-// `/` on that domain except that -0 / d gives +0, which the + 0.5 that follows erases.
-struct Divisor {
-  float d, r;
-};
-__device__ __forceinline__ Divisor make_divisor(float d) {
-  float r = __builtin_amdgcn_rcpf(d);
-  const float e = __builtin_fmaf(-d, r, 1.0f);
-  r = __builtin_fmaf(e, r, r);
-  return {d, r};
-}
-__device__ __forceinline__ float div_by(float n, Divisor k) {
-  float q = n * k.r;
-  float rem = __builtin_fmaf(-k.d, q, n);
-  q = __builtin_fmaf(rem, k.r, q);
-  rem = __builtin_fmaf(-k.d, q, n);
-  return __builtin_fmaf(rem, k.r, q);
-}
-// floor(min(x / scale + 0.5, qmax + 0.5)) as a float: the code.  x >= 0, so the lower clamp of
-// the reference never acts, and clamping before the floor gives the same integer.
-__device__ __forceinline__ float code_of(float x_minus_min, Divisor k, float qlim) {
-  return __builtin_floorf(fminf(div_by(x_minus_min, k) + 0.5f, qlim));
-}
 // The same codes for N values of one group at a time, mostly without the division:
 //   t = fma(x, r, c0),  c0 = fma(-min, r, 0.5),  r = the refined reciprocal of the scale.
 // Against the reference's fl(fl((x - min) / scale) + 0.5) this differs by the roundings of x - min,
@@ -749,8 +708,8 @@ __global__ __launch_bounds__(64) void chunk_advance_kernel(kitty_kv_layer L, int
 int check_src(const void* p, int64_t sb, int64_t sh, int64_t st, int B, int H, int T, int D, int t_offset,
               int pages, int page_size) {
   KITTY_REQUIRE(p != nullptr, KITTY_E_NULL, "source tensor is NULL");
-  KITTY_REQUIRE(D == kD && page_size == kPage, KITTY_E_SHAPE,
-                "kernels are built for head_dim 128 and page_size 128, got D=%d page_size=%d", D, page_size);
+  KITTY_REQUIRE(head_dim_supported(D) && page_size == kPage, KITTY_E_SHAPE,
+                "kernels are built for head_dim 64, 128 or 256 and page_size 128, got D=%d page_size=%d", D, page_size);
   KITTY_REQUIRE(B >= 0 && H >= 1 && pages >= 0 && t_offset >= 0, KITTY_E_RANGE,
                 "bad B=%d H=%d pages=%d t_offset=%d", B, H, pages, t_offset);
   KITTY_REQUIRE((int64_t)t_offset + (int64_t)pages * page_size <= (int64_t)T, KITTY_E_RANGE,
@@ -782,8 +741,14 @@ extern "C" int kitty_select_boost_k(const void* key, int64_t stride_b, int64_t s
                                     uint8_t* slot_map, void* stream) {
   if (int rc = check_src(key, stride_b, stride_h, stride_t, B, H, T, D, t_offset, pages, page_size)) return rc;
   KITTY_REQUIRE(slot_map != nullptr, KITTY_E_NULL, "slot_map is NULL");
-  KITTY_REQUIRE(d_boost >= 0 && d_boost <= D, KITTY_E_SHAPE, "d_boost must be in [0, %d], got %d", D, d_boost);
+  KITTY_REQUIRE(d_boost >= 0 && d_boost <= D && d_boost <= 255, KITTY_E_SHAPE,
+                "d_boost must be in [0, %d] and fit the uint8 slot map, got %d", D, d_boost);
   if (B == 0 || pages == 0) return 0;
+  if (D != kD) {
+    launch_quant_k_any(D, 2, key, stride_b, stride_h, stride_t, B, H, t_offset, pages, d_boost, nullptr, slot_map,
+                       nullptr, 0, 0, nullptr, 0, nullptr, 0, 0, nullptr, (hipStream_t)stream);
+    return check_launch("kitty_select_boost_k");
+  }
   hipLaunchKernelGGL(quant_pack_k_kernel<2>, dim3(pages, H, B), dim3(256), 0, (hipStream_t)stream,
                      (const uint8_t*)key, stride_b, stride_h, stride_t, t_offset, d_boost, nullptr, slot_map,
                      pages, nullptr, 0, 0, nullptr, 0, nullptr, 0, 0, nullptr);
@@ -801,13 +766,20 @@ extern "C" int kitty_quant_pack_k(const void* key, int64_t stride_b, int64_t str
   KITTY_REQUIRE(((uintptr_t)status % 4) == 0, KITTY_E_ALIGN, "status needs 4-byte alignment");
   // the slot map is a uint8 with d_boost as the "not boosted" marker, and the high plane has
   // d_boost rows: keep rows 4-byte friendly
-  KITTY_REQUIRE(d_boost >= 0 && d_boost <= D, KITTY_E_SHAPE, "d_boost must be in [0, %d], got %d", D, d_boost);
-  KITTY_REQUIRE((k_head_bytes(d_boost) % 16) == 0, KITTY_E_ALIGN,
+  KITTY_REQUIRE(d_boost >= 0 && d_boost <= D && d_boost <= 255, KITTY_E_SHAPE,
+                "d_boost must be in [0, %d] and fit the uint8 slot map, got %d", D, d_boost);
+  KITTY_REQUIRE((k_head_bytes_d(D, d_boost) % 16) == 0, KITTY_E_ALIGN,
                 "d_boost=%d gives a per-head page size that is not a multiple of 16 bytes", d_boost);
   if (int rc = check_dst(page_table, page_offset, cache, cache_stride_page, meta, meta_stride_page, cache_pages,
-                         (int64_t)H * k_head_bytes(d_boost), (int64_t)H * kD * 4))
+                         (int64_t)H * k_head_bytes_d(D, d_boost), (int64_t)H * D * 4))
     return rc;
   if (B == 0 || pages == 0) return 0;
+  if (D != kD) {
+    launch_quant_k_any(D, slot_map ? 0 : 1, key, stride_b, stride_h, stride_t, B, H, t_offset, pages, d_boost, slot_map,
+                       nullptr, page_table, page_table_stride_b, page_offset, cache, cache_stride_page, meta,
+                       meta_stride_page, cache_pages, status, (hipStream_t)stream);
+    return check_launch("kitty_quant_pack_k");
+  }
   dim3 grid(pages, H, B), block(256);
   if (slot_map)
     hipLaunchKernelGGL(quant_pack_k_kernel<0>, grid, block, 0, (hipStream_t)stream, (const uint8_t*)key, stride_b,
@@ -831,9 +803,15 @@ extern "C" int kitty_quant_pack_v(const void* value, int64_t stride_b, int64_t s
   if (int rc = check_src(value, stride_b, stride_h, stride_t, B, H, T, D, t_offset, pages, page_size)) return rc;
   KITTY_REQUIRE(((uintptr_t)status % 4) == 0, KITTY_E_ALIGN, "status needs 4-byte alignment");
   if (int rc = check_dst(page_table, page_offset, cache, cache_stride_page, meta, meta_stride_page, cache_pages,
-                         (int64_t)H * kVBytes, (int64_t)H * kPage * 4))
+                         (int64_t)H * v_head_bytes_d(D), (int64_t)H * kPage * 4))
     return rc;
   if (B == 0 || pages == 0) return 0;
+  if (D != kD) {
+    launch_quant_v_any(D, value, stride_b, stride_h, stride_t, B, H, t_offset, pages, page_table, page_table_stride_b,
+                       page_offset, cache, cache_stride_page, meta, meta_stride_page, cache_pages, status,
+                       (hipStream_t)stream);
+    return check_launch("kitty_quant_pack_v");
+  }
   hipLaunchKernelGGL(quant_pack_v_kernel, dim3(pages, H, B), dim3(256), 0, (hipStream_t)stream,
                      (const uint8_t*)value, stride_b, stride_h, stride_t, t_offset, page_table,
                      page_table_stride_b, page_offset, cache, cache_stride_page, (uint8_t*)meta, meta_stride_page,
@@ -847,7 +825,8 @@ int check_append_layer(const kitty_kv_layer* layer, int B) {
   const kitty_kv_layer& L = *layer;
   KITTY_REQUIRE(L.seq_counts != nullptr, KITTY_E_NULL, "this entry point needs per-sequence counters (seq_counts)");
   KITTY_REQUIRE(L.D == kD && L.PAGE_SIZE == kPage, KITTY_E_SHAPE,
-                "kernels are built for head_dim 128 and page_size 128, got D=%d page_size=%d", L.D, L.PAGE_SIZE);
+                "the device-counter entry points are built for head_dim 128 and page_size 128 (other head dimensions "
+                "keep the counters on the host), got D=%d page_size=%d", L.D, L.PAGE_SIZE);
   KITTY_REQUIRE(L.H_KV >= 1 && L.H_KV <= 65535 && B >= 1 && B <= 65535, KITTY_E_RANGE, "bad H_KV=%d or B=%d", L.H_KV, B);
   KITTY_REQUIRE(L.S >= 0 && L.S <= kPage && L.MAX_PAGE >= 0 && L.D_BOOSTED >= 0 && L.D_BOOSTED <= kD &&
                     k_head_bytes(L.D_BOOSTED) % 16 == 0,

@@ -121,6 +121,10 @@ class PagedKittyCache(KittyCache):
 
     def __init__(self, config, max_batch_size: int, max_length: int, pool_pages: int, *, device="cuda") -> None:
         dev = torch.device(device)
+        head_dim = getattr(config, "head_dim", None) or config.hidden_size // config.num_attention_heads
+        if head_dim != 128:
+            raise ValueError(f"a page pool keeps its counters on the device, which is built for head_dim 128 "
+                             f"(got {head_dim}); use KittyCache for other head dimensions")
         max_page = -(-max_length // 128)          # the layers' MAX_PAGE (page size 128, kitty.py:43)
         self.PageTable_K = torch.full((max_batch_size, max_page), -1, dtype=torch.int64, device=dev)
         self.PageTable_V = torch.full((max_batch_size, max_page), -1, dtype=torch.int64, device=dev)

@@ -115,6 +115,9 @@ class KVCache_Layer:
         a shadow of the longest sequence: they advance by the same rules on every step, without
         reading the device, and answer ``get_total_length()`` and the capacity checks.
         """
+        if self.D != 128:
+            raise ValueError(f"device-side counters (fused append, flush and chunk kernels) are built for head_dim 128; "
+                             f"a cache with head_dim {self.D} keeps the reference's host counters")
         if seq_counts is None:
             seq_counts = torch.tensor([self.counts()] * self.MAX_BS, dtype=torch.int32)
         if tuple(seq_counts.shape) != (self.MAX_BS, _lib.SEQ_COUNT_FIELDS):

@@ -8,7 +8,10 @@ from it is copied.  Only this container has the reference mounted, so the
 vectors are committed and the tests read the ``.npz`` files, never the
 reference.
 
-    TRITON_INTERPRET=1 python tests/golden/make_quant_golden.py
+    TRITON_INTERPRET=1 python tests/golden/make_quant_golden.py [case name ...]
+
+Without names every case is written; with names only those (the cases for head dimensions 64 and 256
+were added later than the others).
 """
 import importlib.util
 import os
@@ -33,7 +36,7 @@ def load_reference():
 
 def make_inputs(case, seed):
     g = torch.Generator().manual_seed(seed)
-    B, H, T, D = case["B"], case["H"], case["T"], 128
+    B, H, T, D = case["B"], case["H"], case["T"], case.get("D", 128)
     kind = case["kind"]
     if kind == "normal_outlier":
         x = torch.randn(B, H, T, D, generator=g)
@@ -52,7 +55,7 @@ def make_inputs(case, seed):
         # any correct top-k then returns the same slot map (no ties to break)
         x = torch.randn(B, H, T, D, generator=g)
         for h in range(H):
-            mult = 1.06 ** torch.randperm(D, generator=g).float()
+            mult = 1.06 ** (torch.randperm(D, generator=g).float() * (128.0 / D))   # same spread of magnitudes for every D
             x[:, h] *= mult.view(1, 1, D)
     elif kind == "edge":
         # constant groups, tiny ranges, large magnitudes, subnormals, exact .5 ties
@@ -83,6 +86,11 @@ CASES = [
          max_page=2, page_offset=0, seed=14),
     dict(name="k_v_edge", kind="edge", B=1, H=1, T=128, t_offset=0, pages=1,
          max_page=2, page_offset=1, seed=13),
+    # other head dimensions (the reference boosts head_dim // 4 channels, kitty.py:44); tie-free scores
+    dict(name="k_v_d64", kind="spread", D=64, B=1, H=2, T=32 + 2 * 128, t_offset=32, pages=2,
+         max_page=3, page_offset=1, seed=15),
+    dict(name="k_v_d256", kind="spread", D=256, B=1, H=1, T=128, t_offset=0, pages=1,
+         max_page=2, page_offset=1, seed=16),
 ]
 
 
@@ -98,8 +106,13 @@ def tie_free(x, case, d_boost):
 
 def main():
     ref = load_reference()
-    D, PAGE, DB = 128, 128, 32
+    PAGE = 128
+    only = set(sys.argv[1:])
     for case in CASES:
+        if only and case["name"] not in only:
+            continue
+        D = case.get("D", 128)
+        DB = D // 4
         x = make_inputs(case, case["seed"])
         if case["kind"] == "spread":
             seed = case["seed"]

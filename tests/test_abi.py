@@ -59,8 +59,13 @@ def test_host_side_rejection_without_gpu(lib):
     assert lib.kitty_quant_pack_v(None, 0, 0, 0, 1, 1, 128, 128, 0, 1, 128, None, 0, 0, None, 0, None, 0, 0, None, None) == E_NULL
     assert b"NULL" in lib.kitty_last_error()
     fake = ctypes.c_void_p(4096)
-    rc = lib.kitty_quant_pack_k(fake, 256, 256, 256, 1, 1, 128, 64, 0, 1, 128, 32, None, fake, 1, 0, fake, 5248, fake, 512, 1, None, None)
-    assert rc == E_SHAPE and b"head_dim 128" in lib.kitty_last_error()
+    rc = lib.kitty_quant_pack_k(fake, 256, 256, 256, 1, 1, 128, 96, 0, 1, 128, 32, None, fake, 1, 0, fake, 5248, fake, 512, 1, None, None)
+    assert rc == E_SHAPE and b"head_dim 64, 128 or 256" in lib.kitty_last_error()
+    # head_dim 64 is served (by the plain kernels for other head dimensions): the checks go on to the strides
+    rc = lib.kitty_quant_pack_k(fake, 256, 256, 256, 1, 1, 128, 64, 0, 1, 128, 16, None, fake, 1, 0, fake, 2000, fake, 256, 1, None, None)
+    assert rc == E_RANGE and b"page stride too small" in lib.kitty_last_error()
+    rc = lib.kitty_quant_pack_k(fake, 512, 512, 512, 1, 1, 128, 256, 0, 1, 128, 256, None, fake, 1, 0, fake, 16640, fake, 1024, 1, None, None)
+    assert rc == E_SHAPE and b"uint8 slot map" in lib.kitty_last_error()
     rc = lib.kitty_quant_pack_k(fake, 32768, 32768, 256, 1, 1, 128, 128, 64, 1, 128, 32, None, fake, 1, 0, fake, 5248, fake, 512, 1, None, None)
     assert rc == E_RANGE and b"exceed" in lib.kitty_last_error()
     rc = lib.kitty_quant_pack_k(ctypes.c_void_p(4098), 32768, 32768, 256, 1, 1, 128, 128, 0, 1, 128, 32, None, fake, 1, 0, fake, 5248, fake, 512, 1, None, None)
@@ -86,7 +91,7 @@ def test_host_side_rejection_without_gpu(lib):
     assert lib.kitty_decode_attn(*args(4, fake, 1 << 20, 4)) == E_RANGE
     assert b"seqlen_K" in lib.kitty_last_error()
     L.counts[2] = 0
-    L.D = 64
+    L.D = 96
     assert lib.kitty_decode_attn(*args(4, fake, 1 << 20, 4)) == E_SHAPE
     L.D = 128
     L.cache_pages_k = -1                                                           # a negative page count
@@ -117,7 +122,9 @@ def test_host_side_rejection_without_gpu(lib):
     # the partials (max / sum pairs, then accumulator rows) and, 256-aligned, a work list of 4 + B * splits words
     assert lib.kitty_decode_attn_workspace_bytes(16, 32, 128, 16) == (
         16 * 32 * 16 * 2 * 4 + 16 * 32 * 16 * 128 * 4 + (4 + 16 * 16) * 4 + 240)
-    assert lib.kitty_decode_attn_workspace_bytes(16, 32, 64, 16) == 0
+    assert lib.kitty_decode_attn_workspace_bytes(16, 32, 96, 16) == 0
+    assert lib.kitty_decode_attn_workspace_bytes(16, 32, 64, 16) == (
+        16 * 32 * 16 * 2 * 4 + 16 * 32 * 16 * 64 * 4 + (4 + 16 * 16) * 4 + 240)
     ds = lib.kitty_decode_attn_default_splits
     assert 1 <= ds(16, 8, 257, 0) <= 257
     assert ds(1, 8, 1025, 0) > ds(16, 8, 1025, 0)

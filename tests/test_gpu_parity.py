@@ -47,7 +47,8 @@ def test_quantizer_against_reference_golden(K, path):
     B, H, _, D = x.shape
     P, t0, po = int(g["pages"]), int(g["t_offset"]), int(g["page_offset"])
     pt = K.u.to_dev(g["page_table"])
-    lay = O.Layout(H_KV=H)
+    DB = int(g["d_boost"])
+    lay = O.Layout(H_KV=H, D=D, D_BOOSTED=DB)
     gk = g["key_cache"].reshape(-1, H, lay.k_stride_h)
     sm = np.zeros((B, H, P, D), np.uint8)
     for b in range(B):
@@ -57,7 +58,7 @@ def test_quantizer_against_reference_golden(K, path):
     km = torch.zeros_like(K.u.to_dev(g["key_meta"]))
     vc = torch.zeros_like(K.u.to_dev(g["value_cache"]))
     vm = torch.zeros_like(K.u.to_dev(g["value_meta"]))
-    K.qk(x, t0, P, pt, po, kc, km, 128, 32, slot_map=K.u.to_dev(sm))
+    K.qk(x, t0, P, pt, po, kc, km, 128, DB, slot_map=K.u.to_dev(sm))
     K.qv(x, t0, P, pt, po, vc, vm, 128)
     torch.cuda.synchronize()
     assert np.array_equal(_np16(vc), g["value_cache"])
@@ -68,13 +69,16 @@ def test_quantizer_against_reference_golden(K, path):
     assert np.array_equal(ok[:, :, lay.k_off_idx:], gk[:, :, lay.k_off_idx:])
     # whole pages (high plane included) against the oracle, which stores slot s in row s
     okc, okm = np.zeros_like(g["key_cache"]), np.zeros_like(g["key_meta"])
-    O.quantize_pack_k(g["x"], t0, P, g["page_table"], po, okc, okm, 128, 32, slot_map=sm)
+    O.quantize_pack_k(g["x"], t0, P, g["page_table"], po, okc, okm, 128, DB, slot_map=sm)
     assert np.array_equal(_np16(kc), okc)
-    if "spread" in path:     # tie-free scores: the fused selection must give the reference's map
+    if any(k in path for k in ("spread", "d64", "d256")):     # tie-free scores: the fused selection must give the reference's map
         kc2, km2 = torch.zeros_like(kc), torch.zeros_like(km)
-        K.qk(x, t0, P, pt, po, kc2, km2, 128, 32)
+        K.qk(x, t0, P, pt, po, kc2, km2, 128, DB)
         torch.cuda.synchronize()
         assert np.array_equal(_np16(kc2), okc)
+        smd = K.sel(x, t0, P, 128, DB)
+        torch.cuda.synchronize()
+        assert np.array_equal(_np16(smd), sm)
 
 
 @pytest.mark.parametrize("student_t", [False, True])

@@ -29,7 +29,9 @@ def _slot_maps(g, lay):
 
 
 def test_golden_files_present():
-    assert len(GOLDEN) == 4
+    assert len(GOLDEN) == 6
+    dims = sorted(int(np.load(p)["x"].shape[-1]) for p in GOLDEN)
+    assert dims == [64, 128, 128, 128, 128, 256]     # head dimensions 64 and 256 boost 16 and 64 channels
 
 
 @pytest.mark.parametrize("path", GOLDEN, ids=[os.path.basename(p) for p in GOLDEN])
@@ -38,11 +40,13 @@ def test_quantizer_matches_reference_output(path):
     x = g["x"]
     B, H, _, D = x.shape
     P, t0, po, pt = int(g["pages"]), int(g["t_offset"]), int(g["page_offset"]), g["page_table"]
-    lay = O.Layout(H_KV=H)
+    DB = int(g["d_boost"])
+    assert DB == D // 4
+    lay = O.Layout(H_KV=H, D=D, D_BOOSTED=DB)
     sm = _slot_maps(g, lay)
     kc, km = np.zeros_like(g["key_cache"]), np.zeros_like(g["key_meta"])
     vc, vm = np.zeros_like(g["value_cache"]), np.zeros_like(g["value_meta"])
-    O.quantize_pack_k(x, t0, P, pt, po, kc, km, 128, 32, slot_map=sm)
+    O.quantize_pack_k(x, t0, P, pt, po, kc, km, 128, DB, slot_map=sm)
     O.quantize_pack_v(x, t0, P, pt, po, vc, vm, 128)
     # V: bytes and metadata bit-exact, including untouched pages (zeros)
     assert np.array_equal(vc, g["value_cache"])
@@ -57,36 +61,41 @@ def test_quantizer_matches_reference_output(path):
     # arithmetic (kitty_quant_pack.py:140), so slot s lands in row s % 8 and four boosted
     # channels collide per row; the CPU interpreter keeps the last writer (largest channel).
     # This build stores slot s in row s.  What the reference kept must equal our row of the
-    # winning slot, and its rows 8..31 were never written.
+    # winning slot, and its rows 8 .. d_boost - 1 were never written (the same wrap for 16 and 64 slots).
     for b in range(B):
         for p in range(P):
             pg = pt[b, po + p]
             for h in range(H):
-                ghi = gk[pg, h, lay.k_off_hi: lay.k_off_idx].reshape(32, 32)
-                ohi = ok[pg, h, lay.k_off_hi: lay.k_off_idx].reshape(32, 32)
+                ghi = gk[pg, h, lay.k_off_hi: lay.k_off_idx].reshape(DB, 32)
+                ohi = ok[pg, h, lay.k_off_hi: lay.k_off_idx].reshape(DB, 32)
                 assert not ghi[8:].any()
                 idx = sm[b, h, p]
                 for r in range(8):
-                    chans = [d for d in range(D) if idx[d] < 32 and idx[d] % 8 == r]
+                    chans = [d for d in range(D) if idx[d] < DB and idx[d] % 8 == r]
                     winner = idx[max(chans)]
                     assert np.array_equal(ghi[r], ohi[winner]), (b, p, h, r)
 
 
-def test_selection_matches_reference_when_tie_free():
-    g = np.load([p for p in GOLDEN if "spread" in p][0])
+TIE_FREE = [p for p in GOLDEN if any(k in p for k in ("spread", "d64", "d256"))]
+
+
+@pytest.mark.parametrize("path", TIE_FREE, ids=[os.path.basename(p) for p in TIE_FREE])
+def test_selection_matches_reference_when_tie_free(path):
+    g = np.load(path)
     x = g["x"]
     B, H, _, D = x.shape
-    lay = O.Layout(H_KV=H)
+    DB, t0 = int(g["d_boost"]), int(g["t_offset"])
+    lay = O.Layout(H_KV=H, D=D, D_BOOSTED=DB)
     sm = _slot_maps(g, lay)
     n = 0
     for b in range(B):
         for p in range(int(g["pages"])):
             for h in range(H):
-                xx = x[b, h, p * 128:(p + 1) * 128]
-                assert O.boost_is_tie_free(xx, 32)
-                assert np.array_equal(O.select_boost(xx, 32), sm[b, h, p])
+                xx = x[b, h, t0 + p * 128: t0 + (p + 1) * 128]
+                assert O.boost_is_tie_free(xx, DB)
+                assert np.array_equal(O.select_boost(xx, DB), sm[b, h, p])
                 n += 1
-    assert n == 4
+    assert n == B * H * int(g["pages"]) >= 1
 
 
 def test_selection_same_scores_on_tied_pages():
@@ -96,7 +105,8 @@ def test_selection_same_scores_on_tied_pages():
         g = np.load(path)
         x = g["x"]
         B, H, _, D = x.shape
-        lay = O.Layout(H_KV=H)
+        DB = int(g["d_boost"])
+        lay = O.Layout(H_KV=H, D=D, D_BOOSTED=DB)
         sm = _slot_maps(g, lay)
         t0 = int(g["t_offset"])
         for b in range(B):
@@ -104,11 +114,11 @@ def test_selection_same_scores_on_tied_pages():
                 for h in range(H):
                     xx = x[b, h, t0 + p * 128: t0 + (p + 1) * 128]
                     sc = O.boost_score(xx).astype(np.float64)
-                    ref_sorted = np.sort(sc[sm[b, h, p] < 32])[::-1]
-                    ours_sorted = np.sort(sc)[::-1][:32]
+                    ref_sorted = np.sort(sc[sm[b, h, p] < DB])[::-1]
+                    ours_sorted = np.sort(sc)[::-1][:DB]
                     assert np.array_equal(ref_sorted, ours_sorted)
                     # the reference's slot order is descending in score as well
-                    by_slot = sc[np.argsort(np.where(sm[b, h, p] < 32, sm[b, h, p], 255))[:32]]
+                    by_slot = sc[np.argsort(np.where(sm[b, h, p] < DB, sm[b, h, p], 255))[:DB]]
                     assert np.all(np.diff(by_slot) <= 0)
 
 
