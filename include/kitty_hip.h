@@ -12,6 +12,11 @@
  *
  * Each function names the reference interface it replaces (paths relative to the reference
  * checkout, src/kitty/kvcache/...).
+ *
+ * Head dimensions: D = 128 runs on the tuned kernels; D = 64 and D = 256 are served by plain kernels
+ * with the same arithmetic and storage format (the reference's kernels take D as a parameter,
+ * kernels/kitty_quant_pack.py:42-45, kernels/kitty_attention.py:59-62); any other D is KITTY_E_SHAPE.
+ * PAGE_SIZE is 128.
  */
 #ifndef KITTY_HIP_H
 #define KITTY_HIP_H
@@ -156,7 +161,7 @@ int kitty_quant_pack_v(const void* value, int64_t stride_b, int64_t stride_h, in
  * num_splits <= 0 picks kitty_decode_attn_default_splits() (max_tiles = 1 + the 128-token tiles
  * after the sink of the longest sequence; per_sequence_counts = layer->seq_counts is set).
  * variant: 0 = default kernel, 1 = the plain reference-order kernel (fp16 dequantization, no
- * matrix cores).
+ * matrix cores).  For D = 64 / 256 both values run the same plain kernel.
  */
 size_t kitty_decode_attn_workspace_bytes(int B, int H_Q, int D, int num_splits);
 int kitty_decode_attn_default_splits(int B, int H_KV, int max_tiles, int per_sequence_counts);
@@ -251,6 +256,8 @@ int kitty_prefill_attn(const kitty_kv_layer* layer,
  * rotation and the kernel stores k * cos + rotate_half(k) * sin, each product and the sum rounded
  * to fp16, which is what the caller's own fp16 tensor expression computes
  * (modeling_qwen3.py:215-220 feeding kitty.py:102-123): one launch less and no rotated copy of K.
+ *
+ * These three entry points are built for D = 128 (KITTY_E_SHAPE otherwise).
  *
  * kitty_flush_full: every sequence whose K (V) Q-buffer holds PAGE_SIZE rows gets it quantized,
  * with channel selection, into page page_table[b][PageCount] and its counters advanced; the

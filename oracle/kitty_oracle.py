@@ -18,8 +18,9 @@ How each function is pinned (what a wrong restatement would fail):
 * ``quantize_group`` / ``pack_k_page`` / ``pack_v_page`` / ``quantize_pack_k`` /
   ``quantize_pack_v``: golden vectors under ``tests/golden/quant_*.npz`` produced
   by the reference's own ``quantize_pack_k/v`` run through Triton's CPU
-  interpreter (script ``tests/golden/make_quant_golden.py``), plus closed-form
-  known-answer bytes and a scalar brute-force loop.
+  interpreter (script ``tests/golden/make_quant_golden.py``; head dimension 128
+  with 32 boosted channels in four cases, 64 with 16 and 256 with 64 in one each),
+  plus closed-form known-answer bytes and a scalar brute-force loop.
 * ``select_boost``: the score is pinned by the golden slot maps wherever the
   reference's scores are tie-free; the tie rule (descending score, then
   ascending channel) is this build's canonical choice because ``torch.topk``
