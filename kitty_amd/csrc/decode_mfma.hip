@@ -1056,6 +1056,18 @@ __device__ __forceinline__ void wave_work(const kitty_kv_layer& L, const __half*
   x.lane = threadIdx.x;
   x.kg = x.lane >> 4;
   x.n = x.lane & 15;
+  // A body wave's start is a chain of round trips: counters, query rows, page ids, first tiles.  The
+  // query rows of a quarter-column body wave do not go through registers the compiler waits for: ONE
+  // global -> LDS load (the four heads' rows, 1 KB, into the space of the q * scale table, which is
+  // first written by the first page) is asked for before anything else and waited for by count after
+  // the first tiles have been asked for, so that its latency lies under theirs.
+  constexpr bool Q_VIA_LDS = QUARTER && MODE == kWaveBody;
+  if constexpr (Q_VIA_LDS) {
+    const int Gq = H_Q / L.H_KV;
+    const uint8_t* qbase = (const uint8_t*)(q + ((int64_t)x.b * H_Q + (int64_t)x.h * Gq) * kD);
+    lds_dma<1, 16>((uint32_t)(min(x.lane >> 4, Gq - 1) * (kD * 2) + (x.lane & 15) * 16), qbase,
+                   (uint32_t)(uintptr_t)&S.qs[0][0]);   // row r of the table's space: head min(r, G - 1)
+  }
   x.c = load_counts(L, x.b);
   x.lane_off = (4 * x.kg + (x.n & 1)) * kRowBytes + (x.n >> 1) * 4;
   x.sel = (x.n & 1) ? 0x03020706u : 0x05040100u;
@@ -1083,10 +1095,12 @@ __device__ __forceinline__ void wave_work(const kitty_kv_layer& L, const __half*
 
   // q of this column: operand-order pairs in registers, natural order in LDS for the slot gather
   const __half* qrow = q + ((int64_t)x.b * H_Q + (int64_t)x.h * G + x.g) * kD;
+  if constexpr (!Q_VIA_LDS) {
 #pragma unroll
-  for (int kc = 0; kc < 4; ++kc)
+    for (int kc = 0; kc < 4; ++kc)
 #pragma unroll
-    for (int pi = 0; pi < 4; ++pi) x.qpair[kc * 4 + pi] = *(const uint32_t*)(qrow + 32 * kc + krow(pi, x.kg));
+      for (int pi = 0; pi < 4; ++pi) x.qpair[kc * 4 + pi] = *(const uint32_t*)(qrow + 32 * kc + krow(pi, x.kg));
+  }
   // the tables of the generic QK / PV path: q in natural order for the slot gather, a zero entry
   // for "no channel", a row of ones
   auto stage_generic_tables = [&]() {
@@ -1106,9 +1120,11 @@ __device__ __forceinline__ void wave_work(const kitty_kv_layer& L, const __half*
 #pragma unroll
     for (int t = 0; t < 4; ++t) S.vs_q[t][x.lane] = 0u;
     if (x.lane < 4) S.ones4[x.lane] = 0x3C003C00u;
+    if constexpr (!Q_VIA_LDS) {
 #pragma unroll
-    for (int r = 0; r < 4; ++r)
-      x.q4[r] = *(const uint32_t*)(q + ((int64_t)x.b * H_Q + (int64_t)x.h * G + min(r, G - 1)) * kD + 2 * x.lane);
+      for (int r = 0; r < 4; ++r)
+        x.q4[r] = *(const uint32_t*)(q + ((int64_t)x.b * H_Q + (int64_t)x.h * G + min(r, G - 1)) * kD + 2 * x.lane);
+    }
     const int row = x.g + (x.lo_part ? 4 : 0);
     x.qs_rd = row * (kQsPitch * 4) + 8 * x.kg;
     x.qb_rd = row * 64 + 8 * x.kg;
@@ -1173,13 +1189,26 @@ __device__ __forceinline__ void wave_work(const kitty_kv_layer& L, const __half*
     // count the instructions issued AFTER the tile that is needed; nothing is loaded past the end
     // of the range (the last two iterations wait on shorter queues).
     if (t0 < t1) {
-      settle_prologue_loads();
+      if constexpr (!Q_VIA_LDS) settle_prologue_loads();   // (else: no load of the prologue fills a register the loop reads)
       constexpr int nK = kDmaK<BOOST>;
       const uint32_t lk0 = (uint32_t)(uintptr_t)&S.kbuf[0][0], lk1 = (uint32_t)(uintptr_t)&S.kbuf[1][0];
       const uint32_t lv = (uint32_t)(uintptr_t)&S.vbuf[0];
       dma_k<BOOST>(x, t0, lk0);
       if (t0 + 1 < t1) dma_k<BOOST>(x, t0 + 1, lk1);
       dma_v(x, t0, lv);
+      if constexpr (Q_VIA_LDS) {
+        // the query rows were asked for before these tiles: everything older than the tiles has landed
+        if (t0 + 1 < t1) wait_vmcnt<2 * nK + kDmaV>(); else wait_vmcnt<nK + kDmaV>();
+        const _Float16* ql = (const _Float16*)&S.qs[0][0];
+#pragma unroll
+        for (int kc = 0; kc < 4; ++kc)
+#pragma unroll
+          for (int pi = 0; pi < 4; ++pi)
+            x.qpair[kc * 4 + pi] = *(const uint32_t*)(ql + (x.n & 3) * kD + 32 * kc + krow(pi, x.kg));
+#pragma unroll
+        for (int r = 0; r < 4; ++r) x.q4[r] = *(const uint32_t*)(ql + r * kD + 2 * x.lane);
+        wave_lds_fence();   // (the table's first write comes after these reads: LDS executes a wave's instructions in order)
+      }
       // Of the two waves that share a SIMD the older one wins arbitration, and it is 8 % faster per
       // tile.  When the launch is a single round (at most two workgroups per SIMD of the device),
       // the workgroups dispatched after every SIMD has one are the younger ones: they raise their
