@@ -145,11 +145,12 @@ def test_group_sizes_and_split_counts(K, D, G):
 
 
 @pytest.mark.parametrize("D", DIMS)
-@pytest.mark.parametrize("T0", [0, 20, 32 + 128 + 50])
-def test_chunked_prefill_attention(K, D, T0):
+@pytest.mark.parametrize("T0,G", [(0, 4), (20, 4), (32 + 128 + 50, 4), (32 + 128 + 50, 3), (32 + 128 + 50, 16), (200, 1)])
+def test_chunked_prefill_attention(K, D, T0, G):
     """A chunk of new tokens over an empty layer (plain causal attention), a sink-only layer and a layer with
     packed pages, against the oracle's chunk attention; then the chunk is appended and the layer compared."""
-    B, H_KV, H_Q, Tq = 1, 2, 8, 37
+    B, H_KV, Tq = 1, 2, 37
+    H_Q = H_KV * G
     k, v = make_kv(B, H_KV, T0 + Tq, D=D, seed=41 + D + T0)
     cache = K.KittyCache(K.u.cfg(H_KV, H_Q, D=D), B, 1024)
     ol = O.OracleLayer(B, 1024, H_KV, D=D, D_BOOSTED=D // 4)

@@ -6,10 +6,10 @@ import torch
 transformers = pytest.importorskip("transformers")
 
 
-def _tiny_llama(attn):
+def _tiny_llama(attn, head_dim=128):
     from transformers import LlamaConfig, LlamaForCausalLM
     cfg = LlamaConfig(vocab_size=256, hidden_size=256, intermediate_size=512, num_hidden_layers=2,
-                      num_attention_heads=2, num_key_value_heads=1, head_dim=128, max_position_embeddings=4096,
+                      num_attention_heads=2, num_key_value_heads=1, head_dim=head_dim, max_position_embeddings=4096,
                       attn_implementation=attn)
     torch.manual_seed(0)
     return LlamaForCausalLM(cfg)
@@ -317,3 +317,45 @@ def test_stock_llama_on_the_paged_cache():
         decode(40)
     paged.check_tables()
     assert paged.active_slots() == [1, 2] and list(paged.seq_lengths()) == [0, 297 + 40, 45 + 110]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("head_dim", [64, 256])
+def test_stock_llama_with_another_head_dimension(head_dim):
+    """The reference takes ``config.head_dim`` (kitty.py:39-44); head dimensions 64 and 256 go through the
+    same hook onto the kernels for other head dimensions.  While everything is fp16 (80 tokens) the logits
+    agree with torch's dense attention; a longer ``generate()`` crosses prefill quantization and both
+    flushes and leaves the counters the state machine predicts."""
+    if not torch.cuda.is_available():
+        pytest.skip("needs a GPU")
+    from transformers import DynamicCache
+    from kitty_amd import hf
+    hf.register()
+    dev = torch.device("cuda")
+    ref = _tiny_llama("sdpa", head_dim).to(dev).half().eval()
+    mod = _tiny_llama("kitty", head_dim).to(dev).half().eval()
+    mod.load_state_dict(ref.state_dict())
+    B, T0, steps = 2, 20, 60
+    ids = torch.randint(0, 256, (B, T0), generator=torch.Generator().manual_seed(3)).to(dev)
+    c_ref, c_mod = DynamicCache(), hf.KittyHFCache(mod.config, B, 1024, device=dev)
+    assert c_mod.kv_cache[0].D == head_dim and c_mod.kv_cache[0].D_BOOSTED == head_dim // 4
+    with torch.no_grad():
+        cur = ids
+        for s in range(steps + 1):
+            a = ref(input_ids=cur, past_key_values=c_ref, use_cache=True).logits[:, -1].float()
+            b = mod(input_ids=cur, past_key_values=c_mod, use_cache=True).logits[:, -1].float()
+            assert torch.isfinite(b).all()
+            assert (a - b).abs().max().item() <= 3e-2, (s, (a - b).abs().max().item())
+            cur = a.argmax(-1, keepdim=True)
+    T1, new = 32 + 128 + 100, 170
+    ids = torch.randint(0, 256, (B, T1), generator=torch.Generator().manual_seed(4)).to(dev)
+    with torch.no_grad():
+        cache = hf.KittyHFCache(mod.config, B, 1024, device=dev)
+        got = mod.generate(ids, past_key_values=cache, max_new_tokens=new, do_sample=False, pad_token_id=0,
+                           eos_token_id=None)
+    assert tuple(got.shape) == (B, T1 + new) and torch.equal(got[:, :T1], ids)
+    n = T1 + new - 1 - 32
+    for L in cache.kv_cache:
+        assert (L.Sink_Count, L.PageCount_K, L.Q_Buffer_Count_K) == (32, n // 128, n % 128)
+        assert (L.PageCount_V, L.Q_Buffer_Count_V, L.Local_Count_V) == ((n - 128) // 128, (n - 128) % 128, 128)
+    cache.check_status()
