@@ -109,9 +109,12 @@ def synth_kv(B, H, T, D, seed, device, student_t=False):
 def algorithmic_bytes(B, H_Q, H_KV, layer):
     """Bytes one decode step has to move: packed pages + metadata + fp16 windows + Q and O."""
     pk, pv = layer.PageCount_K, layer.PageCount_V
-    per_head_packed = 5760 * pk + 4608 * pv
-    per_head_fp16 = 256 * (2 * layer.Sink_Count + layer.Q_Buffer_Count_K + layer.Q_Buffer_Count_V + layer.Local_Count_V)
-    qo = 2 * H_Q * 128 * 2
+    D, DB = layer.D, layer.D_BOOSTED
+    k_page = 32 * (D + DB) + D + 4 * D          # planes, slot map, (scale, zero) pairs: 5760 at D = 128
+    v_page = 32 * D + 512                       # codes, (scale, zero) pairs: 4608 at D = 128
+    per_head_packed = k_page * pk + v_page * pv
+    per_head_fp16 = 2 * D * (2 * layer.Sink_Count + layer.Q_Buffer_Count_K + layer.Q_Buffer_Count_V + layer.Local_Count_V)
+    qo = 2 * H_Q * D * 2
     return B * (H_KV * (per_head_packed + per_head_fp16) + qo), B * H_KV * per_head_packed
 
 
@@ -540,7 +543,11 @@ class DecodeBench:
         self.workload, self.variant = workload, variant
         B, H_Q, H_KV, T, self.desc = WORKLOADS[workload]
         self.B, self.H_Q, self.H_KV, self.T = B, H_Q, H_KV, T
-        D = self.D = 128
+        D = self.D = getattr(args, "head_dim", 128)
+        if D != 128:
+            self.desc = self.desc.replace("D=128", f"D={D}") + " - the plain kernels for other head dimensions"
+            if workload == "c2":
+                raise ValueError("per-sequence counters on the device (c2) are built for head_dim 128")
         cfg = types.SimpleNamespace(num_hidden_layers=1, head_dim=D, num_key_value_heads=H_KV,
                                     num_attention_heads=H_Q, hidden_size=H_Q * D)
         max_len = T + 256
@@ -596,6 +603,7 @@ class DecodeBench:
         L0 = self.L0 = probe.kv_cache[0]
         self.quant_ms = min(quant_ms)
         self.quant_in_bytes = 2 * B * H_KV * (L0.PageCount_K + L0.PageCount_V) * 128 * D
+        self.quant_kernels = self.quantizer_kernels(K, V, L0)
         self.q = torch.randn((B, H_Q, 1, D), generator=torch.Generator(device=dev).manual_seed(7), device=dev,
                              dtype=torch.float32).half()
         self.out = torch.empty((B, 1, H_Q, D), dtype=torch.float16, device=dev)
@@ -611,6 +619,38 @@ class DecodeBench:
         self.stream = torch.cuda.current_stream(dev).cuda_stream
         self.scaling = D ** -0.5
         self.hip = HipEvents()
+
+    def quantizer_kernels(self, K, V, L, rounds=40):
+        """The K and the V quantizer alone, each launched `rounds` times back to back over the first
+        cache's own pages (same input, so the same bytes again) with an event pair around every launch:
+        the median of the second half is the level the kernel holds; a launch after a synchronisation
+        (as `ms` of the whole call is timed) starts on an idle device."""
+        torch = self.torch
+        from kitty_amd.kvcache.kernels import quantize_pack_k, quantize_pack_v
+        P, S, out = L.PAGE_SIZE, L.Sink_Count, {}
+        calls = {"k": lambda: quantize_pack_k(K, S, L.PageCount_K, L.PageTable_K, 0, L.KeyCache, L.KeyCache_metadata,
+                                              P, L.D_BOOSTED),
+                 "v": lambda: quantize_pack_v(V, S, L.PageCount_V, L.PageTable_V, 0, L.ValueCache,
+                                              L.ValueCache_metadata, P)}
+        for name, call in calls.items():
+            pages = L.PageCount_K if name == "k" else L.PageCount_V
+            if pages == 0:
+                continue
+            ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(rounds)]
+            for a, b in ev:
+                a.record()
+                call()
+                b.record()
+            torch.cuda.synchronize()
+            us = sorted(a.elapsed_time(b) * 1e3 for a, b in ev[rounds // 2:])
+            head = self.B * self.H_KV * pages
+            in_bytes = head * P * self.D * 2
+            out_bytes = head * ((32 * (self.D + L.D_BOOSTED) + self.D + 4 * self.D) if name == "k" else (32 * self.D + 512))
+            med = us[len(us) // 2]
+            out[name] = {"median_us": med, "min_us": us[0], "gbps_in": in_bytes / med / 1e3,
+                         "hbm_frac": (in_bytes + out_bytes) / med / 1e3 / HBM_PEAK_GBPS,
+                         "bytes_in": in_bytes, "bytes_out": out_bytes, "launches": rounds}
+        return out
 
     def step(self, i, ev=None, variant=None):
         lib, _lib = self.lib, self._lib
@@ -750,7 +790,9 @@ class DecodeBench:
             },
             "quantizer": {"gbps_in": self.quant_in_bytes / (self.quant_ms * 1e-3) / 1e9, "ms": self.quant_ms,
                           "input_bytes": self.quant_in_bytes,
-                          "what": "quantize_prefill of the whole context (K select+quantize+pack, V quantize+pack)"},
+                          "what": "quantize_prefill of the whole context (K select+quantize+pack, V quantize+pack) "
+                                  "after a synchronisation; `kernels`: each kernel alone, launched back to back",
+                          "kernels": self.quant_kernels},
         }
 
 
@@ -770,7 +812,7 @@ def other_workloads(headline, args):
         gc.collect()
         torch.cuda.empty_cache()
 
-    side = types.SimpleNamespace(copies=0, splits=0, scatter_pages=False)
+    side = types.SimpleNamespace(copies=0, splits=0, scatter_pages=False, head_dim=128)
     guarded("c1_variant1", lambda: headline.summary(10, 3, variant=1, max_windows=4))
     for name in ("c0", "c2", "c4"):
         guarded(name, lambda name=name: DecodeBench(name, 0, side).summary(40, 5))
@@ -805,6 +847,8 @@ def main():
     ap.add_argument("--copies", type=int, default=0, help="independent cache copies to rotate over (0 = auto)")
     ap.add_argument("--splits", type=int, default=0)
     ap.add_argument("--variant", type=int, default=0)
+    ap.add_argument("--head-dim", type=int, default=128, choices=[64, 128, 256],
+                    help="c0 / c1 / c4 with another head dimension (the untuned kernels for 64 and 256)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-other-workloads", action="store_true",
                     help="default workload only: leave out the `workloads` key (configs[0], [2], [3], [4], the plain "
@@ -831,6 +875,9 @@ def main():
     lib_check()
     headline = DecodeBench(args.workload, args.variant, args)
     result = headline.headline(args)
+    if args.head_dim != 128:     # a side measurement of the plain kernels: neither the host baseline nor the other configs
+        args.no_cpu_baseline = args.no_other_workloads = True
+        result["roofline"]["traffic"] = None
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(headline.K.cpu(), headline.V.cpu(), headline.q.cpu(), headline.H_Q,
                                               headline.H_KV)

@@ -36,46 +36,89 @@ __device__ __forceinline__ uint4 nt_load16(const uint8_t* p) {
   return uint4{v.x, v.y, v.z, v.w};
 }
 
-// The same codes for N values of one group at a time, mostly without the division:
-//   t = fma(x, r, c0),  c0 = fma(-min, r, 0.5),  r = the refined reciprocal of the scale.
-// Against the reference's fl(fl((x - min) / scale) + 0.5) this differs by the roundings of x - min,
-// of the quotient and of the sum (1e-6 each for quotients below 16.5), the reciprocal's last bit
-// (2e-6), the rounding of c0 (1.9e-6 while |min * r| <= 32) and its own (1e-6): under 8e-6.  So
-// unless t lies within 2^-16 of an integer, floor(t) is the reference's code; the reference's upper
-// clamp never changes a floor for finite inputs (the largest quotient is qmax * (1 + 2^-24)).  If any
-// lane of the wave has such a t among its N, or a group whose c0 is NaN (fast_offset returns that
-// when |min * r| > 32 or the scale is not finite), the wave redoes these N values with the exact
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+// Half `hi` (0 / 1) of a word of two fp16 numbers, as the compiler's half type: widened where it is used,
+// it enters a mixed-precision FMA as it is (exactly, subnormals included) and costs no conversion.
+__device__ __forceinline__ _Float16 half_of(uint32_t w, int hi) {
+  const half2_t p = __builtin_bit_cast(half2_t, w);
+  return hi ? p.y : p.x;
+}
+// Packed fp16 minimum / maximum of two words.  Written out because the compiler first re-quiets every
+// operand it has not produced itself (one more instruction per loaded word); fp16 numbers order as
+// their fp32 values do, and a quiet NaN loses against a number as in fminf / fmaxf.
+__device__ __forceinline__ uint32_t pk_min_f16(uint32_t a, uint32_t b) {
+  uint32_t d;
+  asm("v_pk_min_f16 %0, %1, %2" : "=v"(d) : "v"(a), "v"(b));
+  return d;
+}
+__device__ __forceinline__ uint32_t pk_max_f16(uint32_t a, uint32_t b) {
+  uint32_t d;
+  asm("v_pk_max_f16 %0, %1, %2" : "=v"(d) : "v"(a), "v"(b));
+  return d;
+}
+
+// |a| + |b| in fp32 and a widened to fp32, for half `hi` of the words a and b: one mixed-precision FMA
+// each, which widens its fp16 operands exactly (subnormals included) on the way in.  (x + -0 = x for
+// every x, -0 included.)
+__device__ __forceinline__ float abs_sum_f16(uint32_t a, uint32_t b, int hi) {
+  float d;
+  if (hi) asm("v_fma_mix_f32 %0, |%1|, 1.0, |%2| op_sel:[1,0,1] op_sel_hi:[1,0,1]" : "=v"(d) : "v"(a), "v"(b));
+  else asm("v_fma_mix_f32 %0, |%1|, 1.0, |%2| op_sel:[0,0,0] op_sel_hi:[1,0,1]" : "=v"(d) : "v"(a), "v"(b));
+  return d;
+}
+__device__ __forceinline__ float widen_f16(uint32_t a, int hi) {
+  float d;
+  const float neg_zero = -0.0f;
+  if (hi) asm("v_fma_mix_f32 %0, %1, 1.0, %2 op_sel:[1,0,0] op_sel_hi:[1,0,0]" : "=v"(d) : "v"(a), "s"(neg_zero));
+  else asm("v_fma_mix_f32 %0, %1, 1.0, %2 op_sel:[0,0,0] op_sel_hi:[1,0,0]" : "=v"(d) : "v"(a), "s"(neg_zero));
+  return d;
+}
+
+// The codes of the 8 values of one group (half `hi` of the words w[0..7]) as bytes of two words,
+// mostly without the division.  The reference floors T = fl(fl(fl(x - min) / scale) + 0.5).  Here
+//   a = fma(x, r, cA),  b = fma(x, r, cB),  cA = fma(-min, r, -2^-16),  cB = fma(-min, r, +2^-16),
+// r = the refined reciprocal of the scale.  Against T - 0.5 -+ 2^-16 these differ by the reference's
+// roundings of x - min, of the quotient and of the sum (1e-6 each for quotients below 16.5), the
+// reciprocal's last bit (2e-6), the rounding of cA / cB (1.9e-6 while |min * r| <= 32) and their own
+// (1e-6): under 8e-6, so a < T - 0.5 < b.  v_cvt_pk_u8_f32 rounds to the nearest integer (ties to even)
+// and saturates at 0 and 255.  If it gives the same integer n for a and for b, then n - 0.5 <= a and
+// b <= n + 0.5, hence n < T < n + 1: n is the reference's code (its upper clamp never changes a floor
+// for finite inputs: the largest quotient is qmax * (1 + 2^-24)).  If the two differ for any of a
+// lane's 8 values in any lane of the wave, or the group's offsets are NaN (fast_offsets returns that
+// when |min * r| > 32 or the scale is not finite), the wave redoes these 8 values with the exact
 // division: about one group in seventy on gaussian data.
-__device__ __forceinline__ float fast_offset(float mn, Divisor k) {
-  const float c0 = __builtin_fmaf(-mn, k.r, 0.5f);
-  return (fabsf(mn * k.r) <= 32.0f && k.d < 3.0e38f) ? c0 : __builtin_nanf("");
-}
-template <int N>
-__device__ __forceinline__ void codes_of(const float (&x)[N], float mn, float c0, Divisor k, float qlim, float (&c)[N]) {
-  float fmn = 1.0f, fmx = 0.0f;
-#pragma unroll
-  for (int r = 0; r < N; ++r) {
-    const float t = __builtin_fmaf(x[r], k.r, c0);
-    c[r] = __builtin_floorf(t);
-    const float f = t - c[r];
-    fmn = fminf(fmn, f);
-    fmx = fmaxf(fmx, f);
-  }
+__device__ __forceinline__ float2 fast_offsets(float mn, Divisor k) {
   constexpr float kEps = 1.52587890625e-05f;   // 2^-16
-  // (min / max skip NaNs, so the group's NaN offset is tested by itself)
-  if (__any(!(c0 == c0 && fmn >= kEps && fmx <= 1.0f - kEps))) {
-#pragma unroll
-    for (int r = 0; r < N; ++r) c[r] = code_of(x[r] - mn, k, qlim);
-  }
+  const float nan = __builtin_nanf("");
+  const bool ok = fabsf(mn * k.r) <= 32.0f && k.d < 3.0e38f;
+  return ok ? float2{__builtin_fmaf(-mn, k.r, -kEps), __builtin_fmaf(-mn, k.r, kEps)} : float2{nan, nan};
 }
-// Bits {1,0} (SHIFT = 0) or {3,2} (SHIFT = 2) of the 8 nibbles of n, packed into 16 bits.
+__device__ __forceinline__ void codes_of(const uint32_t (&w)[8], int hi, float mn, float2 cab, Divisor k, float qlim,
+                                         uint32_t& c0123, uint32_t& c4567) {
+  uint32_t a[2] = {0, 0}, b[2] = {0, 0};
+#pragma unroll
+  for (int r = 0; r < 8; ++r) {
+    const float x = (float)half_of(w[r], hi);
+    a[r >> 2] = __builtin_amdgcn_cvt_pk_u8_f32(__builtin_fmaf(x, k.r, cab.x), r & 3, a[r >> 2]);
+    b[r >> 2] = __builtin_amdgcn_cvt_pk_u8_f32(__builtin_fmaf(x, k.r, cab.y), r & 3, b[r >> 2]);
+  }
+  if (__any(!(cab.x == cab.x) || a[0] != b[0] || a[1] != b[1])) {
+    a[0] = a[1] = 0;
+#pragma unroll
+    for (int r = 0; r < 8; ++r)
+      a[r >> 2] = __builtin_amdgcn_cvt_pk_u8_f32(code_of((float)half_of(w[r], hi) - mn, k, qlim), r & 3, a[r >> 2]);
+  }
+  c0123 = a[0];
+  c4567 = a[1];
+}
+// Bits {1,0} (SHIFT = 0) or {3,2} (SHIFT = 2) of the 8 code bytes of (c0123, c4567), packed into 16
+// bits: a dot product of the four masked bytes with (1, 4, 16, 64) lines their fields up.
 template <int SHIFT>
-__device__ __forceinline__ uint32_t gather_fields(uint32_t n) {
-  uint32_t x = SHIFT ? (n >> SHIFT) : n;
-  x = ((x >> 2) & 0x0C0C0C0Cu) | (x & ~0x0C0C0C0Cu);   // nibble pairs -> low nibble of each byte
-  x = ((x >> 4) & 0x00F000F0u) | (x & ~0x00F000F0u);   // byte pairs -> low byte of each half
-  x = ((x >> 8) & 0x0000FF00u) | (x & ~0x0000FF00u);   // halves -> low half
-  return x & 0xffffu;
+__device__ __forceinline__ uint32_t gather_fields(uint32_t c0123, uint32_t c4567) {
+  constexpr uint32_t kMask = 0x03030303u << SHIFT, kWeights = 0x40100401u;
+  const uint32_t lo = __builtin_amdgcn_udot4(c0123 & kMask, kWeights, 0u, false);
+  const uint32_t hi = __builtin_amdgcn_udot4(c4567 & kMask, kWeights, 0u, false);
+  return ((hi << 8) + lo) >> SHIFT;
 }
 
 // One K page of one head.  MODE 0: slot map given.  MODE 1: selection fused, then quantize.
@@ -86,6 +129,10 @@ struct StridedRows {   // the rows of a page that lies in one tensor
   const uint8_t* base;
   int64_t stride_t;
   __device__ __forceinline__ const uint8_t* operator()(int t) const { return base + (int64_t)t * stride_t; }
+  // row t0 + r, r a constant: the product with the lane's t0 is formed once for all r
+  __device__ __forceinline__ const uint8_t* operator()(int t0, int r) const {
+    return base + (int64_t)t0 * stride_t + (int64_t)r * stride_t;
+  }
 };
 template <int MODE, class ROWS>
 __device__ __forceinline__ void quant_k_page(const ROWS row_of, int d_boost,
@@ -98,49 +145,77 @@ __device__ __forceinline__ void quant_k_page(const ROWS row_of, int d_boost,
   // LDS layouts are chosen so that the 64 lanes of an access fall on 64 different banks.  Per-channel
   // tables are indexed by pos(channel) = (channel % 8) * 16 + channel / 8: the 16 lanes that share a
   // token group work on channels 8 apart and so read / write consecutive entries.  Rows of partials
-  // (one per token group) are 144 entries apart, which moves each of the four token groups of a
-  // wave to its own quarter (floats) or half (doubles, two passes) of the banks.
-  constexpr int kPitch = kD + 16;
-  __shared__ __attribute__((aligned(16))) float s_pmin[16][kPitch];   // later: the low plane on its way out
-  __shared__ float s_pmax[16][kPitch];
-  __shared__ float s_psum[MODE == 0 ? 1 : 16][kPitch];
-  __shared__ unsigned long long s_exact[MODE == 0 ? 1 : kD];   // [pos]: exact sum of |x| * 2^24 where fp32 leaves a doubt
+  // are 80 words (minima / maxima: one per token group, a word of two fp16 channels) or 144 floats
+  // (sums: one per pair of token groups) apart, which moves each of the four token groups of a wave to
+  // its own quarter of the banks.  All of it stays under 20 KB, so that eight workgroups share a CU:
+  // the kernel needs that many to keep the vector units busy across its five barriers.
+  constexpr int kPitchW = kD / 2 + 16, kPitch = kD + 16;
+  __shared__ __attribute__((aligned(16))) uint32_t s_pmin[16][kPitchW];   // later: the low plane on its way out
+  __shared__ __attribute__((aligned(16))) uint32_t s_pmax[16][kPitchW];   // later: the high plane on its way out
+  __shared__ float s_psum[MODE == 0 ? 1 : 8][kPitch];
+  // [pos]: min, scale, refined reciprocal of the scale, qmax + 0.5; before the ranking its first half
+  // holds s_exact, [pos]: the exact sum of |x| * 2^24 where fp32 leaves a doubt
+  __shared__ float4 s_q[kD];
+  unsigned long long* const s_exact = (unsigned long long*)s_q;
   __shared__ uint8_t s_doubt[MODE == 0 ? 1 : kD];              // [pos]
   __shared__ int s_any_doubt;
-  __shared__ float4 s_q[kD];   // [pos]: min, scale, refined reciprocal of the scale, qmax + 0.5
-  __shared__ float s_c0[kD];   // [pos]: the fast path's offset (fast_offset)
-  __shared__ __attribute__((aligned(16))) uint32_t s_key[kD];   // score << 8 | (127 - channel): larger sorts first
+  __shared__ float2 s_cab[kD];   // [pos]: the fast path's two offsets (fast_offsets)
+  // score << 8 | (127 - channel): larger sorts first; after the ranking s_meta, the (scale, zero) pairs by
+  // channel, as they are stored
+  __shared__ __attribute__((aligned(16))) uint32_t s_key[kD];
+  uint32_t* const s_meta = s_key;
   __shared__ __attribute__((aligned(16))) uint8_t s_idx[kD];    // slot by channel, as it is stored
   __shared__ uint8_t s_idx_p[kD];                               // [pos]
-  static_assert(sizeof(s_pmin) >= kD * 32, "the low plane reuses the minima");
+  // A given slot map need not use every slot; the high-plane rows of unused slots keep their old bytes
+  // (the fused selection fills slots 0 .. d_boost - 1, all of them).
+  __shared__ __attribute__((aligned(4))) uint8_t s_slot_used[MODE == 0 ? 256 : 4];
+  static_assert(sizeof(s_pmin) >= kD * 32 && sizeof(s_pmax) >= kD * 32, "the planes reuse the minima and maxima");
   uint8_t* const s_lo = (uint8_t*)&s_pmin[0][0];
+  uint8_t* const s_hi = (uint8_t*)&s_pmax[0][0];   // 32 bytes per slot
 
-  uint4 rows[8];
+  // this thread's 8 tokens x 8 channels: word q of row r holds channels 2q and 2q + 1 of token r
+  uint32_t w[4][8];
+  {
+    uint4 rows[8];
 #pragma unroll
-  for (int r = 0; r < 8; ++r) rows[r] = nt_load16(row_of(tg * 8 + r) + c8 * 16);
+    for (int r = 0; r < 8; ++r) rows[r] = nt_load16(row_of(tg * 8, r) + c8 * 16);
+#pragma unroll
+    for (int r = 0; r < 8; ++r) {
+      w[0][r] = rows[r].x;
+      w[1][r] = rows[r].y;
+      w[2][r] = rows[r].z;
+      w[3][r] = rows[r].w;
+    }
+  }
 
-  // this thread's 8 tokens x 8 channels as floats, and per channel the partial min / max (/ sum
-  // of |x| in fp32: good enough to rank nearly every channel, see below)
+  // per channel the partial min / max (packed fp16, exact) and the partial sum of |x| in fp32 (good
+  // enough to rank nearly every channel, see below)
   if (MODE != 0 && tid == 0) s_any_doubt = 0;
-  float xs[8][8];   // [channel j][token r]
+  if (MODE == 0 && tid < 64) ((uint32_t*)s_slot_used)[tid] = 0;
 #pragma unroll
-  for (int j = 0; j < 8; ++j) {
+  for (int q = 0; q < 4; ++q) {
+    uint32_t mn = w[q][0], mx = w[q][0];
 #pragma unroll
-    for (int r = 0; r < 8; ++r) {
-      const uint32_t w = ((const uint32_t*)&rows[r])[j >> 1];
-      xs[j][r] = h2f((j & 1) ? (uint16_t)(w >> 16) : (uint16_t)(w & 0xffffu));
+    for (int r = 1; r < 8; ++r) {
+      mn = pk_min_f16(mn, w[q][r]);
+      mx = pk_max_f16(mx, w[q][r]);
     }
-    float mn = xs[j][0], mx = xs[j][0];
+    s_pmin[tg][q * 16 + c8] = mn;
+    s_pmax[tg][q * 16 + c8] = mx;
+    if (MODE != 0) {
 #pragma unroll
-    for (int r = 0; r < 8; ++r) {
-      mn = fminf(mn, xs[j][r]);
-      mx = fmaxf(mx, xs[j][r]);
+      for (int hi = 0; hi < 2; ++hi) {
+        // added as a tree: every term goes through three additions here and a fourth with the
+        // neighbouring token group's sum (lane l ^ 16), whose even member keeps the result
+        const float own = ((abs_sum_f16(w[q][0], w[q][1], hi) + abs_sum_f16(w[q][2], w[q][3], hi)) +
+                           (abs_sum_f16(w[q][4], w[q][5], hi) + abs_sum_f16(w[q][6], w[q][7], hi)));
+        const unsigned bits = __builtin_bit_cast(unsigned, own);
+        const auto both = __builtin_amdgcn_permlane16_swap(bits, bits, false, false);
+        const unsigned b0 = both[0], b1 = both[1];   // as scalars first: a bit_cast of both[1] itself reads element 0
+        if ((tg & 1) == 0)
+          s_psum[tg >> 1][(2 * q + hi) * 16 + c8] = __builtin_bit_cast(float, b0) + __builtin_bit_cast(float, b1);
+      }
     }
-    s_pmin[tg][j * 16 + c8] = mn;
-    s_pmax[tg][j * 16 + c8] = mx;
-    if (MODE != 0)   // added as a tree: every term goes through three additions
-      s_psum[tg][j * 16 + c8] = ((fabsf(xs[j][0]) + fabsf(xs[j][1])) + (fabsf(xs[j][2]) + fabsf(xs[j][3]))) +
-                                ((fabsf(xs[j][4]) + fabsf(xs[j][5])) + (fabsf(xs[j][6]) + fabsf(xs[j][7])));
   }
   __syncthreads();
 
@@ -149,18 +224,25 @@ __device__ __forceinline__ void quant_k_page(const ROWS row_of, int d_boost,
   // (the pair's channel follows the table order, so that its reads are consecutive too)
   const int pos = tid >> 1, hf = tid & 1;
   const int ch = (pos & 15) * 8 + (pos >> 4);
-  float ch_min = s_pmin[hf][pos], ch_max = s_pmax[hf][pos];
+  float ch_min, ch_max;
+  {
+    const int word = (pos >> 5) * 16 + (pos & 15);   // the word that holds this channel, in half (pos >> 4) & 1
+    uint32_t mn = s_pmin[hf][word], mx = s_pmax[hf][word];
 #pragma unroll
-  for (int i = 2; i < 16; i += 2) {
-    ch_min = fminf(ch_min, s_pmin[i + hf][pos]);
-    ch_max = fmaxf(ch_max, s_pmax[i + hf][pos]);
+    for (int i = 2; i < 16; i += 2) {
+      mn = pk_min_f16(mn, s_pmin[i + hf][word]);
+      mx = pk_max_f16(mx, s_pmax[i + hf][word]);
+    }
+    mn = pk_min_f16(mn, (uint32_t)__shfl_xor((int)mn, 1));
+    mx = pk_max_f16(mx, (uint32_t)__shfl_xor((int)mx, 1));
+    const int sh = (pos & 16);   // 16 for the upper half
+    ch_min = widen_f16(mn >> sh, 0);
+    ch_max = widen_f16(mx >> sh, 0);
   }
-  ch_min = fminf(ch_min, __shfl_xor(ch_min, 1));
-  ch_max = fmaxf(ch_max, __shfl_xor(ch_max, 1));
   if (MODE != 0) {
     // The score is the mean of |x| over the page, rounded ONCE to fp16.  In the fp32 sum of the 128
-    // non-negative terms every term went through 7 additions (3 in its thread, 3 in this fold, 1
-    // between the lanes), each with a relative error of at most 2^-24, so the exact mean lies within
+    // non-negative terms every term went through 7 additions (3 in its thread, 1 with the next token
+    // group, 2 in this fold, 1 between the lanes), each with a relative error of at most 2^-24, so the exact mean lies within
     // 7.01 * 2^-24 (relative) of sum / 128.  The ends of the interval tested are that mean times
     // 1 -+ 10 * 2^-24 (both factors are fp32 numbers; the products round once more).  If both ends
     // round to the same fp16 number, that is the score; otherwise (one channel in about 600: the
@@ -168,8 +250,7 @@ __device__ __forceinline__ void quant_k_page(const ROWS row_of, int d_boost,
     // channel), or when the mean is so small that fp16 has no normal number for it, the channel's
     // 16 threads add their terms exactly - every |x| is a multiple of 2^-24 below 2^16 - into a
     // 64-bit integer.
-    float sum = ((s_psum[hf][pos] + s_psum[2 + hf][pos]) + (s_psum[4 + hf][pos] + s_psum[6 + hf][pos])) +
-                ((s_psum[8 + hf][pos] + s_psum[10 + hf][pos]) + (s_psum[12 + hf][pos] + s_psum[14 + hf][pos]));
+    float sum = (s_psum[hf][pos] + s_psum[2 + hf][pos]) + (s_psum[4 + hf][pos] + s_psum[6 + hf][pos]);
     sum += __shfl_xor(sum, 1);
     if (hf == 0) {
       uint32_t score = 0;
@@ -200,7 +281,7 @@ __device__ __forceinline__ void quant_k_page(const ROWS row_of, int d_boost,
           uint32_t up = 0, low = 0;
 #pragma unroll
           for (int r = 0; r < 8; ++r) {
-            const float v = fabsf(xs[j][r]) * 0x1p24f;
+            const float v = (float)__builtin_fabsf16(half_of(w[j >> 1][r], j & 1)) * 0x1p24f;
             const float u = floorf(v * 0x1p-20f);
             up += (uint32_t)u;
             low += (uint32_t)__builtin_fmaf(u, -0x1p20f, v);
@@ -213,19 +294,29 @@ __device__ __forceinline__ void quant_k_page(const ROWS row_of, int d_boost,
         s_key[ch] = ((uint32_t)mean_abs_fp16_bits(s_exact[pos]) << 8) | (uint32_t)(kD - 1 - ch);
       __syncthreads();
     }
-    // rank = number of channels that sort before this one: higher score, or equal score and
-    // lower channel index
-    const uint32_t mine = s_key[ch];
-    int rank = 0;
-#pragma unroll 8
-    for (int d = hf * (kD / 2); d < (hf + 1) * (kD / 2); d += 4) {
-      const uint4 o = *(const uint4*)&s_key[d];
-      rank += (o.x > mine) + (o.y > mine) + (o.z > mine) + (o.w > mine);
+    // rank = number of channels that sort before this one: higher score, or equal score and lower
+    // channel index.  Each wave ranks 32 channels: a lane holds two of the 128 keys, a channel's key is
+    // read into every lane, and the lanes whose keys are larger are counted - one compare per 64 pairs
+    // of keys, the counting on the scalar unit.
+    {
+      const int lane = tid & 63, first = (tid >> 6) * (kD / 4);
+      const uint32_t k0 = s_key[lane], k1 = s_key[lane + 64];
+#pragma unroll
+      for (int i = 0; i < kD / 16; ++i) {
+        const uint4 t = *(const uint4*)&s_key[first + 4 * i];
+        const uint32_t key[4] = {t.x, t.y, t.z, t.w};
+        uint32_t slots = 0;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int rank = __popcll(__ballot(k0 > key[e])) + __popcll(__ballot(k1 > key[e]));
+          slots |= (uint32_t)(rank < d_boost ? rank : d_boost) << (8 * e);
+        }
+        ((uint32_t*)s_idx)[(first >> 2) + i] = slots;   // the same word from every lane
+      }
     }
-    rank += __shfl_xor(rank, 1);
-    const uint8_t slot = (uint8_t)(rank < d_boost ? rank : d_boost);
+    __syncthreads();
+    const uint8_t slot = s_idx[ch];
     if (hf == 0) {
-      s_idx[ch] = slot;
       s_idx_p[pos] = slot;
       if (slot_out) slot_out[ch] = slot;
     }
@@ -236,43 +327,46 @@ __device__ __forceinline__ void quant_k_page(const ROWS row_of, int d_boost,
       scale = scale < 1e-6f ? 1e-6f : scale;
       const Divisor k = make_divisor(scale);
       s_q[pos] = float4{ch_min, k.d, k.r, qmax + 0.5f};
-      s_c0[pos] = fast_offset(ch_min, k);
-      *(__half2*)(meta_dst + ch * 4) = __halves2half2(__float2half_rn(scale), __float2half_rn(ch_min));
+      s_cab[pos] = fast_offsets(ch_min, k);
+      s_meta[ch] = __builtin_bit_cast(uint32_t, __halves2half2(__float2half_rn(scale), __float2half_rn(ch_min)));
     }
   } else if (hf == 0) {
     const uint8_t slot = slot_in[ch];
     s_idx[ch] = slot;
     s_idx_p[pos] = slot;
+    if (slot < d_boost) s_slot_used[slot] = 1;
     const float qmax = slot < d_boost ? 15.0f : 3.0f;
     float scale = (ch_max - ch_min) / qmax;
     scale = scale < 1e-6f ? 1e-6f : scale;
     const Divisor k = make_divisor(scale);
     s_q[pos] = float4{ch_min, k.d, k.r, qmax + 0.5f};
-    s_c0[pos] = fast_offset(ch_min, k);
-    *(__half2*)(meta_dst + ch * 4) = __halves2half2(__float2half_rn(scale), __float2half_rn(ch_min));
+    s_cab[pos] = fast_offsets(ch_min, k);
+    s_meta[ch] = __builtin_bit_cast(uint32_t, __halves2half2(__float2half_rn(scale), __float2half_rn(ch_min)));
   }
-  __syncthreads();   // the tables are complete, and nobody reads the partial minima any more (s_lo takes their place)
+  __syncthreads();   // the tables are complete, and nobody reads the partial minima and maxima any more (s_lo, s_hi take their place)
 
 #pragma unroll
   for (int j = 0; j < 8; ++j) {
     const int d = c8 * 8 + j, dp = j * 16 + c8;
     const float4 qp = s_q[dp];
     const Divisor k = {qp.y, qp.z};
-    // the 8 codes (0..15) as one word of nibbles, built in floating point (exact: 16 bits per half)
-    float c[8];
-    codes_of<8>(xs[j], qp.x, s_c0[dp], k, qp.w, c);
-    const float h0 = __builtin_fmaf(__builtin_fmaf(__builtin_fmaf(c[3], 16.f, c[2]), 16.f, c[1]), 16.f, c[0]);
-    const float h1 = __builtin_fmaf(__builtin_fmaf(__builtin_fmaf(c[7], 16.f, c[6]), 16.f, c[5]), 16.f, c[4]);
-    const uint32_t nib = (uint32_t)h0 | ((uint32_t)h1 << 16);
+    uint32_t c0123, c4567;   // the 8 codes (0..15), a byte each
+    codes_of(w[j >> 1], j & 1, qp.x, s_cab[dp], k, qp.w, c0123, c4567);
     // plane row d, tokens 8 tg ..: byte d * 32 + 2 tg, with the row's 16-byte pieces and its three
     // row-in-octet bits flipped by c8 so that the 16 rows written at once (8 apart) spread over the banks
-    *(uint16_t*)(s_lo + ((d * 32 + tg * 2) ^ (c8 << 4))) = (uint16_t)gather_fields<0>(nib);
+    *(uint16_t*)(s_lo + ((d * 32 + tg * 2) ^ (c8 << 4))) = (uint16_t)gather_fields<0>(c0123, c4567);
     const uint8_t slot = s_idx_p[dp];
-    if (slot < d_boost) *(uint16_t*)(dst + kLoBytes + slot * kRowBytes + tg * 2) = (uint16_t)gather_fields<2>(nib);
+    if (slot < d_boost) *(uint16_t*)(s_hi + slot * kRowBytes + tg * 2) = (uint16_t)gather_fields<2>(c0123, c4567);
   }
   __syncthreads();
+  // everything leaves in contiguous pieces: the low plane by all threads (16 bytes each), the high plane by the
+  // first lanes (16 bytes each), the slot map by the second wave and the (scale, zero) pairs by the last two
+  // (4 bytes each: the metadata's alignment is only that)
   ((uint4*)dst)[tid] = *(const uint4*)(s_lo + ((tid * 16) ^ (((tid >> 4) & 15) << 4)));   // piece tid of the plane: row tid / 2, c8 = row / 8
-  if (tid < kD / 4) ((uint32_t*)(dst + kRowBytes * (kD + d_boost)))[tid] = ((const uint32_t*)s_idx)[tid];
+  if (tid < 2 * d_boost && (MODE != 0 || s_slot_used[tid >> 1])) ((uint4*)(dst + kLoBytes))[tid] = ((const uint4*)s_hi)[tid];
+  const int t1 = tid - 64, t2 = tid - 128;
+  if (t1 >= 0 && t1 < kD / 4) ((uint32_t*)(dst + kRowBytes * (kD + d_boost)))[t1] = ((const uint32_t*)s_idx)[t1];
+  if (t2 >= 0) ((uint32_t*)meta_dst)[t2] = s_meta[t2];
 }
 
 template <int MODE>
@@ -299,6 +393,39 @@ __global__ __launch_bounds__(256) void quant_pack_k_kernel(
   }
   quant_k_page<MODE>(StridedRows{src, stride_t}, d_boost, slot_map_in ? slot_map_in + slot_off : nullptr,
                      slot_map_out ? slot_map_out + slot_off : nullptr, dst, mdst);
+}
+
+// The codes of N values of one group of a V page as floats, mostly without the division:
+//   t = fma(x, r, c0),  c0 = fma(-min, r, 0.5),  r = the refined reciprocal of the scale.
+// Against the reference's fl(fl((x - min) / scale) + 0.5) this differs by the roundings of x - min,
+// of the quotient and of the sum (1e-6 each for quotients below 16.5), the reciprocal's last bit
+// (2e-6), the rounding of c0 (1.9e-6 while |min * r| <= 32) and its own (1e-6): under 8e-6.  So
+// unless t lies within 2^-16 of an integer, floor(t) is the reference's code; the reference's upper
+// clamp never changes a floor for finite inputs (the largest quotient is qmax * (1 + 2^-24)).  If any
+// lane of the wave has such a t among its N, or a group whose c0 is NaN (fast_offset returns that
+// when |min * r| > 32 or the scale is not finite), the wave redoes these N values with the exact
+// division: about one group in seventy on gaussian data.
+__device__ __forceinline__ float fast_offset(float mn, Divisor k) {
+  const float c0 = __builtin_fmaf(-mn, k.r, 0.5f);
+  return (fabsf(mn * k.r) <= 32.0f && k.d < 3.0e38f) ? c0 : __builtin_nanf("");
+}
+template <int N>
+__device__ __forceinline__ void codes_of(const float (&x)[N], float mn, float c0, Divisor k, float qlim, float (&c)[N]) {
+  float fmn = 1.0f, fmx = 0.0f;
+#pragma unroll
+  for (int r = 0; r < N; ++r) {
+    const float t = __builtin_fmaf(x[r], k.r, c0);
+    c[r] = __builtin_floorf(t);
+    const float f = t - c[r];
+    fmn = fminf(fmn, f);
+    fmx = fmaxf(fmx, f);
+  }
+  constexpr float kEps = 1.52587890625e-05f;   // 2^-16
+  // (min / max skip NaNs, so the group's NaN offset is tested by itself)
+  if (__any(!(c0 == c0 && fmn >= kEps && fmx <= 1.0f - kEps))) {
+#pragma unroll
+    for (int r = 0; r < N; ++r) c[r] = code_of(x[r] - mn, k, qlim);
+  }
 }
 
 // One V page of one head: 256 threads, 8 consecutive lanes share a token (16 channels each), 4
@@ -593,6 +720,7 @@ struct KStreamRows {
     const int s = first + t;
     return s < rk ? qbuf + (int64_t)s * (kD * 2) : chunk + (int64_t)(s - rk) * stride_t;
   }
+  __device__ __forceinline__ const uint8_t* operator()(int t0, int r) const { return (*this)(t0 + r); }
 };
 struct VStreamRows {
   const uint8_t* qbuf; const uint8_t* ring; const uint8_t* chunk; int64_t stride_t; int rv, er, off, first;
