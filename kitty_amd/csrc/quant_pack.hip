@@ -395,41 +395,31 @@ __global__ __launch_bounds__(256) void quant_pack_k_kernel(
                      slot_map_out ? slot_map_out + slot_off : nullptr, dst, mdst);
 }
 
-// The codes of N values of one group of a V page as floats, mostly without the division:
-//   t = fma(x, r, c0),  c0 = fma(-min, r, 0.5),  r = the refined reciprocal of the scale.
-// Against the reference's fl(fl((x - min) / scale) + 0.5) this differs by the roundings of x - min,
-// of the quotient and of the sum (1e-6 each for quotients below 16.5), the reciprocal's last bit
-// (2e-6), the rounding of c0 (1.9e-6 while |min * r| <= 32) and its own (1e-6): under 8e-6.  So
-// unless t lies within 2^-16 of an integer, floor(t) is the reference's code; the reference's upper
-// clamp never changes a floor for finite inputs (the largest quotient is qmax * (1 + 2^-24)).  If any
-// lane of the wave has such a t among its N, or a group whose c0 is NaN (fast_offset returns that
-// when |min * r| > 32 or the scale is not finite), the wave redoes these N values with the exact
-// division: about one group in seventy on gaussian data.
-__device__ __forceinline__ float fast_offset(float mn, Divisor k) {
-  const float c0 = __builtin_fmaf(-mn, k.r, 0.5f);
-  return (fabsf(mn * k.r) <= 32.0f && k.d < 3.0e38f) ? c0 : __builtin_nanf("");
-}
-template <int N>
-__device__ __forceinline__ void codes_of(const float (&x)[N], float mn, float c0, Divisor k, float qlim, float (&c)[N]) {
-  float fmn = 1.0f, fmx = 0.0f;
+// The 16 codes (0..3) of one lane's 16 channels of a token - both halves of w[0..7], in the order low
+// half of w[0], high half of w[0], low half of w[1] .. - as bytes of four words: the two roundings of codes_of above, the exact division
+// where they disagree.
+__device__ __forceinline__ void codes_of_row(const uint32_t (&w)[8], float mn, float2 cab, Divisor k, uint32_t (&c)[4]) {
+  uint32_t b[4] = {0, 0, 0, 0};
 #pragma unroll
-  for (int r = 0; r < N; ++r) {
-    const float t = __builtin_fmaf(x[r], k.r, c0);
-    c[r] = __builtin_floorf(t);
-    const float f = t - c[r];
-    fmn = fminf(fmn, f);
-    fmx = fmaxf(fmx, f);
+  for (int i = 0; i < 4; ++i) c[i] = 0;
+#pragma unroll
+  for (int e = 0; e < 16; ++e) {
+    const float x = (float)half_of(w[e >> 1], e & 1);
+    c[e >> 2] = __builtin_amdgcn_cvt_pk_u8_f32(__builtin_fmaf(x, k.r, cab.x), e & 3, c[e >> 2]);
+    b[e >> 2] = __builtin_amdgcn_cvt_pk_u8_f32(__builtin_fmaf(x, k.r, cab.y), e & 3, b[e >> 2]);
   }
-  constexpr float kEps = 1.52587890625e-05f;   // 2^-16
-  // (min / max skip NaNs, so the group's NaN offset is tested by itself)
-  if (__any(!(c0 == c0 && fmn >= kEps && fmx <= 1.0f - kEps))) {
+  if (__any(!(cab.x == cab.x) || c[0] != b[0] || c[1] != b[1] || c[2] != b[2] || c[3] != b[3])) {
 #pragma unroll
-    for (int r = 0; r < N; ++r) c[r] = code_of(x[r] - mn, k, qlim);
+    for (int i = 0; i < 4; ++i) c[i] = 0;
+#pragma unroll
+    for (int e = 0; e < 16; ++e)
+      c[e >> 2] = __builtin_amdgcn_cvt_pk_u8_f32(code_of((float)half_of(w[e >> 1], e & 1) - mn, k, 3.5f), e & 3, c[e >> 2]);
   }
 }
 
-// One V page of one head: 256 threads, 8 consecutive lanes share a token (16 channels each), 4
-// tokens per thread.  row_of(t): the 256-byte row of token t of this head.
+// One V page of one head: 256 threads, 8 consecutive lanes share a token, 4 tokens per thread.  A lane
+// holds channels 8 cg .. 8 cg + 7 and 64 + 8 cg .. 64 + 8 cg + 7 of its tokens: each load instruction
+// then reads whole 128-byte half rows, 16 bytes per lane.  row_of(t): the 256-byte row of token t of this head.
 template <class ROWS>
 __device__ __forceinline__ void quant_v_page(const ROWS row_of, uint8_t* __restrict__ dst, uint8_t* __restrict__ mdst) {
   const int tid = threadIdx.x;
@@ -437,43 +427,53 @@ __device__ __forceinline__ void quant_v_page(const ROWS row_of, uint8_t* __restr
   uint4 la[4], lc[4];   // all eight loads of the thread are in flight before the first is used
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
-    const uint8_t* src = row_of((tid >> 3) + 32 * i) + cg * 32;
+    const uint8_t* src = row_of((tid >> 3) + 32 * i) + cg * 16;
     la[i] = nt_load16(src);
-    lc[i] = nt_load16(src + 16);
+    lc[i] = nt_load16(src + kD);
   }
+  // The lane's codes make bytes 2 cg, 2 cg + 1 and 16 + 2 cg, 17 + 2 cg of the token's 32-byte row.  Lanes
+  // 2 m and 2 m + 1 swap one of the two pairs, so that the even lane has bytes 4 m .. 4 m + 3 and the odd
+  // lane bytes 16 + 4 m .. 19 + 4 m: one 4-byte store per lane.
+  const bool odd = cg & 1;
+  const uint32_t pick = odd ? 0x03020706u : 0x05040100u;   // odd: (partner's upper pair, own upper pair); even: (own lower, partner's lower)
+  const int out_off = odd ? 14 + 2 * cg : 2 * cg;
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int t = (tid >> 3) + 32 * i;
     const uint4 a = la[i], c = lc[i];
     const uint32_t w[8] = {a.x, a.y, a.z, a.w, c.x, c.y, c.z, c.w};
-    float x[16];
-    float mn = INFINITY, mx = -INFINITY;
+    // The token's minimum and maximum in packed fp16 (exact): over the lane's 8 words, then with the
+    // maximum negated beside the minimum in one word, so that one packed minimum per step serves both,
+    // over the word's own halves and over the 8 lanes that share the token.
+    uint32_t mnw = w[0], mxw = w[0];
 #pragma unroll
-    for (int k = 0; k < 8; ++k) {
-      x[2 * k] = h2f((uint16_t)(w[k] & 0xffffu));
-      x[2 * k + 1] = h2f((uint16_t)(w[k] >> 16));
-      mn = fminf(mn, fminf(x[2 * k], x[2 * k + 1]));
-      mx = fmaxf(mx, fmaxf(x[2 * k], x[2 * k + 1]));
+    for (int k = 1; k < 8; ++k) {
+      mnw = pk_min_f16(mnw, w[k]);
+      mxw = pk_max_f16(mxw, w[k]);
     }
-#pragma unroll
-    for (int o = 1; o < 8; o <<= 1) {
-      mn = fminf(mn, __shfl_xor(mn, o));
-      mx = fmaxf(mx, __shfl_xor(mx, o));
-    }
+    const uint32_t nmx = mxw ^ 0x80008000u;
+    uint32_t m = pk_min_f16(__builtin_amdgcn_perm(nmx, mnw, 0x05040100u),    // (mnw.lo, nmx.lo)
+                            __builtin_amdgcn_perm(nmx, mnw, 0x07060302u));   // (mnw.hi, nmx.hi)
+    // lanes l ^ 1, l ^ 2, then 7 - l of the group of 8 (whose quads agree by then): data-parallel moves,
+    // no trip through the LDS crossbar
+    m = pk_min_f16(m, (uint32_t)__builtin_amdgcn_mov_dpp((int)m, 0xB1 /* quad_perm [1,0,3,2] */, 0xf, 0xf, true));
+    m = pk_min_f16(m, (uint32_t)__builtin_amdgcn_mov_dpp((int)m, 0x4E /* quad_perm [2,3,0,1] */, 0xf, 0xf, true));
+    m = pk_min_f16(m, (uint32_t)__builtin_amdgcn_mov_dpp((int)m, 0x141 /* row_half_mirror */, 0xf, 0xf, true));
+    const float mn = widen_f16(m, 0), mx = -widen_f16(m, 1);
     float scale = (mx - mn) / 3.0f;
     scale = scale < 1e-6f ? 1e-6f : scale;
     const Divisor kd = make_divisor(scale);
-    float code[16];
-    codes_of<16>(x, mn, fast_offset(mn, kd), kd, 3.5f, code);
-    // 16 codes (0..3), 2 bits each, built in floating point in two exact 16-bit halves
-    float h0 = 0.f, h1 = 0.f;
-#pragma unroll
-    for (int k = 7; k >= 0; --k) {
-      h0 = __builtin_fmaf(h0, 4.f, code[k]);
-      h1 = __builtin_fmaf(h1, 4.f, code[8 + k]);
-    }
-    const uint32_t packed = (uint32_t)h0 | ((uint32_t)h1 << 16);
-    __builtin_nontemporal_store(packed, (uint32_t*)(dst + t * kRowBytes + cg * 4));   // written once, read much later
+    uint32_t code[4];
+    codes_of_row(w, mn, fast_offsets(mn, kd), kd, code);
+    // 16 codes, 2 bits each: a dot product of four code bytes with (1, 4, 16, 64) is a byte of the row
+    constexpr uint32_t kWeights = 0x40100401u;
+    const uint32_t own = __builtin_amdgcn_udot4(code[0], kWeights, 0u, false) |
+                         (__builtin_amdgcn_udot4(code[1], kWeights, 0u, false) << 8) |
+                         (__builtin_amdgcn_udot4(code[2], kWeights, 0u, false) << 16) |
+                         (__builtin_amdgcn_udot4(code[3], kWeights, 0u, false) << 24);
+    const uint32_t partner = (uint32_t)__builtin_amdgcn_mov_dpp((int)own, 0xB1 /* quad_perm [1,0,3,2] */, 0xf, 0xf, true);
+    const uint32_t packed = __builtin_amdgcn_perm(partner, own, pick);
+    __builtin_nontemporal_store(packed, (uint32_t*)(dst + t * kRowBytes + out_off));   // written once, read much later
     if (cg == 0) *(__half2*)(mdst + t * 4) = __halves2half2(__float2half_rn(scale), __float2half_rn(mn));
   }
 }
