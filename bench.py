@@ -697,10 +697,14 @@ class DecodeBench:
 
     def timed(self, steps, warmup, variant=None):
         """`steps` steps as a caller runs them (wall clock, synchronised on both sides), then the same
-        steps once more with events on the split kernel's dispatch."""
+        steps twice more with events on the split kernel's dispatch: once right after the
+        synchronisation, as the wall clock saw them, and once behind `warmup` + 20 untimed steps
+        with no wait in between.  The first launch after a blocking synchronisation reads 15-20 us
+        long and the next ones up to 5 us, on some boxes; the kernel's own duration is the second
+        figure, which is also what a kernel trace of the run averages to."""
         torch, hip = self.torch, self.hip
-        events = [(hip.create(), hip.create()) for _ in range(steps)]   # before the warm-up: no host work (and no
-        for i in range(warmup):                                          # idle device) between it and the timed steps
+        events = [(hip.create(), hip.create()) for _ in range(2 * steps)]   # before the warm-up: no host work (and
+        for i in range(warmup):                                              # no idle device) between it and the timed steps
             self.step(self.n_done + i, None, variant)
         self.n_done += warmup
         torch.cuda.synchronize()
@@ -715,7 +719,15 @@ class DecodeBench:
         torch.cuda.synchronize()
         us_per_step_events = (time.perf_counter() - t0) / steps * 1e6
         self.n_done += 2 * steps
-        kern_us = sorted(hip.elapsed_us(a, b) for a, b in events)
+        for i in range(warmup + 20):
+            self.step(self.n_done + i, None, variant)
+        self.n_done += warmup + 20
+        for i in range(steps):
+            self.step(self.n_done + i, events[steps + i], variant)
+        torch.cuda.synchronize()
+        self.n_done += steps
+        self.kern_us_after_sync = sorted(hip.elapsed_us(a, b) for a, b in events[:steps])
+        kern_us = sorted(hip.elapsed_us(a, b) for a, b in events[steps:])
         return us_per_step, us_per_step_events, kern_us
 
     n_done = 0
@@ -733,6 +745,7 @@ class DecodeBench:
                 "algorithmic_bytes_per_launch": self.total_bytes, "packed_bytes_per_launch": self.packed_bytes,
                 "achieved_gbps": gbps, "frac": gbps / HBM_PEAK_GBPS,
                 "packed_frac": self.packed_bytes / (avg * 1e-6) / 1e9 / HBM_PEAK_GBPS,
+                "kernel_avg_us_after_sync": sum(self.kern_us_after_sync) / len(self.kern_us_after_sync),
                 "settled_after_launches": settle["launches"], "settled": settle["settled"]}
 
     def headline(self, args):
@@ -781,8 +794,13 @@ class DecodeBench:
                 "packed_frac": self.packed_bytes / (kern_avg_us * 1e-6) / 1e9 / HBM_PEAK_GBPS,
                 "cache_hot_kernel_us": hot_us,
                 "timing": "HIP events attached to the split kernel's dispatch on the launch stream (kernel begin to "
-                          "end), averaged over the timed steps run a second time with the events attached (their "
-                          "marker packets cost a step about 5 us, so `value` is timed without them)",
+                          "end), averaged over the timed steps run again with the events attached (their marker "
+                          "packets cost a step about 5 us, so `value` is timed without them) behind untimed steps "
+                          "with no wait in between; `kernel_avg_us_after_sync`: the same steps right after a "
+                          "synchronisation, as `value` runs them (the first launch after a blocking wait reads "
+                          "15-20 us long, the next ones up to 5 us on some boxes)",
+                "kernel_avg_us_after_sync": sum(self.kern_us_after_sync) / len(self.kern_us_after_sync),
+                "kernel_median_us_after_sync": self.kern_us_after_sync[len(self.kern_us_after_sync) // 2],
                 "us_per_step_with_events": us_per_step_events,
                 "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE summary committed under profiles/ (a run "
                                   "of its own, calibrated by a 1 GiB copy), not measured in this run",
