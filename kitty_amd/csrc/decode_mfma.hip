@@ -1191,14 +1191,13 @@ __device__ __forceinline__ void wave_work(const kitty_kv_layer& L, const __half*
     if (t0 < t1) {
       if constexpr (!Q_VIA_LDS) settle_prologue_loads();   // (else: no load of the prologue fills a register the loop reads)
       constexpr int nK = kDmaK<BOOST>;
-      const uint32_t lk0 = (uint32_t)(uintptr_t)&S.kbuf[0][0], lk1 = (uint32_t)(uintptr_t)&S.kbuf[1][0];
+      const uint32_t lk0 = (uint32_t)(uintptr_t)&S.kbuf[0][0];
       const uint32_t lv = (uint32_t)(uintptr_t)&S.vbuf[0];
       dma_k<BOOST>(x, t0, lk0);
-      if (t0 + 1 < t1) dma_k<BOOST>(x, t0 + 1, lk1);
       dma_v(x, t0, lv);
       if constexpr (Q_VIA_LDS) {
         // the query rows were asked for before these tiles: everything older than the tiles has landed
-        if (t0 + 1 < t1) wait_vmcnt<2 * nK + kDmaV>(); else wait_vmcnt<nK + kDmaV>();
+        wait_vmcnt<nK + kDmaV>();
         const _Float16* ql = (const _Float16*)&S.qs[0][0];
 #pragma unroll
         for (int kc = 0; kc < 4; ++kc)
@@ -1223,31 +1222,26 @@ __device__ __forceinline__ void wave_work(const kitty_kv_layer& L, const __half*
 #pragma unroll 1
       for (int i = t0; i < t1; ++i) {
         float cz;
-        const int buf = (i - t0) & 1;
-        const bool k1 = i + 1 < t1, k2 = i + 2 < t1;   // K(i+1) has been, K(i+2) will be asked for
+        const bool k1 = i + 1 < t1;
         const bool fav = SWITCH && 4 * (i - t0) >= t1 - t0;
         // K(i) is followed in the queue by V(i-1) (not in the first iteration), K(i+1) if any, V(i)
-        if (i == t0) {
-          if (k1) wait_vmcnt<nK + kDmaV>(); else wait_vmcnt<kDmaV>();
-        } else {
-          if (k1) wait_vmcnt<nK + 2 * kDmaV>(); else wait_vmcnt<2 * kDmaV>();
-        }
+        wait_vmcnt<kDmaV>();   // K(i) is followed by V(i)
         if (fav) __builtin_amdgcn_s_setprio(KITTY_PRIO_MFMA + 1); else __builtin_amdgcn_s_setprio(KITTY_PRIO_MFMA);
-        if constexpr (QUARTER) qk_packed_tab<BOOST>(S, x, S.kbuf[buf], C, cz);
-        else qk_packed<BOOST, SPLIT_COLS>(S, x, KLds{S.kbuf[buf]}, C, cz);
+        if constexpr (QUARTER) qk_packed_tab<BOOST>(S, x, S.kbuf[0], C, cz);
+        else qk_packed<BOOST, SPLIT_COLS>(S, x, KLds{S.kbuf[0]}, C, cz);
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-        if (k2) dma_k<BOOST>(x, i + 2, buf ? lk1 : lk0);
+        if (k1) dma_k<BOOST>(x, i + 1, lk0);
         if (fav) __builtin_amdgcn_s_setprio(KITTY_PRIO_VALU + 1); else __builtin_amdgcn_s_setprio(KITTY_PRIO_VALU);
         if constexpr (QUARTER) {
           float4v own[2];
           combine_quarter(x, C, own);
           softmax_quarter(x, A, own, cz);
-          if (k2) wait_vmcnt<nK>(); else wait_vmcnt<0>();   // V(i) is followed by K(i+2) if any
+          if (k1) wait_vmcnt<nK>(); else wait_vmcnt<0>();
           if (fav) __builtin_amdgcn_s_setprio(KITTY_PRIO_MFMA + 1); else __builtin_amdgcn_s_setprio(KITTY_PRIO_MFMA);
           pv_quarter(S, x, A.out, A.lz, VLds{S.vbuf}, own);
         } else {
           softmax_tile<true>(x, A, C, cz, kPage);
-          if (k2) wait_vmcnt<nK>(); else wait_vmcnt<0>();
+          if (k1) wait_vmcnt<nK>(); else wait_vmcnt<0>();
           if (fav) __builtin_amdgcn_s_setprio(KITTY_PRIO_MFMA + 1); else __builtin_amdgcn_s_setprio(KITTY_PRIO_MFMA);
           pv_packed(S, x, A.out, A.lz, VLds{S.vbuf}, C);
         }
