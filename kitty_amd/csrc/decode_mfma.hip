@@ -1183,11 +1183,14 @@ __device__ __forceinline__ void wave_work(const kitty_kv_layer& L, const __half*
     t1 = t0;   // (a split with tail work has no body tiles; this tells the compiler)
   }
   if constexpr (MODE != kWaveTail && DMA) {
-    // Tiles stream through LDS: two K buffers, one V buffer.  Issue order
-    //   K(t0) K(t0+1) V(t0) | QK(i) -> K(i+2) -> softmax -> PV(i) -> V(i+1) | ...
-    // so K(i) has a lead of one and a half iterations and V(i) of half an iteration.  The waits
+    // Tiles stream through LDS, one K tile and one V tile at a time: a buffer is asked to be filled
+    // again as soon as its tile has been consumed.  Issue order
+    //   K(t0) V(t0) | QK(i) -> K(i+1) -> softmax -> PV(i) -> V(i+1) | ...
+    // so each tile has a lead of half an iteration.  (A second K buffer with a lead of one and a
+    // half iterations was 2.6 % slower at 32k tokens x 16 sequences and 3.5 % at 128k x 1: the
+    // memory system serves this many concurrent streams better with less in flight.)  The waits
     // count the instructions issued AFTER the tile that is needed; nothing is loaded past the end
-    // of the range (the last two iterations wait on shorter queues).
+    // of the range (the last iteration waits on a shorter queue).
     if (t0 < t1) {
       if constexpr (!Q_VIA_LDS) settle_prologue_loads();   // (else: no load of the prologue fills a register the loop reads)
       constexpr int nK = kDmaK<BOOST>;
