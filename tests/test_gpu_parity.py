@@ -121,6 +121,39 @@ def test_quantize_pack_bit_exact_random(K, student_t):
     assert np.array_equal(_np16(kc2), okc2)      # unmapped high-plane rows keep their old bytes
 
 
+@pytest.mark.parametrize("DB", [8, 64, 128])
+def test_quantize_pack_other_boost_counts(K, DB):
+    """Boost counts other than the reference's D // 4 (its kernels take d_boost as a parameter,
+    kitty_quant_pack.py:42-45): the high plane has DB rows of 32 bytes, the slot map DB as its
+    "not boosted" mark.  Fused selection, and a given map that leaves slots unused."""
+    B, H, P, t0 = 1, 2, 3, 32
+    k, _ = make_kv(B, H, t0 + P * 128 + 5, seed=70 + DB)
+    rng = np.random.default_rng(DB)
+    pt = rng.permutation(B * 4).reshape(B, 4).astype(np.int64)
+    lay = O.Layout(H_KV=H, D=128, D_BOOSTED=DB)
+    okc = np.full((B * 4, lay.bytes_per_page_K), 0xA5, np.uint8)
+    okm = np.zeros((B * 4, H, 128, 2), np.float16)
+    used = O.quantize_pack_k(k, t0, P, pt, 1, okc, okm, 128, DB)
+    kc, km = K.u.to_dev(np.full_like(okc, 0xA5)), K.u.to_dev(np.zeros_like(okm))
+    kd, ptd = K.u.to_dev(k), K.u.to_dev(pt)
+    K.qk(kd, t0, P, ptd, 1, kc, km, 128, DB)
+    sm = K.sel(kd, t0, P, 128, DB)
+    torch.cuda.synchronize()
+    assert np.array_equal(_np16(sm), used)
+    assert np.array_equal(_np16(kc), okc)
+    assert np.array_equal(_np16(km).view(np.uint16), okm.view(np.uint16))
+    n_used = DB // 2 + 1
+    sm2 = np.full((B, H, P, 128), DB, np.uint8)
+    for idx in np.ndindex(B, H, P):
+        sm2[idx][rng.permutation(128)[:n_used]] = rng.permutation(DB)[:n_used]
+    okc2 = np.full_like(okc, 0x5A)
+    O.quantize_pack_k(k, t0, P, pt, 1, okc2, okm.copy(), 128, DB, slot_map=sm2)
+    kc2 = K.u.to_dev(np.full_like(okc, 0x5A))
+    K.qk(kd, t0, P, ptd, 1, kc2, km, 128, DB, slot_map=K.u.to_dev(sm2))
+    torch.cuda.synchronize()
+    assert np.array_equal(_np16(kc2), okc2)      # unmapped high-plane rows keep their old bytes
+
+
 def _awkward_page(rng):
     """[128 tokens, 128 channels] fp16 whose channel groups exercise the quantizer's exact-division
     fallback: offsets far larger than the range, constant groups (scale floor), values that sit
