@@ -45,8 +45,9 @@
 #include "decode_common.h"
 
 // Wave priority while a phase is dominated by matrix instructions / by vector instructions: the
-// wave that feeds the matrix pipe wins arbitration, the other one fills the gaps (worth ~2 %).
-#define KITTY_PRIO_MFMA 2
+// wave that feeds the matrix pipe wins arbitration, the other one fills the gaps (worth ~2 %; one
+// level of difference, not two: at 2 / 0 the kernel is 1-2 % slower, at 3 / 0 4 %, at equal levels 2 %).
+#define KITTY_PRIO_MFMA 1
 #define KITTY_PRIO_VALU 0
 
 namespace kitty {
@@ -589,9 +590,11 @@ __device__ __forceinline__ void combine_quarter(const Ctx& x, const float4v (&C)
 // are in natural order - slot (kg, 2pi + h) = channel 32kc + 8kg + 2pi + h - so that an operand is one
 // 16-byte load of the row, and q comes from its natural-order copy in LDS (q_nat).  The loads of
 // four tiles (16 per lane) are issued together: the rows come straight from HBM and a wave has
-// nothing else to do while it waits, so the depth of the queue is what the phase costs.
+// nothing else to do while it waits, so the depth of the queue is what the phase costs.  Lanes whose
+// row lies past the `nrows` valid ones read the last valid row again (their logits are masked later):
+// nothing is fetched that does not count.
 template <class LDS>
-__device__ __forceinline__ void qk_fp16(const LDS& S, const Ctx& x, const uint8_t* rows, int nrows_alloc, float4v (&C)[8]) {
+__device__ __forceinline__ void qk_fp16(const LDS& S, const Ctx& x, const uint8_t* rows, int nrows, float4v (&C)[8]) {
   uint4v bq[4];
 #pragma unroll
   for (int kc = 0; kc < 4; ++kc) bq[kc] = *(const uint4v*)&S.q_nat[x.g][32 * kc + 8 * x.kg];
@@ -600,7 +603,7 @@ __device__ __forceinline__ void qk_fp16(const LDS& S, const Ctx& x, const uint8_
     uint4v a[4][4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const int row = min(8 * x.n + 4 * half + i, nrows_alloc - 1);   // A row of this lane; clamped rows are masked later
+      const int row = min(8 * x.n + 4 * half + i, nrows - 1);   // A row of this lane; clamped rows are masked later
       const uint8_t* rp = rows + (int64_t)row * (kD * 2) + 16 * x.kg;
 #pragma unroll
       for (int kc = 0; kc < 4; ++kc) a[i][kc] = *(const uint4v*)(rp + 64 * kc);
@@ -1287,7 +1290,7 @@ __device__ __forceinline__ void wave_work(const kitty_kv_layer& L, const __half*
         qk_packed<BOOST, SPLIT_COLS>(S, x, kb, C, cz);
         softmax_tile<true>(x, A, C, cz, ntok);
       } else {
-        qk_fp16(S, x, qbuf_k, kPage, C);
+        qk_fp16(S, x, qbuf_k, ntok, C);
         softmax_tile<false>(x, A, C, 0.f, ntok);
       }
       if (i < x.c.pv) {
@@ -1310,7 +1313,7 @@ __device__ __forceinline__ void wave_work(const kitty_kv_layer& L, const __half*
     }
     if (do_sink && x.c.sink > 0) {
       const uint8_t* sink_k = (const uint8_t*)L.sink_k + (int64_t)x.b * L.sink_stride_b + (int64_t)x.h * L.sink_stride_h;
-      qk_fp16(S, x, sink_k, L.S, C);
+      qk_fp16(S, x, sink_k, x.c.sink, C);
       softmax_tile<false>(x, A, C, 0.f, x.c.sink);
       pv_fp16<true, QUARTER>(&S.kbuf[0][0], x, A, 0, x.c.sink, C);
     }
