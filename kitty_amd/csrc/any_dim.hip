@@ -7,9 +7,9 @@
 // arithmetic and the same storage format - plain vector-ALU code, one template parameter for D:
 //
 //   quant_k_any_kernel / quant_v_any_kernel   quantize-and-pack, boost selection fused or given
-//   attn_any_kernel<D, false>                 decode attention, split pass (the reference's order of
+//   attn_any_kernel<D, false, ROWS>           decode attention, split pass (the reference's order of
 //                                             operations: fp16 dequantization with both roundings)
-//   attn_any_kernel<D, true>                  chunked-prefill attention, one pass
+//   attn_any_kernel<D, true, 16>              chunked-prefill attention, one pass
 //   merge_any_kernel                          the merge pass of split-K
 //
 // Wire format for general D (PAGE = 128 tokens): a K page-head is 32 D bytes of low plane (channel d at
@@ -21,7 +21,7 @@
 namespace kitty {
 namespace {
 
-constexpr int kMaxRows = 16;   // query rows per workgroup: the group's heads (decode), heads x positions (prefill)
+constexpr int kMaxRows = 16;   // query rows per workgroup at most: the group's heads (decode), heads x positions (prefill)
 
 // ---------------------------------------------------------------------------------------------
 // quantize and pack
@@ -185,7 +185,7 @@ __device__ inline float dequant_two(uint32_t code, __half scale, __half zero) {
 // goes to out [B, T_q, H_Q, D].
 // Logits: thread = (token, half of the channels).  Output: thread = (channel, 1 / (256 / D) of the tile's
 // tokens).  Logits and probabilities stay fp32.
-template <int D, bool PREFILL>
+template <int D, bool PREFILL, int ROWS>
 __global__ __launch_bounds__(256) void attn_any_kernel(
     kitty_kv_layer L, const uint8_t* __restrict__ q, int64_t q_stride_b, int64_t q_stride_h, int64_t q_stride_t,
     const uint8_t* __restrict__ k_new, const uint8_t* __restrict__ v_new, int64_t new_stride_b,
@@ -199,7 +199,7 @@ __global__ __launch_bounds__(256) void attn_any_kernel(
   const int G = H_Q / L.H_KV;
   const int DB = L.D_BOOSTED;
   const SeqCounts c = load_counts(L, b);
-  const int PB = PREFILL ? max(1, kMaxRows / G) : 1;
+  const int PB = PREFILL ? max(1, ROWS / G) : 1;
   const int R = PREFILL ? G * PB : G;
   const int p0 = PREFILL ? (int)blockIdx.x * PB : 0;
   const int kv_chunk = PREFILL ? min(Tq, p0 + PB) : 0;           // chunk tokens this workgroup can see
@@ -212,18 +212,18 @@ __global__ __launch_bounds__(256) void attn_any_kernel(
   }
   int bad_page = 0;
 
-  __shared__ float s_q[kMaxRows][D];
+  __shared__ __attribute__((aligned(16))) float s_q[D][ROWS];        // [channel][row]: a thread reads the rows of a channel at once
   __shared__ __attribute__((aligned(16))) uint8_t s_codes[kRowBytes * 2 * D + D];   // a K page-head with d_boost up to D
   __shared__ __half2 s_meta[D > kPage ? D : kPage];
-  __shared__ float s_p[kMaxRows][kPage];
+  __shared__ __attribute__((aligned(16))) float s_p[kPage][ROWS];    // [token][row]
   __shared__ union {
-    float part[2][kMaxRows][kPage];        // logits: [half of the channels][row][token]
-    float o[kParts][kMaxRows][D];          // the output's partial sums at the end
+    float part[2][ROWS][kPage];        // logits: [half of the channels][row][token]
+    float o[kParts][ROWS][D];          // the output's partial sums at the end
   } s_u;
-  __shared__ float s_m[kMaxRows], s_l[kMaxRows], s_alpha[kMaxRows];
-  __shared__ int s_pos[kMaxRows];          // prefill: chunk position of a row, -1 = no such row
+  __shared__ float s_m[ROWS], s_l[ROWS], s_alpha[ROWS];
+  __shared__ int s_pos[ROWS];          // prefill: chunk position of a row, -1 = no such row
 
-  if (tid < kMaxRows) {
+  if (tid < ROWS) {
     s_m[tid] = -INFINITY;
     s_l[tid] = 0.f;
     int pos = 0;
@@ -234,11 +234,11 @@ __global__ __launch_bounds__(256) void attn_any_kernel(
     const int r = i / D, d = i % D;
     const int g = PREFILL ? r / PB : r, pos = PREFILL ? min(p0 + r % PB, Tq - 1) : 0;
     const uint8_t* row = q + (int64_t)b * q_stride_b + (int64_t)(h * G + g) * q_stride_h + (int64_t)pos * q_stride_t;
-    s_q[r][d] = __half2float(((const __half*)row)[d]);
+    s_q[d][r] = __half2float(((const __half*)row)[d]);
   }
-  float acc_o[kMaxRows];
+  float acc_o[ROWS];
 #pragma unroll
-  for (int g = 0; g < kMaxRows; ++g) acc_o[g] = 0.f;
+  for (int g = 0; g < ROWS; ++g) acc_o[g] = 0.f;
   __syncthreads();
 
   const int t = tid & 127, half = tid >> 7;
@@ -257,9 +257,9 @@ __global__ __launch_bounds__(256) void attn_any_kernel(
     const bool v_packed = !chunk && tile > 0 && body < c.pv;
 
     // ---- logits -----------------------------------------------------------------------------
-    float acc[kMaxRows];
+    float acc[ROWS];
 #pragma unroll
-    for (int g = 0; g < kMaxRows; ++g) acc[g] = 0.f;
+    for (int g = 0; g < ROWS; ++g) acc[g] = 0.f;
     if (k_packed) {
       const int64_t pg = checked_page(page_id(L.page_table_k, (int64_t)b * L.page_table_k_stride_b + body), L.cache_pages_k, bad_page);
       const uint8_t* src = L.key_cache + pg * L.key_cache_stride_page + (int64_t)h * k_head_bytes_d(D, DB);
@@ -277,8 +277,8 @@ __global__ __launch_bounds__(256) void attn_any_kernel(
         const __half2 m = s_meta[d];
         const float x = dequant_two(code, __low2half(m), __high2half(m));
 #pragma unroll
-        for (int g = 0; g < kMaxRows; ++g)
-          if (g < R) acc[g] += s_q[g][d] * x;
+        for (int g = 0; g < ROWS; ++g)
+          if (g < R) acc[g] += s_q[d][g] * x;
       }
     } else if (t < ntok) {
       const __half* row = chunk      ? (const __half*)(kc + (int64_t)(chunk_t0 + t) * new_stride_t)
@@ -287,12 +287,12 @@ __global__ __launch_bounds__(256) void attn_any_kernel(
       for (int d = half * (D / 2); d < (half + 1) * (D / 2); ++d) {
         const float x = __half2float(row[d]);
 #pragma unroll
-        for (int g = 0; g < kMaxRows; ++g)
-          if (g < R) acc[g] += s_q[g][d] * x;
+        for (int g = 0; g < ROWS; ++g)
+          if (g < R) acc[g] += s_q[d][g] * x;
       }
     }
 #pragma unroll
-    for (int g = 0; g < kMaxRows; ++g)
+    for (int g = 0; g < ROWS; ++g)
       if (g < R) s_u.part[half][g][t] = acc[g];
     __syncthreads();
 
@@ -315,8 +315,8 @@ __global__ __launch_bounds__(256) void attn_any_kernel(
 #pragma unroll
       for (int o = 32; o > 0; o >>= 1) sum += __shfl_xor(sum, o);
       const float alpha = (m_old == -INFINITY) ? 0.f : __expf(m_old - m_new);
-      s_p[g][lane] = p0v;
-      s_p[g][lane + 64] = p1v;
+      s_p[lane][g] = p0v;
+      s_p[lane + 64][g] = p1v;
       if (lane == 0) { s_m[g] = m_new; s_l[g] = s_l[g] * alpha + sum; s_alpha[g] = alpha; }
     }
     // ---- stage V ---------------------------------------------------------------------------
@@ -333,7 +333,7 @@ __global__ __launch_bounds__(256) void attn_any_kernel(
     // ---- out += P V : thread = (channel, part of the tile's tokens) ---------------------------
     {
 #pragma unroll
-      for (int g = 0; g < kMaxRows; ++g)
+      for (int g = 0; g < ROWS; ++g)
         if (g < R) acc_o[g] *= s_alpha[g];
       const int t0 = opart * kPartTok, t1 = min(ntok, (opart + 1) * kPartTok);
       for (int tt = t0; tt < t1; ++tt) {
@@ -350,8 +350,8 @@ __global__ __launch_bounds__(256) void attn_any_kernel(
           x = __half2float(v_tail_row(L, c, b, h, (body - c.pv) * kPage + tt, D)[od]);
         }
 #pragma unroll
-        for (int g = 0; g < kMaxRows; ++g)
-          if (g < R) acc_o[g] += s_p[g][tt] * x;   // (a masked token has probability 0)
+        for (int g = 0; g < ROWS; ++g)
+          if (g < R) acc_o[g] += s_p[tt][g] * x;   // (a masked token has probability 0)
       }
     }
     __syncthreads();
@@ -359,7 +359,7 @@ __global__ __launch_bounds__(256) void attn_any_kernel(
 
   if (tid == 0) report_bad_page(L, b, bad_page);
 #pragma unroll
-  for (int g = 0; g < kMaxRows; ++g)
+  for (int g = 0; g < ROWS; ++g)
     if (g < R) s_u.o[opart][g][od] = acc_o[g];
   __syncthreads();
   for (int i = tid; i < R * D; i += 256) {
@@ -453,14 +453,22 @@ void launch_decode_any(const kitty_kv_layer& L, const void* q, int B, int H_Q, f
                        float* ws_acc, int num_splits, hipStream_t stream) {
   const dim3 grid(num_splits, L.H_KV, B), block(256);
   const int64_t qb = (int64_t)H_Q * L.D * 2, qh = (int64_t)L.D * 2;
-  if (L.D == 64)
-    hipLaunchKernelGGL((attn_any_kernel<64, false>), grid, block, 0, stream, L, (const uint8_t*)q, qb, qh, (int64_t)0,
-                       nullptr, nullptr, (int64_t)0, (int64_t)0, (int64_t)0, H_Q, 1, scaling, ws_ml, ws_acc,
-                       num_splits, nullptr);
-  else
-    hipLaunchKernelGGL((attn_any_kernel<256, false>), grid, block, 0, stream, L, (const uint8_t*)q, qb, qh,
-                       (int64_t)0, nullptr, nullptr, (int64_t)0, (int64_t)0, (int64_t)0, H_Q, 1, scaling, ws_ml,
-                       ws_acc, num_splits, nullptr);
+  const int G = H_Q / L.H_KV;
+  // the kernel is instantiated for 4, 8 and 16 query rows: a group of 4 heads does not pay for 16
+#define KITTY_ATTN_ANY(DD, RR)                                                                                       \
+  hipLaunchKernelGGL((attn_any_kernel<DD, false, RR>), grid, block, 0, stream, L, (const uint8_t*)q, qb, qh,         \
+                     (int64_t)0, nullptr, nullptr, (int64_t)0, (int64_t)0, (int64_t)0, H_Q, 1, scaling, ws_ml,       \
+                     ws_acc, num_splits, nullptr)
+  if (L.D == 64) {
+    if (G <= 4) KITTY_ATTN_ANY(64, 4);
+    else if (G <= 8) KITTY_ATTN_ANY(64, 8);
+    else KITTY_ATTN_ANY(64, 16);
+  } else {
+    if (G <= 4) KITTY_ATTN_ANY(256, 4);
+    else if (G <= 8) KITTY_ATTN_ANY(256, 8);
+    else KITTY_ATTN_ANY(256, 16);
+  }
+#undef KITTY_ATTN_ANY
 }
 
 void launch_merge_any(int D, const float* ws_ml, const float* ws_acc, void* out, int B, int H_Q, int num_splits,
@@ -480,11 +488,11 @@ void launch_prefill_any(const kitty_kv_layer& L, const void* q, int64_t q_stride
   const int PB = kMaxRows / G > 0 ? kMaxRows / G : 1;
   const dim3 grid((Tq + PB - 1) / PB, L.H_KV, B), block(256);
   if (L.D == 64)
-    hipLaunchKernelGGL((attn_any_kernel<64, true>), grid, block, 0, stream, L, (const uint8_t*)q, q_stride_b,
+    hipLaunchKernelGGL((attn_any_kernel<64, true, kMaxRows>), grid, block, 0, stream, L, (const uint8_t*)q, q_stride_b,
                        q_stride_h, q_stride_t, (const uint8_t*)k_new, (const uint8_t*)v_new, new_stride_b,
                        new_stride_h, new_stride_t, H_Q, Tq, scaling, nullptr, nullptr, 1, (__half*)out);
   else
-    hipLaunchKernelGGL((attn_any_kernel<256, true>), grid, block, 0, stream, L, (const uint8_t*)q, q_stride_b,
+    hipLaunchKernelGGL((attn_any_kernel<256, true, kMaxRows>), grid, block, 0, stream, L, (const uint8_t*)q, q_stride_b,
                        q_stride_h, q_stride_t, (const uint8_t*)k_new, (const uint8_t*)v_new, new_stride_b,
                        new_stride_h, new_stride_t, H_Q, Tq, scaling, nullptr, nullptr, 1, (__half*)out);
 }
