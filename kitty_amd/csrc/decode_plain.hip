@@ -26,6 +26,8 @@ __device__ inline float dequant_ref(uint32_t code, __half scale, __half zero) {
   return (float)r;
 }
 
+// ROWS: 4, 8 or 16 query heads per kv head at most (a group of 4 does not pay for 16).
+template <int ROWS>
 __global__ __launch_bounds__(256) void decode_plain_kernel(kitty_kv_layer L, const __half* __restrict__ q, int H_Q,
                                                            float scaling, float* __restrict__ ws_ml,
                                                            float* __restrict__ ws_acc, int num_splits) {
@@ -38,19 +40,19 @@ __global__ __launch_bounds__(256) void decode_plain_kernel(kitty_kv_layer L, con
   const int tile_begin = split * per, tile_end = min(c.ntiles, tile_begin + per);
   int bad_page = 0;
 
-  __shared__ float s_q[kMaxGroup][kD];
+  __shared__ __attribute__((aligned(16))) float s_q[kD][ROWS];      // [channel][head]: a thread reads the heads of a channel at once
   __shared__ __attribute__((aligned(16))) uint8_t s_codes[kMaxHeadBytes];
   __shared__ __half2 s_meta[kD];
-  __shared__ float s_p[kMaxGroup][kPage];
-  __shared__ float s_part[2][kMaxGroup][kPage];
-  __shared__ float s_m[kMaxGroup], s_l[kMaxGroup], s_alpha[kMaxGroup];
+  __shared__ __attribute__((aligned(16))) float s_p[kPage][ROWS];   // [token][head]
+  __shared__ float s_part[2][ROWS][kPage];
+  __shared__ float s_m[ROWS], s_l[ROWS], s_alpha[ROWS];
 
   for (int i = tid; i < G * kD; i += 256)
-    s_q[i / kD][i % kD] = __half2float(q[((int64_t)b * H_Q + (int64_t)h * G) * kD + i]);
-  if (tid < kMaxGroup) { s_m[tid] = -INFINITY; s_l[tid] = 0.f; }
-  float acc_o[kMaxGroup];
+    s_q[i % kD][i / kD] = __half2float(q[((int64_t)b * H_Q + (int64_t)h * G) * kD + i]);
+  if (tid < ROWS) { s_m[tid] = -INFINITY; s_l[tid] = 0.f; }
+  float acc_o[ROWS];
 #pragma unroll
-  for (int g = 0; g < kMaxGroup; ++g) acc_o[g] = 0.f;
+  for (int g = 0; g < ROWS; ++g) acc_o[g] = 0.f;
   __syncthreads();
 
   const int t = tid & 127, half = tid >> 7;
@@ -64,9 +66,9 @@ __global__ __launch_bounds__(256) void decode_plain_kernel(kitty_kv_layer L, con
     const bool v_packed = tile > 0 && body < c.pv;
 
     // ---- logits -----------------------------------------------------------------------------
-    float acc[kMaxGroup];
+    float acc[ROWS];
 #pragma unroll
-    for (int g = 0; g < kMaxGroup; ++g) acc[g] = 0.f;
+    for (int g = 0; g < ROWS; ++g) acc[g] = 0.f;
     if (k_packed) {
       const int64_t pg = checked_page(page_id(L.page_table_k, (int64_t)b * L.page_table_k_stride_b + body), L.cache_pages_k, bad_page);
       const uint8_t* src = L.key_cache + pg * L.key_cache_stride_page + (int64_t)h * k_head_bytes(DB);
@@ -84,8 +86,8 @@ __global__ __launch_bounds__(256) void decode_plain_kernel(kitty_kv_layer L, con
         const __half2 m = s_meta[d];
         const float x = dequant_ref(code, __low2half(m), __high2half(m));
 #pragma unroll
-        for (int g = 0; g < kMaxGroup; ++g)
-          if (g < G) acc[g] += s_q[g][d] * x;
+        for (int g = 0; g < ROWS; ++g)
+          if (g < G) acc[g] += s_q[d][g] * x;
       }
     } else if (t < ntok) {
       const __half* row = tile == 0 ? (const __half*)((const uint8_t*)L.sink_k + sink_base) + (int64_t)t * kD
@@ -93,12 +95,12 @@ __global__ __launch_bounds__(256) void decode_plain_kernel(kitty_kv_layer L, con
       for (int d = half * 64; d < half * 64 + 64; ++d) {
         const float x = __half2float(row[d]);
 #pragma unroll
-        for (int g = 0; g < kMaxGroup; ++g)
-          if (g < G) acc[g] += s_q[g][d] * x;
+        for (int g = 0; g < ROWS; ++g)
+          if (g < G) acc[g] += s_q[d][g] * x;
       }
     }
 #pragma unroll
-    for (int g = 0; g < kMaxGroup; ++g)
+    for (int g = 0; g < ROWS; ++g)
       if (g < G) s_part[half][g][t] = acc[g];
     __syncthreads();
 
@@ -118,8 +120,8 @@ __global__ __launch_bounds__(256) void decode_plain_kernel(kitty_kv_layer L, con
 #pragma unroll
       for (int o = 32; o > 0; o >>= 1) sum += __shfl_xor(sum, o);
       const float alpha = (m_old == -INFINITY) ? 0.f : __expf(m_old - m_new);
-      s_p[g][lane] = p0;
-      s_p[g][lane + 64] = p1;
+      s_p[lane][g] = p0;
+      s_p[lane + 64][g] = p1;
       if (lane == 0) { s_m[g] = m_new; s_l[g] = s_l[g] * alpha + sum; s_alpha[g] = alpha; }
     }
     // ---- stage V ---------------------------------------------------------------------------
@@ -137,7 +139,7 @@ __global__ __launch_bounds__(256) void decode_plain_kernel(kitty_kv_layer L, con
     {
       const int d = t;
 #pragma unroll
-      for (int g = 0; g < kMaxGroup; ++g)
+      for (int g = 0; g < ROWS; ++g)
         if (g < G) acc_o[g] *= s_alpha[g];
       const int t0 = half * 64, t1 = min(ntok, half * 64 + 64);
       for (int tt = t0; tt < t1; ++tt) {
@@ -152,8 +154,8 @@ __global__ __launch_bounds__(256) void decode_plain_kernel(kitty_kv_layer L, con
           x = __half2float(v_tail_row(L, c, b, h, (body - c.pv) * kPage + tt)[d]);
         }
 #pragma unroll
-        for (int g = 0; g < kMaxGroup; ++g)
-          if (g < G) acc_o[g] += s_p[g][tt] * x;
+        for (int g = 0; g < ROWS; ++g)
+          if (g < G) acc_o[g] += s_p[tt][g] * x;
       }
     }
     __syncthreads();
@@ -162,7 +164,7 @@ __global__ __launch_bounds__(256) void decode_plain_kernel(kitty_kv_layer L, con
   if (tid == 0) report_bad_page(L, b, bad_page);
   // ---- write this split's partial --------------------------------------------------------------
 #pragma unroll
-  for (int g = 0; g < kMaxGroup; ++g)
+  for (int g = 0; g < ROWS; ++g)
     if (g < G) s_part[half][g][t] = acc_o[g];
   __syncthreads();
   for (int i = tid; i < G * kD; i += 256) {
@@ -239,8 +241,14 @@ __global__ __launch_bounds__(GROUPS * kMergeChannels) void decode_merge_kernel(
 
 void launch_decode_plain(const kitty_kv_layer& L, const void* q, int B, int H_Q, float scaling, float* ws_ml,
                          float* ws_acc, int num_splits, hipStream_t stream) {
-  hipLaunchKernelGGL(decode_plain_kernel, dim3(num_splits, L.H_KV, B), dim3(256), 0, stream, L, (const __half*)q,
-                     H_Q, scaling, ws_ml, ws_acc, num_splits);
+  const int G = H_Q / L.H_KV;
+  const dim3 grid(num_splits, L.H_KV, B), block(256);
+  if (G <= 4)
+    hipLaunchKernelGGL(decode_plain_kernel<4>, grid, block, 0, stream, L, (const __half*)q, H_Q, scaling, ws_ml, ws_acc, num_splits);
+  else if (G <= 8)
+    hipLaunchKernelGGL(decode_plain_kernel<8>, grid, block, 0, stream, L, (const __half*)q, H_Q, scaling, ws_ml, ws_acc, num_splits);
+  else
+    hipLaunchKernelGGL(decode_plain_kernel<16>, grid, block, 0, stream, L, (const __half*)q, H_Q, scaling, ws_ml, ws_acc, num_splits);
 }
 
 namespace {
