@@ -9,6 +9,7 @@
 // 106-112, 201-204, 227-230): min/max, range, scale = range / qmax (IEEE fp32 divide, floored at
 // 1e-6), (x - min) / scale in fp32, floor(. + 0.5), clamp to [0, qmax]; the stored scale is the
 // fp32 scale rounded to fp16, the stored zero point is the minimum itself.
+#include "half_ops.h"
 #include "quant_arith.h"
 
 namespace kitty {
@@ -36,42 +37,8 @@ __device__ __forceinline__ uint4 nt_load16(const uint8_t* p) {
   return uint4{v.x, v.y, v.z, v.w};
 }
 
-typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
-// Half `hi` (0 / 1) of a word of two fp16 numbers, as the compiler's half type: widened where it is used,
-// it enters a mixed-precision FMA as it is (exactly, subnormals included) and costs no conversion.
-__device__ __forceinline__ _Float16 half_of(uint32_t w, int hi) {
-  const half2_t p = __builtin_bit_cast(half2_t, w);
-  return hi ? p.y : p.x;
-}
-// Packed fp16 minimum / maximum of two words.  Written out because the compiler first re-quiets every
-// operand it has not produced itself (one more instruction per loaded word); fp16 numbers order as
-// their fp32 values do, and a quiet NaN loses against a number as in fminf / fmaxf.
-__device__ __forceinline__ uint32_t pk_min_f16(uint32_t a, uint32_t b) {
-  uint32_t d;
-  asm("v_pk_min_f16 %0, %1, %2" : "=v"(d) : "v"(a), "v"(b));
-  return d;
-}
-__device__ __forceinline__ uint32_t pk_max_f16(uint32_t a, uint32_t b) {
-  uint32_t d;
-  asm("v_pk_max_f16 %0, %1, %2" : "=v"(d) : "v"(a), "v"(b));
-  return d;
-}
-
-// |a| + |b| in fp32 and a widened to fp32, for half `hi` of the words a and b: one mixed-precision FMA
-// each, which widens its fp16 operands exactly (subnormals included) on the way in.  (x + -0 = x for
-// every x, -0 included.)
-__device__ __forceinline__ float abs_sum_f16(uint32_t a, uint32_t b, int hi) {
-  float d;
-  if (hi) asm("v_fma_mix_f32 %0, |%1|, 1.0, |%2| op_sel:[1,0,1] op_sel_hi:[1,0,1]" : "=v"(d) : "v"(a), "v"(b));
-  else asm("v_fma_mix_f32 %0, |%1|, 1.0, |%2| op_sel:[0,0,0] op_sel_hi:[1,0,1]" : "=v"(d) : "v"(a), "v"(b));
-  return d;
-}
-__device__ __forceinline__ float widen_f16(uint32_t a, int hi) {
-  float d;
-  const float neg_zero = -0.0f;
-  if (hi) asm("v_fma_mix_f32 %0, %1, 1.0, %2 op_sel:[1,0,0] op_sel_hi:[1,0,0]" : "=v"(d) : "v"(a), "s"(neg_zero));
-  else asm("v_fma_mix_f32 %0, %1, 1.0, %2 op_sel:[0,0,0] op_sel_hi:[1,0,0]" : "=v"(d) : "v"(a), "s"(neg_zero));
-  return d;
+__device__ __forceinline__ void nt_store16(uint8_t* p, const uint4& v) {
+  __builtin_nontemporal_store(u32x4{v.x, v.y, v.z, v.w}, (u32x4*)p);
 }
 
 // The codes of the 8 values of one group (half `hi` of the words w[0..7]) as bytes of two words,
@@ -362,8 +329,9 @@ __device__ __forceinline__ void quant_k_page(const ROWS row_of, int d_boost,
   // everything leaves in contiguous pieces: the low plane by all threads (16 bytes each), the high plane by the
   // first lanes (16 bytes each), the slot map by the second wave and the (scale, zero) pairs by the last two
   // (4 bytes each: the metadata's alignment is only that)
-  ((uint4*)dst)[tid] = *(const uint4*)(s_lo + ((tid * 16) ^ (((tid >> 4) & 15) << 4)));   // piece tid of the plane: row tid / 2, c8 = row / 8
-  if (tid < 2 * d_boost && (MODE != 0 || s_slot_used[tid >> 1])) ((uint4*)(dst + kLoBytes))[tid] = ((const uint4*)s_hi)[tid];
+  // the planes are written once and read much later: non-temporal stores
+  nt_store16(dst + tid * 16, *(const uint4*)(s_lo + ((tid * 16) ^ (((tid >> 4) & 15) << 4))));   // piece tid of the plane: row tid / 2, c8 = row / 8
+  if (tid < 2 * d_boost && (MODE != 0 || s_slot_used[tid >> 1])) nt_store16(dst + kLoBytes + tid * 16, ((const uint4*)s_hi)[tid]);
   const int t1 = tid - 64, t2 = tid - 128;
   if (t1 >= 0 && t1 < kD / 4) ((uint32_t*)(dst + kRowBytes * (kD + d_boost)))[t1] = ((const uint32_t*)s_idx)[t1];
   if (t2 >= 0) ((uint32_t*)meta_dst)[t2] = s_meta[t2];
