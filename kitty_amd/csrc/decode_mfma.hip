@@ -38,6 +38,7 @@
 //   C[u][j] of lane (kg, n) = token 32kg + 8j + u, column n.
 //   V plane rows are tokens: lane group kg owns rows 32kg .. 32kg+31 (its own tokens), k-chunk j
 //   = rows 32kg + 8j .. +7, d-tile u = channels {8n + u}; O^T[u][j] = channel 32kg + 8j + u.
+#include <algorithm>
 #include <type_traits>
 
 #include <hip/hip_ext.h>
@@ -951,13 +952,15 @@ __device__ __forceinline__ void settle_prologue_loads() {
 struct WorkItem {
   int b, h, split;
   bool crowded, valid;
+  int t0, t1;    // flat shares (below): the body tiles of this item
+  int n_used;    // flat shares, the tail's item: partials of the sequence that some workgroup writes
 };
 __device__ __forceinline__ WorkItem work_item_of_block(int h_kv, const uint32_t* plan) {
-  if (!plan) return WorkItem{(int)blockIdx.z, (int)blockIdx.y, (int)blockIdx.x, false, true};
+  if (!plan) return WorkItem{(int)blockIdx.z, (int)blockIdx.y, (int)blockIdx.x, false, true, 0, 0, 0};
   const uint32_t j = blockIdx.x / (uint32_t)h_kv;
-  if (j >= plan[0]) return WorkItem{0, 0, 0, true, false};
+  if (j >= plan[0]) return WorkItem{0, 0, 0, true, false, 0, 0, 0};
   const uint32_t item = plan[kPlanHeader + j];
-  return WorkItem{(int)(item >> 16), (int)(blockIdx.x % (uint32_t)h_kv), (int)(item & 0xFFFFu), true, true};
+  return WorkItem{(int)(item >> 16), (int)(blockIdx.x % (uint32_t)h_kv), (int)(item & 0xFFFFu), true, true, 0, 0, 0};
 }
 constexpr int kCrowdedMinTiles = 16;   // body tiles per split a crowded launch aims for
 constexpr int kCrowdedTailCost = 12;   // what the tail's split takes, in body tiles (for the order)
@@ -1033,6 +1036,131 @@ __device__ __forceinline__ int tail_splits(const SeqCounts& c, int num_splits, b
   return num_splits >= 4 && npp < 12 * (num_splits - 3) ? 3 : (num_splits >= 2 ? 1 : 0);
 }
 
+// Flat shares: a crowded launch over at most kFlatMaxB sequences needs no list.  The body tiles of
+// all sequences (of one kv head: the heads of a sequence are alike) form one row, sequence after
+// sequence, which is cut into `chunks` pieces; workgroup (chunk c, head h) walks the sequences its
+// piece touches and leaves one partial per sequence, in the slot after the slots of the pieces that
+// cut the same sequence before it (slot 0 is the tail's).  The launch is one round of two
+// workgroups per SIMD, in which every workgroup has the same amount of work, whatever the lengths of
+// the sequences are.  Every workgroup works the cuts out for itself from the sequences' counters:
+// one round trip more at its start instead of a kernel ahead of the launch.
+// The tails: with at most `chunks` sequences, tail j is the LAST thing the workgroup of chunk
+// floor-inverse(j * chunks / B) does (the tails lie evenly over the chunks, at most one each), and that
+// chunk's piece is shorter by what a tail costs, in tiles (tc).  With more sequences than chunks the
+// tails have workgroups of their own behind the others.
+// No sequence may be cut into more pieces than it has slots: if the pieces are too small for the
+// longest sequence (num_splits - 2 whole pieces and two part ones at most), first the tails' cost
+// is left out of the account, then the pieces take the fixed size that fits the longest sequence
+// and the last chunks stay empty.
+constexpr int kFlatMaxB = 256;
+// A tail's cost in body tiles.  By its bytes (96 KB of fp16 rows at most) it is 9; under the load of
+// the streaming workgroups its scattered rows take longer (ragged batch of 64: 83.5 us with 9, 78.3
+// with 12, 78.6 with 15, 80.3 with 18).
+constexpr int kFlatTailCost = 12;
+struct FlatPlan {
+  int total;         // body tiles of all sequences
+  int chunks, B;
+  int fixed;         // 0: piece c starts at bound(c) below; else at c * fixed
+  int tc;            // what a tail takes off its chunk's piece
+  uint64_t step_w;   // (total + tc * B) / chunks, in units of 2^-20
+  uint32_t step_b;   // B / chunks in units of 2^-20; 0: the tails have workgroups of their own
+};
+// tails [tails_before(c), tails_before(c + 1)) belong to chunk c
+__device__ __forceinline__ int flat_tails_before(const FlatPlan& p, int c) {
+  return c >= p.chunks ? p.B : (int)(((uint64_t)(uint32_t)c * p.step_b) >> 20);
+}
+__device__ __forceinline__ int flat_bound(const FlatPlan& p, int c) {
+  if (p.fixed) return min(p.total, c * p.fixed);
+  if (c >= p.chunks) return p.total;
+  return (int)(((uint64_t)(uint32_t)c * p.step_w) >> 20) - p.tc * flat_tails_before(p, c);
+}
+// the piece that holds tile `pos` of the row: the last one that starts at or before it
+__device__ __forceinline__ int flat_chunk_of(const FlatPlan& p, int pos) {
+  if (p.fixed) return pos / p.fixed;
+  int lo = 0, hi = p.chunks;   // bound(lo) <= pos < bound(hi)
+  while (hi - lo > 1) {
+    const int mid = (lo + hi) >> 1;
+    if (flat_bound(p, mid) <= pos) lo = mid; else hi = mid;
+  }
+  return lo;
+}
+// The cuts, from the row's length and the longest sequence (wave-uniform arithmetic).  Without the
+// fixed size a piece has at least floor(row / chunks) - tc >= 1 tiles: the bounds rise strictly.
+__device__ __forceinline__ FlatPlan flat_decide(int total, int longest, int B, int chunks, int num_splits,
+                                                bool tails_apart) {
+  FlatPlan p;
+  p.total = total;
+  p.chunks = chunks;
+  p.B = B;
+  p.step_b = tails_apart ? 0u : (uint32_t)(((uint64_t)(uint32_t)B << 20) / (uint32_t)chunks);
+  p.tc = tails_apart ? 0 : kFlatTailCost;
+  // A sequence cut into m pieces holds m - 2 whole ones: if any num_splits - 2 pieces in a row add
+  // up to the longest sequence or more, no sequence has more than num_splits - 1 pieces.  They add up
+  // to at least their number times the whole part of the quotient, less the tails among them.
+  const int k = num_splits - 2;
+  const int tails_in_k = (int)(((uint64_t)(uint32_t)k * p.step_b) >> 20) + 1;
+  uint32_t row = (uint32_t)total + (uint32_t)(p.tc * B);
+  uint32_t whole = row / (uint32_t)chunks;
+  if (p.tc && !((int)whole - p.tc >= 1 && k * (int)whole - p.tc * tails_in_k >= longest)) {
+    p.tc = 0;
+    row = (uint32_t)total;
+    whole = row / (uint32_t)chunks;
+  }
+  const bool fits = (int)whole - p.tc >= 1 && k * (int)whole - p.tc * tails_in_k >= longest;
+  p.fixed = fits ? 0 : max(1, c_div_up(longest, k));
+  const uint32_t rest = row - whole * (uint32_t)chunks;   // rest < chunks <= 2^11
+  p.step_w = ((uint64_t)whole << 20) + ((rest << 20) / (uint32_t)chunks);
+  return p;
+}
+// The chunk and the kv head of a workgroup that streams body tiles.  (The tails then lie on every
+// n-th chunk, i.e. evenly over the XCDs and, as workgroups i and i + half of the launch share a SIMD,
+// two to a SIMD.  Measured and dropped, ragged batch of 64: tails paired with streaming workgroups
+// on a SIMD +3 %, tails in blocks of 4 / 8 / 32 consecutive chunks +1 %, all tails on two XCDs +9 %.)
+__device__ __forceinline__ int flat_chunk_of_block(int H) { return blockIdx.x / H; }
+__device__ __forceinline__ int flat_head_of_block(int H) { return blockIdx.x % H; }
+// What a workgroup keeps in LDS of the plan: where sequence b begins in the row (b = 0 .. B), the
+// row's length and the longest sequence.  It lies in the part of the second K buffer that the tail's
+// staging of fp16 rows does not reach.
+struct FlatTable {
+  uint32_t starts[kFlatMaxB + 1];
+  int total, longest;
+};
+constexpr int kFlatTableOff = kKTile + (10240 - kKTile);   // from the first K buffer: behind the 10240 bytes of staging
+static_assert(kFlatTableOff + sizeof(FlatTable) <= 2 * kKTile, "the table fits behind the staging area");
+// ends[k]: where this lane's sequence 4 * lane + k ends in the row
+__device__ __forceinline__ void flat_scan(const kitty_kv_layer& L, int B, FlatTable& T, int (&ends)[4]) {
+  const int lane = threadIdx.x;
+  int nb[4], sum = 0, longest = 0;
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    const int b = 4 * lane + k;
+    nb[k] = b < B ? body_tiles_of(load_counts(L, min(b, B - 1))) : 0;
+    sum += nb[k];
+    longest = max(longest, nb[k]);
+  }
+  int upto = sum;
+#pragma unroll
+  for (int o = 1; o < 64; o <<= 1) {
+    const int v = __shfl_up(upto, o);
+    if (lane >= o) upto += v;
+  }
+#pragma unroll
+  for (int o = 32; o; o >>= 1) longest = max(longest, __shfl_xor(longest, o));
+  int at = upto - sum;
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    T.starts[4 * lane + k] = (uint32_t)at;
+    at += nb[k];
+    ends[k] = at;
+  }
+  if (lane == 63) {
+    T.starts[256] = (uint32_t)at;
+    T.total = at;
+    T.longest = longest;
+  }
+  wave_lds_fence();
+}
+
 // What one wave does.  DMA: packed tiles are streamed global -> LDS (G <= 8); otherwise they are
 // loaded into registers.  QUARTER (needs DMA; at most 4 query heads per kv head): body pages go
 // through combine_quarter / softmax_quarter / pv_quarter.
@@ -1045,7 +1173,7 @@ __device__ __forceinline__ int tail_splits(const SeqCounts& c, int num_splits, b
 // when the pressure is on the wrong side of the edge, with spills of its own (a reload inside the
 // loop is a vector load that the hand-counted waits do not know of).
 enum WaveMode { kWaveSolo, kWaveBody, kWaveTail };
-template <bool BOOST, bool DMA, bool QUARTER, WaveMode MODE, class LDS>
+template <bool BOOST, bool DMA, bool QUARTER, WaveMode MODE, bool FLAT = false, class LDS>
 __device__ __forceinline__ void wave_work(const kitty_kv_layer& L, const __half* __restrict__ q, int H_Q, float scaling,
                                           float* __restrict__ ws_ml, float* __restrict__ ws_acc, int num_splits,
                                           int n_simds, const WorkItem& w, LDS& S) {
@@ -1160,7 +1288,10 @@ __device__ __forceinline__ void wave_work(const kitty_kv_layer& L, const __half*
   int t0 = 0, t1 = 0;          // body tiles of this split
   int u0 = nbt, u1 = nbt;      // tail tiles of this split
   bool do_sink = false;
-  if (num_splits == 1) {
+  if constexpr (FLAT) {
+    if constexpr (MODE == kWaveTail) { u0 = npp; do_sink = true; }
+    else { t0 = w.t0; t1 = w.t1; }
+  } else if (num_splits == 1) {
     t1 = npp; u0 = npp; do_sink = true;
   } else if (split < n_tail) {
     if (n_tail == 1) { u0 = npp; do_sink = true; }
@@ -1359,7 +1490,7 @@ __device__ __forceinline__ void wave_work(const kitty_kv_layer& L, const __half*
     // a crowded launch has no workgroups for the splits without work: the tail's split marks their
     // partials as empty (the merge pass then does not read their accumulator rows)
     if (w.crowded) {
-      const int s0 = 1 + crowded_body_splits(npp, num_splits);
+      const int s0 = FLAT ? w.n_used : 1 + crowded_body_splits(npp, num_splits);
       const int n_empty = num_splits - s0;
       for (int i = x.lane; i < G * n_empty; i += 64) {
         const int g = i / n_empty, s = s0 + i - g * n_empty;
@@ -1381,6 +1512,8 @@ struct KernArgs {
   float* ws_acc;
   int num_splits, n_simds;
   const uint32_t* plan;   // the work list of a crowded launch (see WorkItem), else NULL
+  int B, flat_chunks;     // flat shares (see FlatPlan): sequences, chunks (workgroups per kv head that stream body tiles)
+  bool flat_tails_apart;  // flat shares: the tails have workgroups of their own
 };
 
 __device__ __forceinline__ const KernArgs& kernel_args_of(const KernArgs* p) {   // the address as a scalar again
@@ -1405,6 +1538,65 @@ __device__ __attribute__((noinline, noreturn)) void tail_wave(const KernArgs* ke
                                              *(WaveLds<DMA, QUARTER>*)lds);
   __builtin_amdgcn_endpgm();
 }
+// A crowded launch with flat shares (see FlatPlan): workgroups [0, flat_chunks * H_KV) stream body
+// tiles - chunk = id / H_KV of head id % H_KV - and then take the chunk's tail, if it has one; the
+// workgroups behind them (flat_tails_apart) take the tail of one (sequence, head) each.  The tail's
+// function marks the sequence's unused partials as empty and ends the wave.
+template <bool BOOST, bool QUARTER>
+__device__ __attribute__((noinline, noreturn)) void flat_tail_wave(const KernArgs* kernel_args,
+                                                                    __attribute__((address_space(3))) WaveLds<true, QUARTER>* lds) {
+  const KernArgs& a = kernel_args_of(kernel_args);
+  WaveLds<true, QUARTER>& S = *(WaveLds<true, QUARTER>*)lds;
+  const FlatTable& T = *(const FlatTable*)(&S.kbuf[0][0] + kFlatTableOff);
+  const int H = a.L.H_KV, id = blockIdx.x, n_body = a.flat_chunks * H;
+  const FlatPlan P = flat_decide(__builtin_amdgcn_readfirstlane(T.total), __builtin_amdgcn_readfirstlane(T.longest), a.B,
+                                 a.flat_chunks, a.num_splits, a.flat_tails_apart);
+  const int b = id >= n_body ? (id - n_body) / H : flat_tails_before(P, flat_chunk_of_block(H));
+  const int s = __builtin_amdgcn_readfirstlane((int)T.starts[b]), e = __builtin_amdgcn_readfirstlane((int)T.starts[b + 1]);
+  const int pieces = e > s ? flat_chunk_of(P, e - 1) - flat_chunk_of(P, s) + 1 : 0;
+  const WorkItem w{b, id >= n_body ? id % H : flat_head_of_block(H), 0, true, true, 0, 0, 1 + pieces};
+  wave_work<BOOST, true, QUARTER, kWaveTail, true>(a.L, a.q, a.H_Q, a.scaling, a.ws_ml, a.ws_acc, a.num_splits, 0, w, S);
+  __builtin_amdgcn_endpgm();
+}
+template <bool BOOST, bool QUARTER>
+__global__ __launch_bounds__(64, 2) void decode_mfma_flat_kernel(KernArgs a) {
+  __shared__ WaveLds<true, QUARTER> S;
+  static_assert(sizeof(S.kbuf) == 2 * kKTile, "the plan's table lies in the second K buffer");
+  FlatTable& T = *(FlatTable*)(&S.kbuf[0][0] + kFlatTableOff);
+  const int H = a.L.H_KV;
+  int ends[4];
+  flat_scan(a.L, a.B, T, ends);
+  auto tail = [&]() {
+    flat_tail_wave<BOOST, QUARTER>(
+        (const KernArgs*)(const __attribute__((address_space(4))) KernArgs*)__builtin_amdgcn_kernarg_segment_ptr(),
+        (__attribute__((address_space(3))) WaveLds<true, QUARTER>*)&S);
+  };
+  if ((int)blockIdx.x >= a.flat_chunks * H) tail();
+  const FlatPlan P = flat_decide(__builtin_amdgcn_readfirstlane(T.total), __builtin_amdgcn_readfirstlane(T.longest), a.B,
+                                 a.flat_chunks, a.num_splits, a.flat_tails_apart);
+  const int c = flat_chunk_of_block(H), h = flat_head_of_block(H);
+  const int lo = flat_bound(P, c), hi = flat_bound(P, c + 1);
+  const bool has_tail = !a.flat_tails_apart && flat_tails_before(P, c + 1) > flat_tails_before(P, c);
+  if (lo < hi) {
+    // the first sequence of the piece: as many sequences end at or before its first tile
+    int b = 0;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) b += __popcll(__ballot(4 * (int)threadIdx.x + k < a.B && ends[k] <= lo));
+    int slot = -1;   // of the first sequence: found by search; the others begin inside the piece
+#pragma unroll 1
+    for (; b < a.B; ++b) {
+      const int s = __builtin_amdgcn_readfirstlane((int)T.starts[b]), e = __builtin_amdgcn_readfirstlane((int)T.starts[b + 1]);
+      if (s >= hi) break;
+      if (e <= s) continue;
+      if (slot < 0) slot = min(1 + c - flat_chunk_of(P, s), a.num_splits - 1); else slot = 1;   // (the plan keeps it below num_splits; the workspace ends there)
+      const WorkItem w{b, h, slot, true, true, max(lo, s) - s, min(hi, e) - s, 0};
+      wave_work<BOOST, true, QUARTER, kWaveBody, true>(a.L, a.q, a.H_Q, a.scaling, a.ws_ml, a.ws_acc, a.num_splits,
+                                                       a.n_simds, w, S);
+    }
+  }
+  if (has_tail) tail();
+}
+
 // SOLO: the launch has one split.  Otherwise the first tail_splits() splits of a (batch row, kv head)
 // go through tail_wave and the others stream the body.
 template <bool BOOST, bool DMA, bool QUARTER, bool SOLO>
@@ -1440,8 +1632,19 @@ struct LaunchArgs {
   hipStream_t stream;
   hipEvent_t ev_start, ev_stop;
 };
+template <bool BOOST, bool QUARTER>
+void launch_flat(const LaunchArgs& a) {
+  const dim3 grid((uint32_t)((a.k.flat_chunks + (a.k.flat_tails_apart ? a.B : 0)) * a.k.L.H_KV)), block(64);
+  if (a.ev_start)
+    hipExtLaunchKernelGGL((decode_mfma_flat_kernel<BOOST, QUARTER>), grid, block, 0, a.stream, a.ev_start, a.ev_stop, 0, a.k);
+  else
+    hipLaunchKernelGGL((decode_mfma_flat_kernel<BOOST, QUARTER>), grid, block, 0, a.stream, a.k);
+}
 template <bool BOOST, bool DMA, bool QUARTER, bool SOLO>
 void launch_one(const LaunchArgs& a) {
+  if constexpr (DMA && !SOLO) {
+    if (a.k.flat_chunks > 0) return launch_flat<BOOST, QUARTER>(a);
+  }
   const bool crowded = a.k.plan != nullptr;
   const dim3 grid = crowded ? dim3((uint32_t)(a.B * a.k.L.H_KV * a.k.num_splits), 1, 1)
                             : dim3(a.k.num_splits, a.k.L.H_KV, a.B);
@@ -1473,11 +1676,17 @@ void launch_decode_mfma(const kitty_kv_layer& L, const void* q, int B, int H_Q, 
                         hipEvent_t ev_start, hipEvent_t ev_stop) {
   const int64_t n_wg = (int64_t)B * L.H_KV * num_splits;
   const bool crowded = num_splits > 1 && n_wg > 2 * (int64_t)n_simds && n_wg <= INT32_MAX;
-  const LaunchArgs a{KernArgs{L, (const __half*)q, H_Q, scaling, ws_ml, ws_acc, num_splits, n_simds,
-                              crowded ? ws_plan : nullptr},
-                     B, stream, ev_start, ev_stop};
   const int G = H_Q / L.H_KV;
   const bool boost = L.D_BOOSTED == 32, dma = G <= 8, quarter = G <= 4;
+  // flat shares: a launch of one round - two workgroups per SIMD, of which the tails take theirs and
+  // the body at least half
+  const bool flat = crowded && dma && B <= kFlatMaxB && num_splits >= 3;
+  const int all_slots = std::min(2048, std::max(1, 2 * n_simds / L.H_KV));
+  const bool tails_apart = B > all_slots;
+  const int flat_chunks = !flat ? 0 : !tails_apart ? all_slots : std::max(1, std::max(2 * n_simds - B * L.H_KV, n_simds) / L.H_KV);
+  const LaunchArgs a{KernArgs{L, (const __half*)q, H_Q, scaling, ws_ml, ws_acc, num_splits, n_simds,
+                              crowded && !flat ? ws_plan : nullptr, B, flat_chunks, tails_apart},
+                     B, stream, ev_start, ev_stop};
   if (boost && quarter) launch_variant<true, true, true>(a);
   else if (boost && dma) launch_variant<true, true, false>(a);
   else if (boost) launch_variant<true, false, false>(a);
