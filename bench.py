@@ -740,7 +740,7 @@ class DecodeBench:
         gbps = self.total_bytes / (avg * 1e-6) / 1e9
         return {"workload": self.desc, "variant": self.variant if variant is None else variant,
                 "num_splits": self.splits, "value": us_per_step, "unit": "us/step", "steps": steps,
-                "kernel": "decode split pass" + (" (work-list kernel + split kernel)" if self.workload == "c2" else ""),
+                "kernel": "decode split pass" + (" (one round of flat shares)" if self.workload == "c2" else ""),
                 "kernel_avg_us": avg, "kernel_median_us": kern_us[len(kern_us) // 2],
                 "algorithmic_bytes_per_launch": self.total_bytes, "packed_bytes_per_launch": self.packed_bytes,
                 "achieved_gbps": gbps, "frac": gbps / HBM_PEAK_GBPS,

@@ -944,7 +944,8 @@ __device__ __forceinline__ void settle_prologue_loads() {
 // the workgroups matters: the dispatcher hands them out by linear id as slots free up.  With the
 // grid laid out (splits, heads, rows) the splits without work come in bursts between the busy ones,
 // the slots they free are refilled late (ragged batch of 64: 1,500 of 2,048 resident on average)
-// and the launch ends with whatever sequence came last.  So a crowded launch runs from a work
+// and the launch ends with whatever sequence came last.  So a crowded launch either becomes one
+// round of equal shares (at most kFlatMaxB sequences, see FlatPlan below) or runs from a work
 // list: decode_plan_kernel, one small workgroup ahead of the split pass, reads the sequences'
 // counters and writes the items that have work, the longest first; workgroup j of the split pass
 // takes item j / H_KV for kv head j % H_KV, and the workgroups past the end of the list - all at
