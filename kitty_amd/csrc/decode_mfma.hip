@@ -1102,13 +1102,15 @@ __device__ __forceinline__ FlatPlan flat_decide(int total, int longest, int B, i
   const int tails_in_k = (int)(((uint64_t)(uint32_t)k * p.step_b) >> 20) + 1;
   uint32_t row = (uint32_t)total + (uint32_t)(p.tc * B);
   uint32_t whole = row / (uint32_t)chunks;
-  if (p.tc && !((int)whole - p.tc >= 1 && k * (int)whole - p.tc * tails_in_k >= longest)) {
+  auto fits_with = [&](uint32_t whole_part, int tc) {
+    return (int)whole_part - tc >= 1 && (int64_t)k * whole_part - (int64_t)tc * tails_in_k >= longest;
+  };
+  if (p.tc && !fits_with(whole, p.tc)) {
     p.tc = 0;
     row = (uint32_t)total;
     whole = row / (uint32_t)chunks;
   }
-  const bool fits = (int)whole - p.tc >= 1 && k * (int)whole - p.tc * tails_in_k >= longest;
-  p.fixed = fits ? 0 : max(1, c_div_up(longest, k));
+  p.fixed = fits_with(whole, p.tc) ? 0 : max(1, c_div_up(longest, k));
   const uint32_t rest = row - whole * (uint32_t)chunks;   // rest < chunks <= 2^11
   p.step_w = ((uint64_t)whole << 20) + ((rest << 20) / (uint32_t)chunks);
   return p;

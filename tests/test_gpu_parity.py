@@ -407,8 +407,10 @@ def test_config0_roundtrip_and_decode(K, variant):
 
 
 @pytest.mark.parametrize("variant", [0, 1])
-@pytest.mark.parametrize("splits", [1, 3, 7, 64])
+@pytest.mark.parametrize("splits", [1, 3, 7, 64, 600])
 def test_split_counts_agree(K, variant, splits):
+    """600 splits: more workgroups than the device holds at once, with one set of counters for the whole
+    batch (the launch then runs as one round of equal shares, like a ragged one)."""
     B, H_KV, H_Q, T = 2, 2, 8, 32 + 128 * 9 + 50
     cache, ol = _build(K, B, H_KV, H_Q, T, 2048, seed=5)
     q = make_q(B, H_Q, seed=5)
