@@ -1056,7 +1056,8 @@ __device__ __forceinline__ int tail_splits(const SeqCounts& c, int num_splits, b
 constexpr int kFlatMaxB = 256;
 // A tail's cost in body tiles.  By its bytes (96 KB of fp16 rows at most) it is 9; under the load of
 // the streaming workgroups its scattered rows take longer (ragged batch of 64: 83.5 us with 9, 78.3
-// with 12, 78.6 with 15, 80.3 with 18).
+// with 12, 78.6 with 15, 80.3 with 18).  A cost per sequence, a base plus the tail's tokens over a
+// divisor, did no better than one number for all (four pairs tried: +0 to +5 us).
 constexpr int kFlatTailCost = 12;
 struct FlatPlan {
   int total;         // body tiles of all sequences
@@ -1349,14 +1350,15 @@ __device__ __forceinline__ void wave_work(const kitty_kv_layer& L, const __half*
         wave_lds_fence();   // (the table's first write comes after these reads: LDS executes a wave's instructions in order)
       }
       // Of the two waves that share a SIMD the older one wins arbitration, and it is 8 % faster per
-      // tile.  When the launch is a single round (at most two workgroups per SIMD of the device),
+      // tile.  When the launch is a single round (at most two workgroups per SIMD of the device; a
+      // launch of flat shares is one: 2 % on the ragged batch of 64),
       // the workgroups dispatched after every SIMD has one are the younger ones: they raise their
       // priority by one level after the first quarter of their range, which evens out the finishes.
       // (Two copies of the loop: the conditional priorities cost the other launches 1.5 %.)
       const uint32_t kSimds = (uint32_t)n_simds;
       const uint32_t n_wg = gridDim.x * gridDim.y * gridDim.z;
       const uint32_t lin_id = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
-      const bool young = !w.crowded && n_wg <= 2 * kSimds && lin_id >= kSimds;
+      const bool young = (FLAT || !w.crowded) && n_wg <= 2 * kSimds && lin_id >= kSimds;
       auto loop = [&](auto switch_priority) {
       constexpr bool SWITCH = decltype(switch_priority)::value;
 #pragma unroll 1
