@@ -176,8 +176,9 @@ int kitty_decode_attn(const kitty_kv_layer* layer, const void* q, int B, int H_Q
  * shards one long sequence over several devices runs the split pass on each shard, gathers the
  * partials into one workspace (splits of all shards side by side) and runs the merge pass once.
  * (The last kitty_decode_attn_workspace_bytes() - partials bytes of a workspace belong to the split
- * pass alone: when it has more workgroups than the device holds at once, a small kernel ahead of it
- * leaves the list of the splits that have work there.  The merge pass does not read them.)
+ * pass alone: when it has more workgroups than the device holds at once and the batch is larger than
+ * 256 sequences (or a kv head serves more than 8 query heads), a small kernel ahead of it leaves the
+ * list of the splits that have work there.  The merge pass does not read them.)
  * No counterpart in the reference, whose grid is (B, H_KV) with no split over the sequence
  * (kernels/kitty_attention.py:433,484).
  */
