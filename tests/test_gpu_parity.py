@@ -655,6 +655,21 @@ def test_launches_of_several_rounds_with_shares_cut_from_one_row(K, B, H_KV, H_Q
                     tol_fma=FLAT_TOL_FMA, tol_literal=FLAT_TOL_LITERAL)
 
 
+def test_as_many_sequences_as_the_shares_table_holds(K):
+    """256 sequences x 8 kv heads with three partials each: the largest batch that runs as one round of
+    shares (every share ends with a tail, the table of sequence starts is full to its last entry)."""
+    B, H_KV, H_Q = 256, 8, 8
+    shapes = [(20, 0), (100, 0), (32 + 128 + 5, 0), (32 + 128 * 2 + 77, 60), (32 + 128 * 3 + 100, 20)]
+    cache, L, ols, which = _batch_of_prototypes(K, B, H_KV, H_Q, shapes, 32 + 128 * 4, 1200)
+    q = make_q(B, H_Q, seed=12)
+    out, _ = K.attn(K.u.module(H_KV, H_Q), K.u.to_dev(q), L, 128 ** -0.5, variant=0, num_splits=3)
+    got = _np16(out).astype(np.float64)
+    assert np.isfinite(got).all()
+    for b in list(range(0, B, 5)) + [B - 1]:
+        _check_attn(got[b:b + 1], ols[which[b]], q[b:b + 1], what=f"row {b}", variant=0, tol_two=FLAT_TOL_TWO,
+                    tol_fma=FLAT_TOL_FMA, tol_literal=FLAT_TOL_LITERAL)
+
+
 def test_all_equal_keys_give_mean_of_values(K):
     """Closed form: identical keys -> uniform weights -> output = mean of the dequantized values."""
     B, H_KV, H_Q, T = 1, 1, 4, 32 + 128 * 3
