@@ -1317,8 +1317,9 @@ __device__ __forceinline__ void wave_work(const kitty_kv_layer& L, const __half*
       // neighbouring pages, page-table entries and (scale, zero) blocks at about the same time instead of
       // fifteen places 17 pages apart.  16 sequences of 32k tokens: 60.3 against 62.6 us (61.3 against
       // 63.7 on a slower box; 60.8 against 62.0 with the pages scattered over the cache at random);
-      // dealt in groups of two or four tiles: 65.5 / 68.8.  (A crowded launch's shares stay ranges.)
-      if (!w.crowded) { first_tile = i_body; tile_step = n_body; }
+      // dealt in groups of two or four tiles: 65.5 / 68.8.  Shares of a few tiles stay ranges (1 sequence
+      // of 128k tokens over 240 splits: 26.05 us in turn against 25.85), and so do a crowded launch's.
+      if (!w.crowded && base >= 8) { first_tile = i_body; tile_step = n_body; }
     }
   }
   const bool tail = MODE != kWaveBody && (do_sink || u0 < u1);
