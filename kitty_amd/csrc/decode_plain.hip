@@ -9,7 +9,6 @@ using namespace kitty;
 
 namespace kitty {
 
-constexpr int kMaxGroup = 16;                        // kitty_attention.py:418
 constexpr int kMaxHeadBytes = kRowBytes * (kD + kD) + kD;   // d_boost up to D
 
 // fp16(code) * scale + zero with BOTH operations rounded to fp16, as eager torch and the Triton

@@ -78,9 +78,6 @@ struct Stage {
 __device__ __forceinline__ int slot_of(int e) {   // element (token or channel) -> LDS slot
   return (e & ~15) | ((e & 7) << 1) | ((e >> 3) & 1);
 }
-__device__ __forceinline__ int elem_of(int s) {   // LDS slot -> element
-  return (s & ~15) | ((s & 15) >> 1) | ((s & 1) << 3);
-}
 
 __device__ __forceinline__ half4 lds_tr(const uint8_t* p) {
   short4v r = __builtin_amdgcn_ds_read_tr16_b64_v4i16((short4v __attribute__((address_space(3)))*)p);
